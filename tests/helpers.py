@@ -1,0 +1,57 @@
+"""Tiny configurations and helpers shared by the tests.
+
+The configurations differ in every size and option: layers, width, heads and
+groups, head size, feed-forward width, vocabulary, rotation base, eps, tied or
+untied head, window.  None of their sizes is a power of two where it can be
+avoided (B, C)."""
+import json
+import os
+
+import numpy as np
+
+CONFIGS = {
+    # 2 layers, width 64, 4 heads in 2 groups, head 16, tied head, theta 1e4, eps 1e-6
+    "A": dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2, hidden_size=64,
+              num_attention_heads=4, num_key_value_heads=2, head_dim=16, intermediate_size=128,
+              vocab_size=256, rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+              attention_bias=False, hidden_act="silu", max_position_embeddings=4096),
+    # 3 layers, width 96, 6 heads in 2 groups (ratio 3), head 32 (heads*head = 192 != width), untied
+    "B": dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=3, hidden_size=96,
+              num_attention_heads=6, num_key_value_heads=2, head_dim=32, intermediate_size=224,
+              vocab_size=1000, rope_theta=1000000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+              attention_bias=False, hidden_act="silu", max_position_embeddings=4096),
+    # 4 layers, width 80, 5 heads each its own group, head 48, a window of 20 on layers 2 and 3
+    "C": dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=4, hidden_size=80,
+              num_attention_heads=5, num_key_value_heads=5, head_dim=48, intermediate_size=176,
+              vocab_size=517, rope_theta=500000.0, rms_norm_eps=3e-6, tie_word_embeddings=False,
+              attention_bias=False, hidden_act="silu", max_position_embeddings=4096,
+              use_sliding_window=True, sliding_window=20, max_window_layers=2),
+}
+
+
+def read_folder(path):
+    """(config dict, {name: float64 array}) of a model folder, read with the
+    safetensors package (not with the framework's own reader)."""
+    import torch
+    from safetensors.torch import load_file
+    with open(os.path.join(path, "config.json")) as f:
+        cfg = json.load(f)
+    w = {k: v.to(torch.float64).numpy() for k, v in load_file(os.path.join(path, "model.safetensors")).items()}
+    return cfg, w
+
+
+def sharpen_folder(path, factor=4.0):
+    """Scale every q_norm weight so that attention scores spread out and single
+    keys dominate: a wrong key, mask edge or page then changes the logits visibly."""
+    import torch
+    from safetensors.torch import load_file, save_file
+    fn = os.path.join(path, "model.safetensors")
+    t = load_file(fn)
+    for k in t:
+        if k.endswith("q_norm.weight"):
+            t[k] = (t[k].to(torch.float32) * factor).to(t[k].dtype)
+    save_file(t, fn)
+
+
+def random_tokens(n, vocab, seed):
+    return [int(t) for t in np.random.default_rng(seed).integers(0, vocab, size=n)]

@@ -1,0 +1,187 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16, under
+every way of cutting the work: each request alone and whole; most of it in one
+step and the last 32 tokens one by one; in portions of changing size, down to
+two tokens; and mixed, up to four live requests, portions of some beside decoded
+tokens of others, with so few pages that they are used again."""
+import numpy as np
+import pytest
+import torch
+
+import traces
+from helpers import CONFIGS, random_tokens, read_folder
+from plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+# Largest allowed |engine - plain| over all logits.  Random-weight logits of the
+# tiny models are of order 0.1 to 1.
+#   float32: against the plain model in float64 with no rounding: 2e-5.
+#   bfloat16: against the plain model with bfloat16 rounding where the engine
+#   rounds (matrix operands, cached keys/values, q), from the same bfloat16
+#   weights.  A value that lies near a rounding boundary may round the other way
+#   in the engine (its 32-bit sums differ from float64 in the last bits), and
+#   such flips spread like the rounding itself; so the bound is the size of that
+#   rounding's own effect on this model and these tokens, measured on the plain
+#   model as max |rounded - exact|, times two.
+TOL = {"float32": 2e-5}
+BF16_NOISE_FACTOR = 2.0
+
+REQUEST_LENGTHS = {"a": 97, "b": 45, "c": 130, "d": 33, "e": 71, "f": 58}
+PROMPT_LENGTHS = {"a": 60, "b": 12, "c": 101, "d": 30, "e": 2, "f": 41}
+ROUNDED = plain.bf16_sites(("gemm_in", "kv_cache", "q"))
+
+
+def make_requests(vocab, seed=7):
+    return {r: random_tokens(n, vocab, seed + i) for i, (r, n) in enumerate(REQUEST_LENGTHS.items())}
+
+
+_plain_cache = {}
+
+
+def plain_logits(folder, requests, dtype):
+    """({request: logits [T, V]}, tolerance) of the plain model for this dtype."""
+    for d in ("float32", "bfloat16"):
+        if (folder, d) not in _plain_cache:
+            cfg, w = read_folder(folder)
+            rnd = ROUNDED if d == "bfloat16" else plain.no_rounding
+            _plain_cache[(folder, d)] = {r: plain.forward(w, cfg, t, rnd) for r, t in requests.items()}
+    want = _plain_cache[(folder, dtype)]
+    if dtype == "float32":
+        return want, TOL["float32"]
+    exact = _plain_cache[(folder, "float32")]
+    noise = max(float(np.abs(want[r] - exact[r]).max()) for r in want)
+    return want, BF16_NOISE_FACTOR * noise
+
+
+def replay(engine, trace):
+    """Feed a trace through Engine.step; {request: [logits row per position]}."""
+    from tinyinfer_amd.engine import StepEntry
+    got = {}
+    for step in trace:
+        logits = engine.step([StepEntry(r, t, w) for r, t, w in step["entries"]])
+        rows = logits.cpu().numpy().astype(np.float64)
+        i = 0
+        for r, t, w in step["entries"]:
+            for _ in w:
+                got.setdefault(r, []).append(rows[i])
+                i += 1
+        for r in step["end"]:
+            engine.release(r)
+        engine.cache.check()
+    return {r: np.stack(v) for r, v in got.items()}
+
+
+def build_engine(folder, dtype, max_tokens, page_size=16):
+    import tinyinfer_amd  # noqa: F401
+    from tinyinfer_amd.engine import Engine
+    return Engine.from_folder(folder, dtype, page_size=page_size, max_tokens=max_tokens, max_requests=4,
+                              max_seq=max_tokens)
+
+
+def worst(got, want):
+    w = 0.0
+    where = None
+    for r in want:
+        assert got[r].shape == want[r].shape, (r, got[r].shape, want[r].shape)
+        d = np.abs(got[r] - want[r]).max(axis=1)
+        if d.max() > w:
+            w, where = float(d.max()), (r, int(d.argmax()))
+    return w, where
+
+
+def make_trace(mode, requests):
+    if mode == "whole":
+        return traces.whole(requests)
+    if mode == "tail":
+        return traces.tail_one_by_one(requests, 32)
+    if mode == "portions":
+        return traces.portions(requests)
+    return traces.mixed(requests, PROMPT_LENGTHS, live=4)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,sharp,page_size", [("A", False, 16), ("B", False, 4), ("B", True, 16), ("C", True, 16)])
+@pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
+def test_engine_matches_plain(model_folders, name, sharp, page_size, dtype, mode):
+    folder = model_folders(name, "bfloat16", sharp)
+    requests = make_requests(CONFIGS[name]["vocab_size"])
+    want, tol = plain_logits(folder, requests, dtype)
+    trace = make_trace(mode, requests)
+    n_tok = traces.max_tokens(trace)
+    engine = build_engine(folder, dtype, n_tok, page_size)
+    got = replay(engine, trace)
+    assert not engine.cache.live_requests()
+    for _, g in engine.cache.paged_groups():
+        assert g.pool.num_free == g.pool.num_pages            # every page came back
+    if mode == "mixed":
+        for _, g in engine.cache.paged_groups():
+            assert g.pool.taken_total > g.pool.num_pages      # pages were handed out again
+    err, where = worst(got, want)
+    print(f"\n[{name} sharp={sharp} P={page_size} {dtype} {mode}] max |engine - plain| = {err:.3e} at {where}"
+          f" (allowed {tol:.3e})")
+    assert err < tol, (err, tol, where)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_float32_weights_stay_32bit(model_folders, dtype):
+    """A folder stored in float32: the float32 engine uses every bit of it."""
+    folder = model_folders("A", "float32")
+    requests = {"a": random_tokens(40, 256, 3)}
+    cfg, w = read_folder(folder)
+    exact = plain.forward(w, cfg, requests["a"])
+    if dtype == "bfloat16":
+        w = {k: (plain.round_bf16(v) if v.ndim == 2 else v) for k, v in w.items()}
+        want = plain.forward(w, cfg, requests["a"], ROUNDED)
+        tol = BF16_NOISE_FACTOR * np.abs(want - exact).max()
+    else:
+        want, tol = exact, TOL["float32"]
+    engine = build_engine(folder, dtype, 64)
+    got = replay(engine, traces.whole(requests))
+    assert np.abs(got["a"] - want).max() < tol
+
+
+def test_first_tokens_and_long_decoding(model_folders):
+    """The first tokens of a sequence one by one from an empty cache, then a long
+    run of single-token steps across many pages."""
+    folder = model_folders("B", "bfloat16", True)
+    toks = random_tokens(400, 1000, 11)
+    cfg, w = read_folder(folder)
+    want = plain.forward(w, cfg, toks)
+    engine = build_engine(folder, "float32", 448, page_size=16)
+    trace = [{"entries": [("r", [t], [0])], "end": []} for t in toks]
+    trace[-1]["end"] = ["r"]
+    got = replay(engine, trace)
+    assert np.abs(got["r"] - want).max() < TOL["float32"]
+
+
+def test_cuts_agree_bitwise_in_float32(model_folders):
+    """In 32-bit every output element is reduced in an order that does not depend
+    on the batch, so different cuts give the same bits, not just close ones."""
+    folder = model_folders("B", "bfloat16", True)
+    requests = make_requests(1000)
+    results = []
+    for mode in ("whole", "portions", "mixed"):
+        trace = make_trace(mode, requests)
+        engine = build_engine(folder, "float32", traces.max_tokens(trace), 4)
+        results.append(replay(engine, trace))
+    for r in requests:
+        assert np.array_equal(results[0][r], results[1][r]), r
+        assert np.array_equal(results[0][r], results[2][r]), r
+
+
+def test_step_refuses_what_it_cannot_run(model_folders):
+    from tinyinfer_amd.engine import StepEntry, EngineError
+    from tinyinfer_amd.cache import OutOfPages
+    engine = build_engine(model_folders("A"), "float32", 64)
+    with pytest.raises(EngineError):
+        engine.step([StepEntry("x", [1, 2, 999], [0])])           # token outside the vocabulary
+    with pytest.raises(EngineError):
+        engine.step([StepEntry("x", [1, 2], [2])])                # wanted place outside the entry
+    with pytest.raises(EngineError):
+        engine.step([StepEntry("x", [1], []), StepEntry("x", [2], [])])
+    engine.step([StepEntry("x", list(range(60)), [59])])
+    free = engine.cache.num_free_pages()
+    with pytest.raises(OutOfPages):
+        engine.step([StepEntry("y", list(range(10)), [0])])       # the pool is full
+    assert engine.cache.num_free_pages() == free and not engine.cache.has("y")
+    engine.cache.check()

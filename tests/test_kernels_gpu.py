@@ -1,0 +1,392 @@
+"""Each kernel alone against a plain PyTorch reference of the same op (float64
+on the CPU), at sizes other than the engine's.  Vectors that the reference's own
+selftest holds are marked with its file:line."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import tinyinfer_amd  # noqa: F401
+    from tinyinfer_amd.ops.kernels import get_ops
+    return get_ops()
+
+
+def dev(t):
+    return t.to("cuda")
+
+
+def f64(t):
+    return t.detach().to("cpu", torch.float64)
+
+
+# ------------------------------------------------------------------ embedding
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed(ops, dtype):
+    g = torch.Generator().manual_seed(5)
+    V, H, M = 301, 72, 9
+    table = torch.randn(V, H, generator=g).to(DT[dtype])
+    tok = torch.randint(0, V, (M,), generator=g, dtype=torch.int32)
+    x = torch.full((M, H), 7.0, device="cuda")
+    ops.embed(dev(table), dev(tok), x)
+    assert torch.equal(x.cpu(), table.float()[tok.long()])
+
+
+# -------------------------------------------------------------------- RMSNorm
+def ref_rmsnorm(x, w, eps):
+    x = f64(x)
+    return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * f64(w)
+
+
+def test_rmsnorm_reference_vector(ops):
+    """n=1024, rows=3, U(-1,1), eps 1e-6, tolerance 1e-4: src/selftest.cpp:74-100."""
+    g = torch.Generator().manual_seed(2)
+    x = torch.rand(3, 1024, generator=g) * 2 - 1
+    w = torch.rand(1024, generator=g) * 2 - 1
+    out = torch.empty(3, 1024, device="cuda")
+    ops.rmsnorm(dev(x), dev(w), 1e-6, out)
+    assert (f64(out) - ref_rmsnorm(x, w, 1e-6)).abs().max() < 1e-4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_rmsnorm_gather_odd_width(ops, dtype):
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(11, 100, generator=g) * 3
+    w = 1 + 0.1 * torch.randn(100, generator=g)
+    rows = torch.tensor([10, 0, 3, 3], dtype=torch.int32)
+    out = torch.empty(4, 100, device="cuda", dtype=DT[dtype])
+    ops.rmsnorm(dev(x), dev(w), 1e-5, out, dev(rows))
+    ref = ref_rmsnorm(x[rows.long()], w, 1e-5)
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    assert (f64(out) - ref).abs().max() < tol
+
+
+def test_rmsnorm_eps_inside_root(ops):
+    """Tiny inputs tell rsqrt(mean + eps) from 1/(rms + eps)."""
+    x = torch.full((1, 64), 1e-4)
+    w = torch.ones(64)
+    out = torch.empty(1, 64, device="cuda")
+    ops.rmsnorm(dev(x), dev(w), 1e-6, out)
+    want = 1e-4 / math.sqrt(1e-8 + 1e-6)
+    assert abs(out[0, 0].item() - want) < 1e-6
+    assert abs(out[0, 0].item() - 1e-4 / (1e-4 + 1e-6)) > 0.5
+
+
+# ----------------------------------------------------------------------- rope
+def ref_rope(x, pos, theta):
+    x = f64(x)
+    hd = x.shape[-1]
+    half = hd // 2
+    k = torch.arange(half, dtype=torch.float64)
+    ang = torch.tensor(pos, dtype=torch.float64)[:, None] * theta ** (-2.0 * k / hd)
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    lo, hi = x[..., :half], x[..., half:]
+    return torch.cat([lo * c - hi * s, lo * s + hi * c], -1)
+
+
+def inv_freq(hd, theta):
+    k = torch.arange(hd // 2, dtype=torch.float64)
+    return (theta ** (-2.0 * k / hd)).to(torch.float32)
+
+
+def test_rope_reference_vector(ops):
+    """rows=2, heads=4, hd=128, theta=1e6, positions {0,5}, tolerance 1e-4: src/selftest.cpp:102-134."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.rand(2, 4, 128, generator=g) * 2 - 1
+    xd = dev(x.clone())
+    ops.rope_neox(xd, dev(torch.tensor([0, 5], dtype=torch.int32)), dev(inv_freq(128, 1e6)))
+    ref = ref_rope(x, [0, 5], 1e6)
+    assert (f64(xd) - ref).abs().max() < 1e-4
+    assert torch.equal(xd[0].cpu(), x[0])           # position 0 is the identity
+
+
+def test_rope_pairs_are_half_split(ops):
+    """Only pair (k, k + hd/2) mixes: a one-hot at dim 1 spreads to dims 1 and 1 + hd/2."""
+    x = torch.zeros(1, 1, 16)
+    x[0, 0, 1] = 1.0
+    xd = dev(x.clone())
+    ops.rope_neox(xd, dev(torch.tensor([3], dtype=torch.int32)), dev(inv_freq(16, 100.0)))
+    nz = set(torch.nonzero(xd[0, 0].cpu().abs() > 1e-7).flatten().tolist())
+    assert nz == {1, 9}
+
+
+# ------------------------------------------------- qk norm + rope + cache write
+class View:
+    def __init__(self, table):
+        self.table = table
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hd,nh,nkv,P", [(48, 3, 3, 4), (128, 4, 2, 16), (16, 6, 2, 8)])
+def test_qk_norm_rope_kv_write(ops, dtype, hd, nh, nkv, P):
+    g = torch.Generator().manual_seed(11)
+    M, pages, W = 7, 9, 5
+    eps, theta = 1e-5, 3e4
+    width = (nh + 2 * nkv) * hd
+    qkv = torch.randn(M, width, generator=g)
+    qw = 1 + 0.1 * torch.randn(hd, generator=g)
+    kw = 1 + 0.1 * torch.randn(hd, generator=g)
+    # two requests: rows 0..3 are request 0 at positions 5..8, rows 4..6 request 1 at 0..2
+    pos = torch.tensor([5, 6, 7, 8, 0, 1, 2], dtype=torch.int32)
+    slot = torch.tensor([0, 0, 0, 0, 1, 1, 1], dtype=torch.int32)
+    table = torch.full((2, W), -1, dtype=torch.int32)
+    table[0, :3] = torch.tensor([7, 2, 5])[: 3]
+    table[1, :1] = 4
+    need0 = 8 // P + 1
+    assert need0 <= 3
+    pool = torch.zeros(pages, 2, nkv, P, hd, dtype=DT[dtype], device="cuda")
+    q_out = torch.empty(M, nh * hd, dtype=DT[dtype], device="cuda")
+    ops.qk_norm_rope_kv_write(dev(qkv), dev(qw), dev(kw), eps, dev(inv_freq(hd, theta)), dev(pos), dev(slot),
+                              View(dev(table)), pool, q_out, nh, nkv, hd)
+    q = qkv[:, :nh * hd].reshape(M, nh, hd)
+    k = qkv[:, nh * hd:(nh + nkv) * hd].reshape(M, nkv, hd)
+    v = qkv[:, (nh + nkv) * hd:].reshape(M, nkv, hd)
+    q_ref = ref_rope(ref_rmsnorm(q, qw, eps), pos.tolist(), theta).reshape(M, -1)
+    k_ref = ref_rope(ref_rmsnorm(k, kw, eps), pos.tolist(), theta)
+    tol = 2e-5 if dtype == "float32" else 3e-2
+    assert (f64(q_out) - q_ref).abs().max() < tol
+    pool_c = f64(pool)
+    touched = torch.zeros(pages, P, dtype=torch.bool)
+    for m in range(M):
+        page = table[slot[m], pos[m] // P].item()
+        r = pos[m].item() % P
+        touched[page, r] = True
+        assert (pool_c[page, 0, :, r, :] - k_ref[m]).abs().max() < tol
+        assert (pool_c[page, 1, :, r, :] - f64(v[m])).abs().max() < (1e-7 if dtype == "float32" else 2e-2)
+    # nothing else was written
+    assert pool_c[~touched.unsqueeze(1).unsqueeze(2).expand(pages, 2, nkv, P)].abs().max() == 0
+
+
+# -------------------------------------------------------------- matrix products
+def ref_linear(a, w):
+    return f64(a) @ f64(w).T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("M,N,K", [(5, 261, 1024), (70, 130, 50), (1, 17, 33), (130, 64, 96)])
+def test_linear_generic_all_epilogues(ops, dtype, M, N, K):
+    """(5, 261, 1024) with U(-1,1) rounded to bfloat16 is the reference's own
+    case: src/selftest.cpp:33-72."""
+    g = torch.Generator().manual_seed(1)
+    a = (torch.rand(M, K, generator=g) * 2 - 1).to(DT[dtype])
+    w = (torch.rand(N, K, generator=g) * 2 - 1).to(DT[dtype])
+    fast = ops.use_fast_gemm
+    ops.use_fast_gemm = False
+    try:
+        ref = ref_linear(a, w)
+        tol = 1e-4 * math.sqrt(K) if dtype == "float32" else 1e-4 * math.sqrt(K)
+        out = torch.empty(M, N, device="cuda")
+        ops.linear(dev(a), dev(w), out, "store")
+        assert (f64(out) - ref).abs().max() < tol
+        base = torch.randn(M, N, generator=g)
+        out = dev(base.clone())
+        ops.linear(dev(a), dev(w), out, "add")
+        assert (f64(out) - (ref + f64(base))).abs().max() < tol
+        out = torch.empty(M, N, device="cuda", dtype=DT[dtype])
+        ops.linear(dev(a), dev(w), out, "store_act")
+        assert (f64(out) - ref).abs().max() < (tol if dtype == "float32" else 0.01 * ref.abs().max())
+        if N % 2 == 0:
+            F = N // 2
+            out = torch.empty(M, F, device="cuda", dtype=DT[dtype])
+            ops.linear(dev(a), dev(w), out, "swiglu")
+            gte, up = ref[:, :F], ref[:, F:]
+            want = gte / (1 + torch.exp(-gte)) * up
+            assert (f64(out) - want).abs().max() < (10 * tol if dtype == "float32" else 0.01 * want.abs().max() + 1e-3)
+    finally:
+        ops.use_fast_gemm = fast
+
+
+def test_linear_identity_and_strided_rows(ops):
+    """W = I copies; rows of A may be strided (a slice of a wider buffer)."""
+    g = torch.Generator().manual_seed(2)
+    wide = torch.randn(6, 40, generator=g)
+    a = dev(wide)[:, 8:24]
+    out = torch.empty(6, 16, device="cuda")
+    ops.linear(a, dev(torch.eye(16)), out, "store")
+    assert torch.equal(out.cpu(), wide[:, 8:24])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_linear_rows_do_not_depend_on_the_batch(ops, dtype):
+    """Row m of the result is the same bits whether it is computed alone or among others."""
+    g = torch.Generator().manual_seed(4)
+    a = torch.randn(37, 200, generator=g).to(DT[dtype])
+    w = torch.randn(150, 200, generator=g).to(DT[dtype])
+    fast = ops.use_fast_gemm
+    ops.use_fast_gemm = False
+    try:
+        full = torch.empty(37, 150, device="cuda")
+        ops.linear(dev(a), dev(w), full, "store")
+        one = torch.empty(1, 150, device="cuda")
+        for m in (0, 17, 36):
+            ops.linear(dev(a[m:m + 1].contiguous()), dev(w), one, "store")
+            assert torch.equal(one[0], full[m])
+    finally:
+        ops.use_fast_gemm = fast
+
+
+# ------------------------------------------------------------------ attention
+def ref_attention(q, k, v, scale, window=None):
+    """q [T, nh, hd], k/v [T, nkv, hd], causal, float64."""
+    q, k, v = f64(q), f64(k), f64(v)
+    T, nh, hd = q.shape
+    G = nh // k.shape[1]
+    out = torch.zeros(T, nh, hd, dtype=torch.float64)
+    for h in range(nh):
+        s = (q[:, h] @ k[:, h // G].T) * scale
+        i = torch.arange(T)
+        mask = i[None, :] > i[:, None]
+        if window is not None:
+            mask |= i[None, :] <= i[:, None] - window
+        s = s.masked_fill(mask, float("-inf"))
+        out[:, h] = torch.softmax(s, -1) @ v[:, h // G]
+    return out
+
+
+def paged_case(dtype, T, nh, nkv, hd, P, seed, sharp=1.0):
+    """One request of T tokens whose pages are scattered over a larger pool."""
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(T, nh, hd, generator=g) * sharp).to(DT[dtype])
+    k = torch.randn(T, nkv, hd, generator=g).to(DT[dtype])
+    v = torch.randn(T, nkv, hd, generator=g).to(DT[dtype])
+    n_pages = -(-T // P)
+    pages = n_pages + 5
+    perm = torch.randperm(pages, generator=g)[:n_pages]
+    pool = torch.randn(pages, 2, nkv, P, hd, generator=g).to(DT[dtype]) * 50    # stale rubbish everywhere
+    for t in range(T):
+        pool[perm[t // P], 0, :, t % P] = k[t]
+        pool[perm[t // P], 1, :, t % P] = v[t]
+    table = torch.full((2, n_pages + 2), -1, dtype=torch.int32)
+    table[1, :n_pages] = perm.to(torch.int32)
+    return q, k, v, pool, table
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T,nh,nkv,hd,P,window", [
+    (37, 4, 2, 64, 16, None), (70, 6, 2, 32, 4, None), (50, 5, 5, 48, 8, 13), (33, 2, 1, 256, 16, None),
+    (300, 4, 4, 16, 16, 64)])
+def test_attention_rows_against_softmax(ops, dtype, T, nh, nkv, hd, P, window):
+    q, k, v, pool, table = paged_case(dtype, T, nh, nkv, hd, P, seed=T + hd, sharp=2.0)
+    scale = 1.0 / math.sqrt(hd)
+    out = torch.empty(T, nh * hd, dtype=DT[dtype], device="cuda")
+    pos = torch.arange(T, dtype=torch.int32)
+    slot = torch.ones(T, dtype=torch.int32)
+    ops.attention_rows(dev(q.reshape(T, -1)), dev(pool), dev(table), dev(pos), dev(slot), out, nh, nkv, hd,
+                       scale, window)
+    ref = ref_attention(q, k, v, scale, window).reshape(T, -1)
+    tol = 2e-5 if dtype == "float32" else 2e-2
+    assert (f64(out) - ref).abs().max() < tol
+
+
+def test_attention_single_key_returns_its_value(ops):
+    """One position: the output is V_0 exactly; and q = 0 gives the mean of the values."""
+    q, k, v, pool, table = paged_case("float32", 5, 2, 1, 32, 4, seed=9)
+    out = torch.empty(5, 64, device="cuda")
+    pos = torch.arange(5, dtype=torch.int32)
+    slot = torch.ones(5, dtype=torch.int32)
+    ops.attention_rows(dev(q.reshape(5, -1)), dev(pool), dev(table), dev(pos), dev(slot), out, 2, 1, 32, 0.3, None)
+    assert torch.equal(out[0, :32].cpu(), v[0, 0])
+    ops.attention_rows(dev(torch.zeros(5, 64)), dev(pool), dev(table), dev(pos), dev(slot), out, 2, 1, 32, 0.3, None)
+    assert (f64(out[4, :32]) - f64(v[:5, 0]).mean(0)).abs().max() < 1e-6
+
+
+def test_attention_far_key_among_hundreds(ops):
+    """One key far back carries almost all the weight: a kernel that skips or
+    misplaces it (a page edge, a split boundary) gives a different row."""
+    T, hd, P = 700, 64, 16
+    g = torch.Generator().manual_seed(21)
+    k = torch.randn(T, 1, hd, generator=g) * 0.1
+    v = torch.randn(T, 1, hd, generator=g)
+    q = torch.randn(T, 1, hd, generator=g) * 0.1
+    far = 17                      # second row of the second page
+    k[far, 0] = 0
+    k[far, 0, 3] = 30.0
+    q[-1, 0, 3] = 30.0
+    n_pages = -(-T // P)
+    pool = torch.zeros(n_pages, 2, 1, P, hd)
+    for t in range(T):
+        pool[t // P, 0, 0, t % P] = k[t, 0]
+        pool[t // P, 1, 0, t % P] = v[t, 0]
+    table = torch.arange(n_pages, dtype=torch.int32)[None, :].contiguous()
+    out = torch.empty(T, hd, device="cuda")
+    ops.attention_rows(dev(q.reshape(T, -1)), dev(pool), dev(table), dev(torch.arange(T, dtype=torch.int32)),
+                       dev(torch.zeros(T, dtype=torch.int32)), out, 1, 1, hd, 1.0 / 8, None)
+    assert (f64(out[-1]) - f64(v[far, 0])).abs().max() < 1e-4
+
+
+# ------------------------------------------------------------------- sampling
+def test_argmax_lowest_index_wins(ops):
+    """Ties go to the lowest index: src/cuda/sample.cu:5-11."""
+    V = 5000
+    logits = torch.zeros(3, V)
+    logits[0, 4000] = logits[0, 123] = logits[0, 124] = 2.5
+    logits[1] = -1.0
+    logits[2, V - 1] = 9.0
+    out = torch.empty(3, dtype=torch.int32, device="cuda")
+    ops.argmax(dev(logits), out)
+    assert out.tolist() == [123, 0, V - 1]
+    g = torch.Generator().manual_seed(0)
+    r = torch.randn(6, 151936, generator=g)
+    out = torch.empty(6, dtype=torch.int32, device="cuda")
+    ops.argmax(dev(r), out)
+    assert out.tolist() == r.argmax(-1).tolist()
+
+
+def run_sample(ops, logits, temp, top_k, top_p, u):
+    n = logits.shape[0]
+    out = torch.empty(n, dtype=torch.int32, device="cuda")
+    ops.sample(dev(logits), dev(torch.full((n,), temp)), dev(torch.full((n,), top_k, dtype=torch.int32)),
+               dev(torch.full((n,), top_p)), dev(torch.tensor(u, dtype=torch.float32)), out)
+    return out.tolist()
+
+
+def test_sample_limits_reduce_to_argmax(ops):
+    g = torch.Generator().manual_seed(1)
+    logits = torch.randn(8, 777, generator=g) * 3
+    u = [0.05, 0.2, 0.35, 0.5, 0.65, 0.8, 0.95, 0.999]
+    want = logits.argmax(-1).tolist()
+    assert run_sample(ops, logits, 0.0, 0, 1.0, u) == want           # temperature 0: greedy
+    assert run_sample(ops, logits, 1e-3, 0, 1.0, u) == want          # T -> 0+
+    assert run_sample(ops, logits, 1.0, 1, 1.0, u) == want           # top-k = 1
+    assert run_sample(ops, logits, 1.0, 0, 1e-6, u) == want          # top-p -> 0
+
+
+def test_sample_matches_inverse_cdf(ops):
+    """The draw is the inverse CDF of softmax(l/T) over the index order at u."""
+    from plain.qwen3_plain import sample_distribution
+    g = torch.Generator().manual_seed(2)
+    V, T = 300, 0.8
+    row = torch.randn(V, generator=g) * 2
+    us = np.linspace(0.001, 0.999, 64).astype(np.float32)
+    logits = row[None, :].repeat(64, 1)
+    for top_k, top_p in ((V, 1.0), (10, 1.0), (V, 0.7), (25, 0.9)):
+        got = run_sample(ops, logits, T, top_k, top_p, us.tolist())
+        p = sample_distribution(row.numpy(), T, top_k, top_p)
+        c = np.cumsum(p)
+        kept = np.nonzero(p)[0]
+        for u, tok in zip(us, got):
+            assert p[tok] > 0, (top_k, top_p, u, tok)
+            lo = c[tok] - p[tok]
+            # u must fall into tok's interval, up to 32-bit rounding of the running sum
+            assert lo - 1e-4 <= u <= c[tok] + 1e-4, (top_k, top_p, u, tok, lo, c[tok])
+        assert set(got) <= set(kept.tolist())
+
+
+def test_sample_frequencies(ops):
+    """Many draws with uniform u reproduce softmax(l/T) (chi-square, tiny vocabulary)."""
+    rng = np.random.default_rng(3)
+    V, n, T = 12, 4096, 1.3
+    row = torch.tensor(rng.normal(size=V) * 1.5, dtype=torch.float32)
+    u = rng.random(n).astype(np.float32)
+    got = np.array(run_sample(ops, row[None, :].repeat(n, 1), T, 0, 1.0, u.tolist()))
+    p = torch.softmax(row.double() / T, -1).numpy()
+    counts = np.bincount(got, minlength=V)
+    chi2 = ((counts - n * p) ** 2 / (n * p)).sum()
+    assert chi2 < 40.0          # 11 degrees of freedom: P(chi2 > 40) < 4e-5

@@ -1,0 +1,182 @@
+"""Compiles the HIP sources for gfx950 into shared libraries, one per source file.
+
+A library's file name carries a hash of its source, the shared header and the
+compiler flags, so a library that exists is always the one its source asks for;
+a changed source compiles again at its next use.  Libraries are written next to
+the sources (the folder travels with the checkout); if that folder cannot be
+written, a per-user folder under the temporary directory is used.
+
+`ensure([...])` compiles only what is asked for, several files at a time, and
+prints a line when each file starts and ends and every few seconds meanwhile.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from typing import Dict, Iterable, List
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ARCH = "gfx950"
+# packed 32-bit float instructions are switched off for every kernel
+FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-shared",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-Wno-unused-command-line-argument"]
+HEADERS = ["common.h"]
+
+# library name -> source file
+SOURCES: Dict[str, str] = {
+    "core": "core.hip",
+    "gemm_generic": "gemm_generic.hip",
+    "attention_generic": "attention_generic.hip",
+    "sampling": "sampling.hip",
+    "gemm_bf16": "gemm_bf16.hip",
+    "attention_bf16": "attention_bf16.hip",
+}
+
+
+class BuildError(RuntimeError):
+    pass
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand):
+            return cand
+    raise BuildError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin): "
+                     "the HIP kernels cannot be compiled")
+
+
+def _digest(name: str) -> str:
+    h = hashlib.sha256()
+    for f in [SOURCES[name]] + HEADERS:
+        with open(os.path.join(HERE, f), "rb") as fh:
+            h.update(fh.read())
+    h.update(" ".join(FLAGS).encode())
+    return h.hexdigest()[:12]
+
+
+def _lib_dirs() -> List[str]:
+    """Where a library may lie: beside the sources first, then the per-user folder."""
+    tmp = os.path.join(tempfile.gettempdir(), f"tinyinfer_amd_{os.getuid()}")
+    return [HERE, tmp]
+
+
+def lib_name(name: str) -> str:
+    return f"libti_{name}.{_digest(name)}.so"
+
+
+def find(name: str):
+    fn = lib_name(name)
+    for d in _lib_dirs():
+        p = os.path.join(d, fn)
+        if os.path.isfile(p):
+            return p
+    return None
+
+
+def _writable_dir() -> str:
+    for d in _lib_dirs():
+        try:
+            os.makedirs(d, exist_ok=True)
+            probe = os.path.join(d, f".probe_{os.getpid()}")
+            with open(probe, "w"):
+                pass
+            os.remove(probe)
+            return d
+        except OSError:
+            continue
+    raise BuildError(f"no folder to write the kernel libraries to (tried {_lib_dirs()})")
+
+
+def _say(msg: str) -> None:
+    print(f"[tinyinfer build] {msg}", file=sys.stderr, flush=True)
+
+
+def _compile(name: str, out_dir: str) -> str:
+    src = os.path.join(HERE, SOURCES[name])
+    final = os.path.join(out_dir, lib_name(name))
+    part = final + f".{os.getpid()}.part"
+    env = dict(os.environ)
+    # the compiler keeps caches under HOME; give it one if the user has none
+    if not env.get("HOME") or not os.access(env["HOME"], os.W_OK):
+        env["HOME"] = tempfile.gettempdir()
+    t0 = time.time()
+    _say(f"compiling {SOURCES[name]} for {ARCH} ...")
+    proc = subprocess.run([_hipcc()] + FLAGS + [src, "-o", part], cwd=HERE, env=env,
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        if os.path.exists(part):
+            os.remove(part)
+        raise BuildError(f"hipcc failed on {SOURCES[name]}:\n{proc.stdout}")
+    os.replace(part, final)
+    # libraries of older versions of this source are of no use any more
+    for f in os.listdir(out_dir):
+        if f.startswith(f"libti_{name}.") and f.endswith(".so") and f != os.path.basename(final):
+            try:
+                os.remove(os.path.join(out_dir, f))
+            except OSError:
+                pass
+    _say(f"compiled {SOURCES[name]} in {time.time() - t0:.1f} s")
+    return final
+
+
+def ensure(names: Iterable[str], force: bool = False) -> Dict[str, str]:
+    """Paths of the libraries `names`, compiling those that are not there
+    (all of them with `force`)."""
+    names = list(names)
+    for n in names:
+        if n not in SOURCES:
+            raise BuildError(f"unknown kernel library {n!r}; known: {sorted(SOURCES)}")
+    paths: Dict[str, str] = {}
+    todo = []
+    for n in names:
+        p = None if force else find(n)
+        if p:
+            paths[n] = p
+        else:
+            todo.append(n)
+    if not todo:
+        return paths
+    out_dir = _writable_dir()
+    errors: List[BaseException] = []
+    done = threading.Event()
+
+    def work(n):
+        try:
+            paths[n] = _compile(n, out_dir)
+        except BaseException as e:  # noqa: BLE001
+            errors.append(e)
+
+    def heartbeat():
+        t0 = time.time()
+        while not done.wait(10.0):
+            _say(f"still compiling ({time.time() - t0:.0f} s) ...")
+
+    threads = [threading.Thread(target=work, args=(n,)) for n in todo]
+    hb = threading.Thread(target=heartbeat, daemon=True)
+    hb.start()
+    limit = max(1, min(8, os.cpu_count() or 1))
+    for i in range(0, len(threads), limit):
+        for t in threads[i:i + limit]:
+            t.start()
+        for t in threads[i:i + limit]:
+            t.join()
+    done.set()
+    if errors:
+        raise errors[0]
+    return paths
+
+
+def build_all(force: bool = True) -> Dict[str, str]:
+    return ensure([n for n, s in SOURCES.items() if os.path.isfile(os.path.join(HERE, s))], force=force)
+
+
+if __name__ == "__main__":
+    for k, v in build_all().items():
+        print(k, v)

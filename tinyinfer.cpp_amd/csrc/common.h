@@ -1,0 +1,106 @@
+// Shared device helpers for the gfx950 kernels: storage types, bfloat16
+// conversion, reductions over 64-lane wavefronts, host-side argument checks.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <math.h>
+
+typedef uint16_t bf16_t;   // bfloat16 bits; arithmetic always happens in float
+
+#define TI_WAVE 64
+
+// dtype codes of the C ABI
+#define TI_F32 0
+#define TI_BF16 1
+
+// epilogues of the matrix products
+#define TI_EPI_STORE_F32 0   // out f32 [M,N] = A W^T
+#define TI_EPI_ADD_F32 1     // out f32 [M,N] += A W^T        (residual sum in 32-bit)
+#define TI_EPI_STORE_ACT 2   // out T   [M,N] = A W^T
+#define TI_EPI_SWIGLU 3      // W = [gate; up] ([2F,K]); out T [M,F] = silu(g) * u
+
+__device__ __forceinline__ float bf2f(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+
+// round to nearest, ties to even; NaN stays NaN
+__device__ __forceinline__ bf16_t f2bf(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ float ld(const T* p);
+template <> __device__ __forceinline__ float ld<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ld<bf16_t>(const bf16_t* p) { return bf2f(*p); }
+template <typename T> __device__ __forceinline__ void st(T* p, float v);
+template <> __device__ __forceinline__ void st<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void st<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
+
+// sum over the `width` consecutive lanes a lane belongs to (width: power of two <= 64);
+// every lane of the group ends with the total
+template <int WIDTH> __device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int o = WIDTH / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, TI_WAVE);
+  return v;
+}
+template <int WIDTH> __device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+  for (int o = WIDTH / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, TI_WAVE));
+  return v;
+}
+
+// sum over a workgroup of NT threads (NT multiple of 64, <= 1024); `red` holds
+// NT/64 floats of LDS.  Every thread gets the total.  Fixed order: deterministic.
+template <int NT> __device__ __forceinline__ float block_sum(float v, float* red) {
+  v = group_sum<TI_WAVE>(v);
+  const int w = threadIdx.x / TI_WAVE;
+  __syncthreads();
+  if ((threadIdx.x & (TI_WAVE - 1)) == 0) red[w] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < NT / TI_WAVE; ++i) t += red[i];
+  return t;
+}
+template <int NT> __device__ __forceinline__ float block_max(float v, float* red) {
+  v = group_max<TI_WAVE>(v);
+  const int w = threadIdx.x / TI_WAVE;
+  __syncthreads();
+  if ((threadIdx.x & (TI_WAVE - 1)) == 0) red[w] = v;
+  __syncthreads();
+  float t = red[0];
+#pragma unroll
+  for (int i = 1; i < NT / TI_WAVE; ++i) t = fmaxf(t, red[i]);
+  return t;
+}
+
+// ---------------------------------------------------------------- host side
+#include <stdarg.h>
+// every kernel library keeps its own last-error text and exports ti_last_error()
+static thread_local char ti_err_buf[512];
+static inline void ti_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(ti_err_buf, sizeof(ti_err_buf), fmt, ap);
+  va_end(ap);
+}
+#define TI_ERROR_API \
+  extern "C" const char* ti_last_error() { return ti_err_buf; }
+
+#define TI_REQUIRE(cond, ...)            \
+  do {                                   \
+    if (!(cond)) {                       \
+      ti_set_error(__VA_ARGS__);         \
+      return 1;                          \
+    }                                    \
+  } while (0)
+
+#define TI_LAUNCH_CHECK()                                                       \
+  do {                                                                          \
+    hipError_t e_ = hipGetLastError();                                          \
+    if (e_ != hipSuccess) {                                                     \
+      ti_set_error("%s:%d: launch failed: %s", __FILE__, __LINE__, hipGetErrorString(e_)); \
+      return 2;                                                                 \
+    }                                                                           \
+  } while (0)

@@ -1,0 +1,200 @@
+// Element-wise and per-row kernels of the step: embedding gather, RMSNorm (with
+// an optional row gather), rotary encoding, and the fused per-head norm +
+// rotation + paged cache write.  All arithmetic is 32-bit; T is the storage
+// type of activations, weights and cache (float or bfloat16).
+#include "common.h"
+
+TI_ERROR_API
+
+// ------------------------------------------------------------------ embedding
+// x[m, :] = float(E[tok[m], :])
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tok,
+                             float* __restrict__ x, int H, int V) {
+  const int m = blockIdx.x;
+  const int t = tok[m];
+  float* row = x + (size_t)m * H;
+  if (t < 0 || t >= V) {   // the host refuses such ids; never read out of bounds
+    for (int i = threadIdx.x; i < H; i += blockDim.x) row[i] = 0.f;
+    return;
+  }
+  const T* src = table + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) row[i] = ld<T>(src + i);
+}
+
+extern "C" int ti_embed(int dtype, const void* table, const int* tok, float* x, int M, int H, int V,
+                        hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && H > 0 && V > 0, "embed: bad sizes M=%d H=%d V=%d", M, H, V);
+  if (M == 0) return 0;
+  if (dtype == TI_F32)
+    embed_kernel<float><<<M, 256, 0, stream>>>((const float*)table, tok, x, H, V);
+  else if (dtype == TI_BF16)
+    embed_kernel<bf16_t><<<M, 256, 0, stream>>>((const bf16_t*)table, tok, x, H, V);
+  else
+    TI_REQUIRE(false, "embed: unknown dtype %d", dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// -------------------------------------------------------------------- RMSNorm
+// out[r, :] = x[src(r), :] * rsqrt(mean(x^2) + eps) * w ; src(r) = rows ? rows[r] : r
+template <typename T>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                               const int* __restrict__ rows, T* __restrict__ out, int H, float eps) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  const float* src = x + (size_t)(rows ? rows[r] : r) * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float v = src[i];
+    ss += v * v;
+  }
+  ss = block_sum<256>(ss, red);
+  const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+  T* dst = out + (size_t)r * H;
+  for (int i = threadIdx.x; i < H; i += 256) st<T>(dst + i, src[i] * scale * w[i]);
+}
+
+extern "C" int ti_rmsnorm(int out_dtype, const float* x, const float* w, const int* rows, void* out,
+                          int n_rows, int H, float eps, hipStream_t stream) {
+  TI_REQUIRE(n_rows >= 0 && H > 0, "rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
+  if (n_rows == 0) return 0;
+  if (out_dtype == TI_F32)
+    rmsnorm_kernel<float><<<n_rows, 256, 0, stream>>>(x, w, rows, (float*)out, H, eps);
+  else if (out_dtype == TI_BF16)
+    rmsnorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(x, w, rows, (bf16_t*)out, H, eps);
+  else
+    TI_REQUIRE(false, "rmsnorm: unknown dtype %d", out_dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------- rotary, by itself
+// In place on f32 x[m, h, :] with row stride `row_stride` floats: pair (k, k+hd/2)
+// turns by pos[m] * inv_freq[k].
+__global__ void rope_neox_kernel(float* __restrict__ x, const int* __restrict__ pos,
+                                 const float* __restrict__ inv_freq, int heads, int hd, long row_stride) {
+  const int m = blockIdx.x;
+  const int half = hd / 2;
+  const float p = (float)pos[m];
+  for (int i = threadIdx.x; i < heads * half; i += blockDim.x) {
+    const int h = i / half, k = i % half;
+    float* v = x + (size_t)m * row_stride + (size_t)h * hd;
+    float s, c;
+    sincosf(p * inv_freq[k], &s, &c);
+    const float lo = v[k], hi = v[k + half];
+    v[k] = lo * c - hi * s;
+    v[k + half] = lo * s + hi * c;
+  }
+}
+
+extern "C" int ti_rope_neox(float* x, const int* pos, const float* inv_freq, int M, int heads, int hd,
+                            long row_stride, hipStream_t stream) {
+  TI_REQUIRE(hd > 0 && hd % 2 == 0, "rope: head_dim %d must be even", hd);
+  TI_REQUIRE(row_stride >= (long)heads * hd, "rope: row stride %ld shorter than heads*head_dim", row_stride);
+  if (M == 0 || heads == 0) return 0;
+  rope_neox_kernel<<<M, 256, 0, stream>>>(x, pos, inv_freq, heads, hd, row_stride);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------- per-head norm + rotation + cache write
+// One workgroup per token; each wave takes whole heads in turn.  For q heads and
+// k heads: RMS-norm over head_dim (if a weight is given), then the half-split
+// rotation (if inv_freq is given).  q goes to q_out (T), k and v into the cache
+// page of the token's position:
+//   pool[page][0 = K | 1 = V][kv head][pos % P][:] with page = table[slot][pos / P].
+// v is copied unchanged.  n_kv == 0: only q is handled (the layer reads another
+// layer's keys and values).
+template <typename T>
+__global__ void qk_norm_rope_kv_write_kernel(
+    const float* __restrict__ qkv, const float* __restrict__ q_w, const float* __restrict__ k_w,
+    const float* __restrict__ inv_freq, const int* __restrict__ pos, const int* __restrict__ slot,
+    const int* __restrict__ table, int table_stride, T* __restrict__ pool, T* __restrict__ q_out,
+    int n_head, int n_kv, int hd, int P, float eps) {
+  const int m = blockIdx.x;
+  const int wave = threadIdx.x / TI_WAVE, lane = threadIdx.x % TI_WAVE;
+  const int n_waves = blockDim.x / TI_WAVE;
+  const int half = hd / 2;
+  const int nq = n_head * hd, nk = n_kv * hd;
+  const float* row = qkv + (size_t)m * (nq + 2 * nk);
+  const int p = pos[m];
+  const float fp = (float)p;
+  size_t page_base = 0;
+  int prow = 0;
+  bool page_ok = false;
+  if (n_kv > 0) {
+    const int page = table[(size_t)slot[m] * table_stride + p / P];
+    page_ok = page >= 0;
+    page_base = (size_t)(page_ok ? page : 0) * 2 * n_kv * P * hd;
+    prow = p % P;
+  }
+  for (int u = wave; u < n_head + 2 * n_kv; u += n_waves) {
+    const bool is_q = u < n_head;
+    const bool is_v = u >= n_head + n_kv;
+    const float* src = row + (size_t)u * hd;
+    T* dst;
+    if (is_q) {
+      dst = q_out + (size_t)m * nq + (size_t)u * hd;
+    } else {
+      if (!page_ok) continue;   // the host reserves pages first; never write astray
+      const int kvh = is_v ? u - n_head - n_kv : u - n_head;
+      dst = pool + page_base + ((size_t)(is_v ? 1 : 0) * n_kv + kvh) * P * hd + (size_t)prow * hd;
+    }
+    if (is_v) {
+      for (int i = lane; i < hd; i += TI_WAVE) st<T>(dst + i, src[i]);
+      continue;
+    }
+    const float* w = is_q ? q_w : k_w;
+    float ss = 0.f;
+    for (int i = lane; i < half; i += TI_WAVE) {
+      const float lo = src[i], hi = src[i + half];
+      ss += lo * lo + hi * hi;
+    }
+    float scale = 1.f;
+    if (w) {
+      ss = group_sum<TI_WAVE>(ss);
+      scale = 1.0f / sqrtf(ss / (float)hd + eps);
+    }
+    for (int i = lane; i < half; i += TI_WAVE) {
+      float lo = src[i] * scale, hi = src[i + half] * scale;
+      if (w) {
+        lo *= w[i];
+        hi *= w[i + half];
+      }
+      if (inv_freq) {
+        float s, c;
+        sincosf(fp * inv_freq[i], &s, &c);
+        const float a = lo * c - hi * s, b = lo * s + hi * c;
+        lo = a;
+        hi = b;
+      }
+      st<T>(dst + i, lo);
+      st<T>(dst + i + half, hi);
+    }
+  }
+}
+
+extern "C" int ti_qk_norm_rope_kv_write(int dtype, const float* qkv, const float* q_w, const float* k_w,
+                                        const float* inv_freq, const int* pos, const int* slot,
+                                        const int* table, int table_stride, void* pool, void* q_out,
+                                        int M, int n_head, int n_kv, int hd, int page_size, float eps,
+                                        hipStream_t stream) {
+  TI_REQUIRE(hd > 0 && hd % 2 == 0, "qk_norm_rope_kv_write: head_dim %d must be even", hd);
+  TI_REQUIRE(n_head > 0 && n_kv >= 0 && page_size > 0 && table_stride > 0,
+             "qk_norm_rope_kv_write: bad sizes heads=%d kv_heads=%d page=%d table_stride=%d", n_head, n_kv,
+             page_size, table_stride);
+  if (M == 0) return 0;
+  if (dtype == TI_F32)
+    qk_norm_rope_kv_write_kernel<float><<<M, 256, 0, stream>>>(qkv, q_w, k_w, inv_freq, pos, slot, table,
+                                                              table_stride, (float*)pool, (float*)q_out,
+                                                              n_head, n_kv, hd, page_size, eps);
+  else if (dtype == TI_BF16)
+    qk_norm_rope_kv_write_kernel<bf16_t><<<M, 256, 0, stream>>>(qkv, q_w, k_w, inv_freq, pos, slot, table,
+                                                               table_stride, (bf16_t*)pool, (bf16_t*)q_out,
+                                                               n_head, n_kv, hd, page_size, eps);
+  else
+    TI_REQUIRE(false, "qk_norm_rope_kv_write: unknown dtype %d", dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}

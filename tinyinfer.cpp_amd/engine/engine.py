@@ -1,0 +1,334 @@
+"""The step function.
+
+`Engine.step(entries)` takes a batch of (request, its next tokens, the places
+whose logits are wanted): portions of prompts beside single decoded tokens, cut
+anywhere.  It reserves pages, runs exactly the tokens it is given as one flat
+batch against the cache that earlier steps left, and returns the logits at the
+wanted places.  The reference's `Inference::forward` has the same shape (flat
+tokens with a position and a sequence id each, logits for chosen rows:
+/root/reference/src/inference.h:26-42, src/inference.cu:178-265) over a
+non-paged cache; its kernel sequence is src/inference.cu:28-72.
+
+Per-step metadata (tokens, positions, block-table rows, output rows, work
+lists) is packed into one pinned host buffer and reaches the device in one copy.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache import CacheManager, CacheStorage, OutOfPages, PagedGroup
+from ..models.model import Model
+from ..ops.kernels import get_ops
+from ..weights.loader import DTYPES
+
+PREFILL_TILE_Q = 64     # query rows per work item of the tiled attention kernels
+
+
+class EngineError(RuntimeError):
+    pass
+
+
+@dataclass
+class StepEntry:
+    """The next tokens of one request, and the places among them (0-based) whose
+    logits are wanted."""
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=tuple)
+
+
+class CacheView:
+    """What a mixer sees of one paged group in this step: the block-table rows of
+    the step's entries, `table[entry][page index] -> page id`."""
+
+    def __init__(self, table: torch.Tensor, page_size: int):
+        self.table = table
+        self.page_size = page_size
+
+
+class StepContext:
+    """Everything a part may touch during one step."""
+
+    def __init__(self, engine: "Engine"):
+        self.engine = engine
+        self.ops = engine.ops
+        self.act_dtype = engine.act_dtype
+        self.f32 = torch.float32
+        self.dtype = engine.dtype
+        self.device = engine.device
+        self.M = 0
+        self.tokens = self.positions = self.slots = None     # int32 [M]
+        self.out_rows = None                                  # int32 [N]
+        # per entry: (row0, n_tokens, start_pos, state_slot); the same as int32 [R, 4] on the device
+        self.entries: List[Tuple[int, int, int, int]] = []
+        self.entry_meta = None
+        self.tiles = None                 # int32 [n_tiles, 2]: (entry, first row) of each query tile
+        self.n_tiles = 0
+        self.decode_only = False
+        self.max_context = 0              # longest context (tokens) any row reads in this step
+        self.run = 0                      # index into the model's run order
+        self._views: Dict[int, CacheView] = {}
+
+    def buf(self, name: str, shape, dtype) -> torch.Tensor:
+        return self.engine._workspace(name, shape, dtype)
+
+    def binding(self, part) -> Tuple[int, int]:
+        return self.engine.model.bindings[self.run][id(part)]
+
+    def kv_pool(self, group: int, layer: int) -> torch.Tensor:
+        return self.engine.storage.kv[group][layer]
+
+    def cache_view(self, group: int) -> CacheView:
+        return self._views[group]
+
+    def state(self, group: int, layer: int) -> torch.Tensor:
+        """[slots, ...] float32 state of one cache layer; index with an entry's state slot."""
+        return self.engine.storage.state[group][layer]
+
+
+class Engine:
+    def __init__(self, model: Model, dtype: str = "bfloat16", page_size: int = 16,
+                 max_tokens: Optional[int] = None, num_pages: Optional[int] = None,
+                 max_requests: int = 64, max_seq: Optional[int] = None, device: str = "cuda"):
+        if dtype not in DTYPES:
+            raise EngineError(f"dtype must be one of {sorted(DTYPES)}, got {dtype!r}")
+        if not torch.cuda.is_available():
+            raise EngineError("no GPU: this engine runs on an AMD GPU only (there is no CPU path)")
+        self.model = model
+        self.dtype = dtype
+        self.act_dtype = DTYPES[dtype]
+        self.device = torch.device(device)
+        self.ops = get_ops()
+        self.page_size = int(page_size)
+        if num_pages is None:
+            if max_tokens is None:
+                raise EngineError("give the cache pool a size: max_tokens or num_pages")
+            num_pages = -(-int(max_tokens) // self.page_size)
+        self.num_pages = int(num_pages)
+        if max_seq is None:
+            max_seq = self.num_pages * self.page_size
+            if model.spec.max_position_embeddings:
+                max_seq = min(max_seq, model.spec.max_position_embeddings)
+        self.max_seq = int(max_seq)
+        self.cache = CacheManager(model.cache_groups, self.page_size, self.num_pages, max_requests, self.max_seq)
+        self.storage = CacheStorage(self.cache, self.act_dtype, self.device)
+        self.table_width = self.cache.max_pages_per_request
+        self._ws: Dict[str, torch.Tensor] = {}
+        self._meta_dev = None
+        self._meta_host: List[torch.Tensor] = []
+        self._meta_events: List[Optional[torch.cuda.Event]] = []
+        self._meta_turn = 0
+        self.steps_run = 0
+
+    # ------------------------------------------------------------- construction
+    @classmethod
+    def from_folder(cls, path: str, dtype: str = "bfloat16", **options) -> "Engine":
+        """Read `path/config.json`, pick the model by its architecture name, load
+        `path/*.safetensors`."""
+        from ..config.base import read_config_json
+        from ..registry import config_and_spec
+        from ..weights.loader import load_weights
+        get_ops().preload(required_libraries(dtype))
+        _, spec = config_and_spec(read_config_json(path))
+        model = Model(spec)
+        load_weights(model, path, dtype, options.get("device", "cuda"))
+        return cls(model, dtype, **options)
+
+    @classmethod
+    def from_config(cls, config: dict, seed: int, dtype: str = "bfloat16", **options) -> "Engine":
+        """Random weights for `config` (a config.json dict), drawn on the device."""
+        from ..registry import config_and_spec
+        from ..weights.loader import load_weights
+        from ..weights.random_init import random_tensors
+        get_ops().preload(required_libraries(dtype))
+        _, spec = config_and_spec(config)
+        model = Model(spec)
+        device = options.get("device", "cuda")
+        tensors = random_tensors(model, seed, DTYPES[dtype], device=device)
+        load_weights(model, tensors, dtype, device)
+        return cls(model, dtype, **options)
+
+    # ---------------------------------------------------------------- workspace
+    def _workspace(self, name: str, shape, dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = f"{name}/{dtype}"
+        t = self._ws.get(key)
+        if t is None or t.numel() < n:
+            cap = max(n, 1)
+            if t is not None:
+                cap = max(cap, int(t.numel() * 1.5))
+            t = torch.empty(cap, dtype=dtype, device=self.device)
+            self._ws[key] = t
+        return t[:n].view(*shape)
+
+    def _meta_buffers(self, n_ints: int):
+        """A pinned host buffer (two take turns) and the device buffer, both >= n_ints."""
+        if self._meta_dev is None or self._meta_dev.numel() < n_ints:
+            cap = max(4096, int(n_ints * 1.5))
+            self._meta_dev = torch.empty(cap, dtype=torch.int32, device=self.device)
+            self._meta_host = [torch.empty(cap, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+            self._meta_events = [None, None]
+        i = self._meta_turn
+        self._meta_turn ^= 1
+        ev = self._meta_events[i]
+        if ev is not None:
+            ev.synchronize()          # the copy that last read this buffer has finished
+        return i, self._meta_host[i], self._meta_dev
+
+    # --------------------------------------------------------------------- step
+    def release(self, request: Hashable) -> None:
+        """The request is over: its pages and its slot are given back."""
+        self.cache.release(request)
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run one batch.  Returns float32 logits [wanted, vocab] in the order of
+        the entries and of their `want` (None if nothing is wanted).  The tensor
+        is engine workspace: it is valid until the next step."""
+        ctx = self.prepare(entries)
+        logits = self.run(ctx)
+        self.finish(ctx)
+        return logits
+
+    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
+        """Check the batch, reserve pages, build and upload the step's metadata."""
+        if not entries:
+            raise EngineError("a step needs at least one entry")
+        V = self.model.vocab_size
+        seen = set()
+        M = 0
+        n_want = 0
+        for e in entries:
+            if e.request in seen:
+                raise EngineError(f"request {e.request!r} appears twice in one step")
+            seen.add(e.request)
+            if len(e.tokens) == 0:
+                raise EngineError(f"request {e.request!r}: an entry needs at least one token")
+            for t in e.tokens:
+                if not (0 <= int(t) < V):
+                    raise EngineError(f"request {e.request!r}: token id {t} is outside the vocabulary [0, {V})")
+            for w in e.want:
+                if not (0 <= int(w) < len(e.tokens)):
+                    raise EngineError(f"request {e.request!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
+            M += len(e.tokens)
+            n_want += len(e.want)
+
+        cache = self.cache
+        # all or nothing: see that every group can cover every entry before taking a page
+        new = [e.request for e in entries if not cache.has(e.request)]
+        if len(new) > cache.num_free_slots():
+            raise EngineError(f"{len(new)} new requests but only {cache.num_free_slots()} free request slots")
+        for gi, g in cache.paged_groups():
+            need = 0
+            for e in entries:
+                base = cache._requests[e.request].reserved if cache.has(e.request) else 0
+                if base + len(e.tokens) > cache.max_seq:
+                    raise EngineError(f"request {e.request!r}: {base + len(e.tokens)} tokens exceed "
+                                      f"max_seq = {cache.max_seq}")
+                need += g.pages_to_cover(e.request if cache.has(e.request) else None, base + len(e.tokens))
+            if need > g.pool.num_free:
+                raise OutOfPages(f"the step needs {need} new pages in cache group {gi}, {g.pool.num_free} are free")
+        for e in entries:
+            if not cache.has(e.request):
+                cache.admit(e.request)
+            cache.reserve(e.request, len(e.tokens))
+        if cache.slots_to_clear:
+            self.storage.clear_slots(cache.slots_to_clear)
+            cache.slots_to_clear.clear()
+
+        ctx = StepContext(self)
+        ctx.M = M
+        R = len(entries)
+        paged = cache.paged_groups()
+        W = self.table_width
+        tiles: List[Tuple[int, int]] = []
+        row0 = 0
+        for i, e in enumerate(entries):
+            n = len(e.tokens)
+            start = cache.length(e.request)
+            ctx.entries.append((row0, n, start, cache.slot(e.request)))
+            ctx.max_context = max(ctx.max_context, start + n)
+            if n > 1:
+                for q0 in range(0, n, PREFILL_TILE_Q):
+                    tiles.append((i, row0 + q0))
+            row0 += n
+        ctx.decode_only = all(n == 1 for _, n, _, _ in ctx.entries)
+        ctx.n_tiles = len(tiles)
+
+        # layout: tokens | positions | slots | out_rows | entries [R,4] | tiles [n_tiles,2] | tables
+        o_tok, o_pos, o_slot = 0, M, 2 * M
+        o_out = 3 * M
+        o_ent = o_out + n_want
+        o_tile = o_ent + 4 * R
+        o_tab = o_tile + 2 * len(tiles)
+        total = o_tab + len(paged) * R * W
+        turn, host, dev = self._meta_buffers(total)
+        h = host.numpy()
+        out_i = o_out
+        for i, (e, (r0, n, start, sslot)) in enumerate(zip(entries, ctx.entries)):
+            h[o_tok + r0:o_tok + r0 + n] = e.tokens
+            h[o_pos + r0:o_pos + r0 + n] = range(start, start + n)
+            h[o_slot + r0:o_slot + r0 + n] = i
+            for w in e.want:
+                h[out_i] = r0 + int(w)
+                out_i += 1
+            h[o_ent + 4 * i:o_ent + 4 * i + 4] = (r0, n, start, sslot)
+        for j, (ei, q0) in enumerate(tiles):
+            h[o_tile + 2 * j] = ei
+            h[o_tile + 2 * j + 1] = q0
+        for k, (gi, g) in enumerate(paged):
+            base = o_tab + k * R * W
+            h[base:base + R * W] = -1
+            for i, e in enumerate(entries):
+                t = g.tables[e.request]
+                h[base + i * W:base + i * W + len(t)] = t
+        dev[:total].copy_(host[:total], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._meta_events[turn] = ev
+
+        ctx.tokens = dev[o_tok:o_tok + M]
+        ctx.positions = dev[o_pos:o_pos + M]
+        ctx.slots = dev[o_slot:o_slot + M]
+        ctx.out_rows = dev[o_out:o_out + n_want] if n_want else None
+        ctx.entry_meta = dev[o_ent:o_ent + 4 * R].view(R, 4)
+        ctx.tiles = dev[o_tile:o_tile + 2 * len(tiles)].view(-1, 2) if tiles else None
+        for k, (gi, g) in enumerate(paged):
+            base = o_tab + k * R * W
+            ctx._views[gi] = CacheView(dev[base:base + R * W].view(R, W), self.page_size)
+        ctx._entries_in = list(entries)
+        return ctx
+
+    def run(self, ctx: StepContext) -> Optional[torch.Tensor]:
+        """The model over the step's tokens: embedding, the layers in run order,
+        then final norm and head on the wanted rows only."""
+        model = self.model
+        x = ctx.buf("x", (ctx.M, model.hidden_size), torch.float32)
+        model.embedding.forward(ctx, ctx.tokens, x)
+        for r, li in enumerate(model.run_order):
+            ctx.run = r
+            model.blocks[li].forward(ctx, x)
+        if ctx.out_rows is None:
+            return None
+        h = model.final_norm.forward(ctx, x, rows=ctx.out_rows)
+        return model.head.forward(ctx, h)
+
+    def finish(self, ctx: StepContext) -> None:
+        for e in ctx._entries_in:
+            self.cache.commit(e.request, len(e.tokens))
+        self.steps_run += 1
+
+
+def required_libraries(dtype: str):
+    """The kernel libraries a model of this dtype needs (what a first call compiles)."""
+    import os
+    from ..csrc import build
+    libs = ["core", "gemm_generic", "attention_generic", "sampling"]
+    if dtype == "bfloat16":
+        libs += [n for n in ("gemm_bf16", "attention_bf16")
+                 if os.path.isfile(os.path.join(build.HERE, build.SOURCES[n]))]
+    return libs

@@ -1,0 +1,250 @@
+"""The kernels, as Python calls on torch tensors.
+
+Each call checks devices, dtypes and shapes on the host, then launches the
+hand-written HIP kernel on torch's current stream through the C ABI of the
+kernel libraries (`csrc/`).  Nothing here computes with torch, and nothing falls
+back to the CPU or to a library: without a GPU or without the compiled
+libraries a call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, Optional
+
+import torch
+
+from ..csrc import build as _build
+
+F32, BF16 = 0, 1
+EPI = {"store": 0, "add": 1, "store_act": 2, "swiglu": 3}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return F32
+    if dt == torch.bfloat16:
+        return BF16
+    raise KernelError(f"dtype {dt} is not served by the kernels (float32, bfloat16)")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+class Ops:
+    """Loads kernel libraries on first use and exposes one method per op."""
+
+    def __init__(self):
+        self._libs: Dict[str, ctypes.CDLL] = {}
+        # switches for tests and measurements: force the generic kernels
+        import os
+        have = lambda n: os.path.isfile(os.path.join(_build.HERE, _build.SOURCES[n]))
+        self.use_fast_gemm = have("gemm_bf16")
+        self.use_fast_attention = have("attention_bf16")
+
+    # ------------------------------------------------------------------ loading
+    def lib(self, name: str) -> ctypes.CDLL:
+        lib = self._libs.get(name)
+        if lib is None:
+            if not torch.cuda.is_available():
+                raise KernelError("no GPU: the kernels of this framework run on an AMD GPU (gfx950) only")
+            path = _build.ensure([name])[name]
+            lib = ctypes.CDLL(path)
+            lib.ti_last_error.restype = ctypes.c_char_p
+            self._libs[name] = lib
+        return lib
+
+    def preload(self, names):
+        """Compile (if needed, several at a time) and load the libraries `names`."""
+        need = [n for n in names if n not in self._libs]
+        if need:
+            if not torch.cuda.is_available():
+                raise KernelError("no GPU: the kernels of this framework run on an AMD GPU (gfx950) only")
+            _build.ensure(need)
+            for n in need:
+                self.lib(n)
+
+    @staticmethod
+    def _check(lib, rc, what):
+        if rc != 0:
+            raise KernelError(f"{what}: {lib.ti_last_error().decode()}")
+
+    @staticmethod
+    def _stream():
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    @staticmethod
+    def _dev(*ts):
+        for t in ts:
+            if t is not None and not t.is_cuda:
+                raise KernelError("kernel arguments must live on the GPU")
+
+    # --------------------------------------------------------------------- ops
+    def embed(self, table, tokens, x):
+        V, H = table.shape
+        M = tokens.shape[0]
+        self._dev(table, tokens, x)
+        if x.shape != (M, H) or x.dtype != torch.float32 or tokens.dtype != torch.int32:
+            raise KernelError(f"embed: x {tuple(x.shape)}/{x.dtype}, tokens {tokens.dtype} do not fit [{M},{H}]")
+        if not (table.is_contiguous() and x.is_contiguous()):
+            raise KernelError("embed: table and x must be contiguous")
+        lib = self.lib("core")
+        rc = lib.ti_embed(_code(table.dtype), _ptr(table), _ptr(tokens), _ptr(x), M, H, V, self._stream())
+        self._check(lib, rc, "embed")
+
+    def rmsnorm(self, x, w, eps, out, rows=None):
+        H = x.shape[-1]
+        n = x.shape[0] if rows is None else rows.shape[0]
+        self._dev(x, w, out, rows)
+        if x.dtype != torch.float32 or w.dtype != torch.float32 or w.shape != (H,):
+            raise KernelError(f"rmsnorm: x {x.dtype} / weight {tuple(w.shape)} {w.dtype} do not fit width {H}")
+        if out.shape != (n, H) or not out.is_contiguous() or not x.is_contiguous():
+            raise KernelError(f"rmsnorm: out {tuple(out.shape)} does not fit [{n},{H}] or is not contiguous")
+        if rows is not None and rows.dtype != torch.int32:
+            raise KernelError("rmsnorm: rows must be int32")
+        lib = self.lib("core")
+        rc = lib.ti_rmsnorm(_code(out.dtype), _ptr(x), _ptr(w), _ptr(rows), _ptr(out), n, H,
+                            ctypes.c_float(eps), self._stream())
+        self._check(lib, rc, "rmsnorm")
+
+    def rope_neox(self, x, positions, inv_freq):
+        """In place on f32 x [M, heads, hd]; the last two dims contiguous, rows may be strided."""
+        M, heads, hd = x.shape
+        self._dev(x, positions, inv_freq)
+        if x.dtype != torch.float32 or x.stride(2) != 1 or x.stride(1) != hd:
+            raise KernelError("rope: x must be float32 with contiguous heads")
+        if inv_freq.shape != (hd // 2,) or inv_freq.dtype != torch.float32 or positions.dtype != torch.int32:
+            raise KernelError("rope: inv_freq must be float32 [hd/2], positions int32")
+        lib = self.lib("core")
+        rc = lib.ti_rope_neox(_ptr(x), _ptr(positions), _ptr(inv_freq), M, heads, hd,
+                              ctypes.c_long(x.stride(0)), self._stream())
+        self._check(lib, rc, "rope")
+
+    def qk_norm_rope_kv_write(self, qkv, q_w, k_w, eps, inv_freq, positions, slots, view, pool, q_out,
+                              heads, kv_heads, head_dim):
+        """qkv f32 [M, (heads + 2 kv_heads) hd] -> q_out T [M, heads hd] and the cache pages.
+        kv_heads = 0: only q (nothing is written to the cache)."""
+        M = qkv.shape[0]
+        width = (heads + 2 * kv_heads) * head_dim
+        self._dev(qkv, q_w, k_w, inv_freq, positions, slots, view.table, pool, q_out)
+        if qkv.shape != (M, width) or qkv.dtype != torch.float32 or not qkv.is_contiguous():
+            raise KernelError(f"qk_norm_rope_kv_write: qkv {tuple(qkv.shape)} {qkv.dtype} does not fit [{M},{width}]")
+        if q_out.shape != (M, heads * head_dim) or not q_out.is_contiguous():
+            raise KernelError("qk_norm_rope_kv_write: q_out has the wrong shape")
+        for wt in (q_w, k_w):
+            if wt is not None and (wt.shape != (head_dim,) or wt.dtype != torch.float32):
+                raise KernelError("qk_norm_rope_kv_write: norm weights must be float32 [head_dim]")
+        if inv_freq is not None and (inv_freq.shape != (head_dim // 2,) or inv_freq.dtype != torch.float32):
+            raise KernelError("qk_norm_rope_kv_write: inv_freq must be float32 [head_dim/2]")
+        if kv_heads > 0:
+            if pool.dim() != 5 or pool.shape[1] != 2 or pool.shape[2] != kv_heads or pool.shape[4] != head_dim \
+                    or pool.dtype != q_out.dtype or not pool.is_contiguous():
+                raise KernelError(f"qk_norm_rope_kv_write: pool {tuple(pool.shape)} {pool.dtype} does not fit "
+                                  f"[pages,2,{kv_heads},P,{head_dim}] of {q_out.dtype}")
+        lib = self.lib("core")
+        rc = lib.ti_qk_norm_rope_kv_write(
+            _code(q_out.dtype), _ptr(qkv), _ptr(q_w), _ptr(k_w), _ptr(inv_freq), _ptr(positions), _ptr(slots),
+            _ptr(view.table), view.table.shape[1], _ptr(pool), _ptr(q_out), M, heads, kv_heads, head_dim,
+            pool.shape[3], ctypes.c_float(eps), self._stream())
+        self._check(lib, rc, "qk_norm_rope_kv_write")
+
+    # ---------------------------------------------------------- matrix products
+    def linear(self, a, w, out, epilogue: str):
+        """out (op)= a w^T.  a: T [M, K] (rows may be strided); w: T [N, K] contiguous.
+        epilogue: "store" f32 out = ; "add" f32 out += ; "store_act" T out = ;
+        "swiglu": w is [2F, K] = [gate; up], T out [M, F] = silu(gate) * up."""
+        epi = EPI[epilogue]
+        M, K = a.shape
+        rows = w.shape[0]
+        N = rows // 2 if epilogue == "swiglu" else rows
+        self._dev(a, w, out)
+        if w.shape[1] != K or a.dtype != w.dtype or a.stride(1) != 1 or not w.is_contiguous():
+            raise KernelError(f"linear: a {tuple(a.shape)} {a.dtype} and w {tuple(w.shape)} {w.dtype} do not fit")
+        if epilogue == "swiglu" and rows % 2:
+            raise KernelError("linear: a SwiGLU weight needs an even number of rows")
+        want = torch.float32 if epilogue in ("store", "add") else a.dtype
+        if out.shape != (M, N) or out.dtype != want or not out.is_contiguous():
+            raise KernelError(f"linear[{epilogue}]: out {tuple(out.shape)} {out.dtype} does not fit [{M},{N}] {want}")
+        if M == 0:
+            return
+        code = _code(a.dtype)
+        if code == BF16 and self.use_fast_gemm and self._linear_bf16(a, w, out, epi, M, N, K):
+            return
+        lib = self.lib("gemm_generic")
+        rc = lib.ti_gemm_generic(code, _ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi,
+                                 self._stream())
+        self._check(lib, rc, "linear")
+
+    def _linear_bf16(self, a, w, out, epi, M, N, K) -> bool:
+        """The MFMA kernels; False if they refuse the shape (the generic kernel takes it)."""
+        if K % 8 or a.stride(0) % 8 or a.data_ptr() % 16 or w.data_ptr() % 16:
+            return False
+        lib = self.lib("gemm_bf16")
+        rc = lib.ti_gemm_bf16(_ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi, self._stream())
+        if rc == 3:          # "shape not served": not an error
+            return False
+        self._check(lib, rc, "linear(bf16)")
+        return True
+
+    # ----------------------------------------------------------------- attention
+    def attention_rows(self, q, pool, table, positions, slots, out, heads, kv_heads, head_dim, scale, window):
+        M = q.shape[0]
+        self._dev(q, pool, table, positions, slots, out)
+        if q.shape != (M, heads * head_dim) or out.shape != q.shape or q.dtype != pool.dtype or out.dtype != q.dtype:
+            raise KernelError("attention: q/out/pool shapes or dtypes do not fit")
+        if pool.dim() != 5 or pool.shape[1] != 2 or pool.shape[2] != kv_heads or pool.shape[4] != head_dim:
+            raise KernelError(f"attention: pool {tuple(pool.shape)} does not fit [pages,2,{kv_heads},P,{head_dim}]")
+        if not (q.is_contiguous() and out.is_contiguous() and pool.is_contiguous() and table.is_contiguous()):
+            raise KernelError("attention: arguments must be contiguous")
+        lib = self.lib("attention_generic")
+        rc = lib.ti_attention_rows(_code(q.dtype), _ptr(q), _ptr(pool), _ptr(table), table.shape[1],
+                                   _ptr(positions), _ptr(slots), _ptr(out), M, heads, kv_heads, head_dim,
+                                   pool.shape[3], ctypes.c_float(scale), int(window or 0), self._stream())
+        self._check(lib, rc, "attention")
+
+    def attention(self, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window):
+        """Attention of every row of the step over its request's pages."""
+        if q.dtype == torch.bfloat16 and self.use_fast_attention:
+            from . import attention_bf16
+            if attention_bf16.run(self, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window):
+                return
+        self.attention_rows(q, pool, view.table, ctx.positions, ctx.slots, out, heads, kv_heads, head_dim,
+                            scale, window)
+
+    # ------------------------------------------------------------------ sampling
+    def argmax(self, logits, out):
+        n, V = logits.shape
+        self._dev(logits, out)
+        if logits.dtype != torch.float32 or not logits.is_contiguous() or out.dtype != torch.int32 or out.shape[0] < n:
+            raise KernelError("argmax: logits must be contiguous float32 [n, V], out int32 [n]")
+        lib = self.lib("sampling")
+        rc = lib.ti_argmax(_ptr(logits), _ptr(out), n, V, self._stream())
+        self._check(lib, rc, "argmax")
+
+    def sample(self, logits, temperature, top_k, top_p, uniform, out):
+        n, V = logits.shape
+        self._dev(logits, temperature, top_k, top_p, uniform, out)
+        if logits.dtype != torch.float32 or not logits.is_contiguous():
+            raise KernelError("sample: logits must be contiguous float32 [n, V]")
+        for t, dt in ((temperature, torch.float32), (top_k, torch.int32), (top_p, torch.float32),
+                      (uniform, torch.float32), (out, torch.int32)):
+            if t.dtype != dt or t.shape[0] < n:
+                raise KernelError("sample: per-row arguments must be float32/int32 [n]")
+        lib = self.lib("sampling")
+        rc = lib.ti_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform), _ptr(out),
+                           n, V, self._stream())
+        self._check(lib, rc, "sample")
+
+
+_OPS: Optional[Ops] = None
+
+
+def get_ops() -> Ops:
+    global _OPS
+    if _OPS is None:
+        _OPS = Ops()
+    return _OPS

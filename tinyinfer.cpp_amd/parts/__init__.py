@@ -1,0 +1,5 @@
+"""Parts a layer is put together from.  Importing the package registers the
+built-in kinds."""
+from .registry import register_part, build_part, registered_parts
+from .base import Part
+from . import norm, rotary, attention, ffn, embedding, block  # noqa: F401  (registration)
