@@ -26,6 +26,13 @@ CONFIGS = {
               vocab_size=517, rope_theta=500000.0, rms_norm_eps=3e-6, tie_word_embeddings=False,
               attention_bias=False, hidden_act="silu", max_position_embeddings=4096,
               use_sliding_window=True, sliding_window=20, max_window_layers=2),
+    # 3 layers, width 96, 3 heads on one kv head, head 64 (served by the matrix-core attention
+    # kernels), a window of 37 on layers 1 and 2
+    "D": dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=3, hidden_size=96,
+              num_attention_heads=3, num_key_value_heads=1, head_dim=64, intermediate_size=160,
+              vocab_size=333, rope_theta=200000.0, rms_norm_eps=2e-6, tie_word_embeddings=True,
+              attention_bias=False, hidden_act="silu", max_position_embeddings=4096,
+              layer_types=["full_attention", "sliding_attention", "sliding_attention"], sliding_window=37),
 }
 
 

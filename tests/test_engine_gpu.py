@@ -100,14 +100,16 @@ def make_trace(mode, requests):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,sharp,page_size", [("A", False, 16), ("B", False, 4), ("B", True, 16), ("C", True, 16)])
+@pytest.mark.parametrize("name,sharp,page_size", [("A", False, 16), ("B", False, 4), ("B", True, 16), ("C", True, 16), ("D", True, 16)])
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_engine_matches_plain(model_folders, name, sharp, page_size, dtype, mode):
     folder = model_folders(name, "bfloat16", sharp)
     requests = make_requests(CONFIGS[name]["vocab_size"])
     want, tol = plain_logits(folder, requests, dtype)
     trace = make_trace(mode, requests)
-    n_tok = traces.max_tokens(trace)
+    # the tightest pool that holds the trace, so that pages given back are handed out again
+    n_tok = traces.max_pages(trace, page_size) * page_size
+    assert n_tok <= traces.max_tokens(trace)
     engine = build_engine(folder, dtype, n_tok, page_size)
     got = replay(engine, trace)
     assert not engine.cache.live_requests()

@@ -159,9 +159,13 @@ def test_qk_norm_rope_kv_write(ops, dtype, hd, nh, nkv, P):
         r = pos[m].item() % P
         touched[page, r] = True
         assert (pool_c[page, 0, :, r, :] - k_ref[m]).abs().max() < tol
-        assert (pool_c[page, 1, :, r, :] - f64(v[m])).abs().max() < (1e-7 if dtype == "float32" else 2e-2)
+        vt = pool_c[page, 1].reshape(nkv, hd, P)              # values lie transposed in a page: [head][d][row]
+        assert (vt[:, :, r] - f64(v[m])).abs().max() < (1e-7 if dtype == "float32" else 2e-2)
     # nothing else was written
-    assert pool_c[~touched.unsqueeze(1).unsqueeze(2).expand(pages, 2, nkv, P)].abs().max() == 0
+    keys = pool_c[:, 0]                                        # [pages, nkv, P, hd]
+    vals = pool_c[:, 1].reshape(pages, nkv, hd, P).transpose(2, 3)
+    mask = ~touched[:, None, :, None].expand(pages, nkv, P, hd)
+    assert keys[mask].abs().max() == 0 and vals[mask].abs().max() == 0
 
 
 # -------------------------------------------------------------- matrix products
@@ -260,9 +264,10 @@ def paged_case(dtype, T, nh, nkv, hd, P, seed, sharp=1.0):
     pages = n_pages + 5
     perm = torch.randperm(pages, generator=g)[:n_pages]
     pool = torch.randn(pages, 2, nkv, P, hd, generator=g).to(DT[dtype]) * 50    # stale rubbish everywhere
+    vt = pool[:, 1].reshape(pages, nkv, hd, P)                 # values lie transposed in a page
     for t in range(T):
         pool[perm[t // P], 0, :, t % P] = k[t]
-        pool[perm[t // P], 1, :, t % P] = v[t]
+        vt[perm[t // P], :, :, t % P] = v[t]
     table = torch.full((2, n_pages + 2), -1, dtype=torch.int32)
     table[1, :n_pages] = perm.to(torch.int32)
     return q, k, v, pool, table
@@ -311,9 +316,10 @@ def test_attention_far_key_among_hundreds(ops):
     q[-1, 0, 3] = 30.0
     n_pages = -(-T // P)
     pool = torch.zeros(n_pages, 2, 1, P, hd)
+    vt = pool[:, 1].reshape(n_pages, 1, hd, P)
     for t in range(T):
         pool[t // P, 0, 0, t % P] = k[t, 0]
-        pool[t // P, 1, 0, t % P] = v[t, 0]
+        vt[t // P, 0, :, t % P] = v[t, 0]
     table = torch.arange(n_pages, dtype=torch.int32)[None, :].contiguous()
     out = torch.empty(T, hd, device="cuda")
     ops.attention_rows(dev(q.reshape(T, -1)), dev(pool), dev(table), dev(torch.arange(T, dtype=torch.int32)),
@@ -390,3 +396,189 @@ def test_sample_frequencies(ops):
     counts = np.bincount(got, minlength=V)
     chi2 = ((counts - n * p) ** 2 / (n * p)).sum()
     assert chi2 < 40.0          # 11 degrees of freedom: P(chi2 > 40) < 4e-5
+
+
+# ------------------------------------------------- bfloat16 matrix-core products
+@pytest.mark.parametrize("M,N,K", [
+    (1, 48, 64), (5, 261, 1024), (8, 1000, 96), (16, 17, 200), (17, 130, 72), (33, 64, 3072), (64, 151, 256),
+    (65, 130, 96), (128, 128, 32), (200, 261, 1024), (300, 520, 104), (77, 1000, 1032)])
+def test_linear_bf16_matrix_cores(ops, M, N, K):
+    """The skinny (M <= 64) and tiled (M > 64) MFMA kernels against float64, every
+    epilogue, at sizes that are no multiples of their tiles.  (5, 261, 1024) is the
+    reference's own case, src/selftest.cpp:33-72."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    g = torch.Generator().manual_seed(M * 7 + N)
+    a = (torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16)
+    w = (torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16)
+    ref = ref_linear(a, w)
+    tol = 2e-5 * K                         # 32-bit accumulation of K products of size <= 1
+    out = torch.empty(M, N, device="cuda")
+    ops.linear(dev(a), dev(w), out, "store")
+    assert (f64(out) - ref).abs().max() < tol
+    base = torch.randn(M, N, generator=g)
+    out = dev(base.clone())
+    ops.linear(dev(a), dev(w), out, "add")
+    assert (f64(out) - (ref + f64(base))).abs().max() < tol
+    out = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+    ops.linear(dev(a), dev(w), out, "store_act")
+    assert (f64(out) - ref).abs().max() < 0.005 * ref.abs().max() + tol
+    if N % 2 == 0:
+        F = N // 2
+        out = torch.empty(M, F, device="cuda", dtype=torch.bfloat16)
+        ops.linear(dev(a), dev(w), out, "swiglu")
+        gte, up = ref[:, :F], ref[:, F:]
+        want = gte / (1 + torch.exp(-gte)) * up
+        assert (f64(out) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
+
+
+def test_linear_bf16_rows_do_not_depend_on_the_batch(ops):
+    """Within one kernel a row's bits do not depend on the other rows."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    g = torch.Generator().manual_seed(4)
+    a = torch.randn(200, 264, generator=g).to(torch.bfloat16)
+    w = torch.randn(150, 264, generator=g).to(torch.bfloat16)
+    full = torch.empty(200, 150, device="cuda")
+    ops.linear(dev(a), dev(w), full, "store")                   # tiled
+    part = torch.empty(70, 150, device="cuda")
+    ops.linear(dev(a[100:170].contiguous()), dev(w), part, "store")     # tiled, other rows
+    assert torch.equal(part, full[100:170])
+    small = torch.empty(40, 150, device="cuda")
+    ops.linear(dev(a[:40].contiguous()), dev(w), small, "store")        # skinny
+    one = torch.empty(1, 150, device="cuda")
+    for m in (0, 17, 39):
+        ops.linear(dev(a[m:m + 1].contiguous()), dev(w), one, "store")  # skinny, alone
+        assert torch.equal(one[0], small[m])
+
+
+# ---------------------------------------------- bfloat16 matrix-core attention
+class FakeCtx:
+    """The fields of a step context that the attention dispatch reads."""
+
+    def __init__(self, entries, decode_rows_only=False):
+        # entries: [(n_tokens, start_pos)], rows laid out in order
+        self.entries = entries
+        pos, slot, tiles, dec, meta = [], [], [], [], []
+        row0 = 0
+        for e, (n, start) in enumerate(entries):
+            meta.append([row0, n, start, 0])
+            pos += list(range(start, start + n))
+            slot += [e] * n
+            if n > 1:
+                tiles += [[e, row0 + q0] for q0 in range(0, n, 64)]
+            else:
+                dec.append(row0)
+            row0 += n
+        self.M = row0
+        self.decode_only = not tiles
+        self.positions = dev(torch.tensor(pos, dtype=torch.int32))
+        self.slots = dev(torch.tensor(slot, dtype=torch.int32))
+        self.entry_meta = dev(torch.tensor(meta, dtype=torch.int32))
+        self.tiles = dev(torch.tensor(tiles, dtype=torch.int32)) if tiles else None
+        self.n_tiles = len(tiles)
+        self.decode_rows = None if self.decode_only else (dev(torch.tensor(dec, dtype=torch.int32)) if dec else None)
+        self.n_decode_rows = 0 if self.decode_only else len(dec)
+        self.max_context = self.split_context = max(s + n for n, s in entries)
+        self._bufs = {}
+
+    def buf(self, name, shape, dtype):
+        t = torch.empty(tuple(shape), dtype=dtype, device="cuda")
+        self._bufs[name] = t
+        return t
+
+
+def fast_attention_case(ops, entries_tokens, nh, nkv, hd, P, window, seed, sharp=2.0):
+    """Several requests with full contexts in a scattered pool; the step holds the
+    last `n` tokens of each.  Returns (got, want) for the step's rows."""
+    from tinyinfer_amd.ops import attention_bf16
+    g = torch.Generator().manual_seed(seed)
+    lens = [s + n for n, s in entries_tokens]
+    n_pages_each = [-(-L // P) for L in lens]
+    pages = sum(n_pages_each) + 7
+    perm = torch.randperm(pages, generator=g)
+    pool = (torch.randn(pages, 2, nkv, P, hd, generator=g) * 30).to(torch.bfloat16)
+    pool[0, 0, 0, 0, 0] = float("nan")                     # rubbish may be anything
+    vt = pool[:, 1].reshape(pages, nkv, hd, P)
+    W = max(n_pages_each) + 1
+    table = torch.full((len(lens), W), -1, dtype=torch.int32)
+    qs, refs = [], []
+    used = 0
+    for e, ((n, start), L) in enumerate(zip(entries_tokens, lens)):
+        q = (torch.randn(L, nh, hd, generator=g) * sharp).to(torch.bfloat16)
+        k = torch.randn(L, nkv, hd, generator=g).to(torch.bfloat16)
+        v = torch.randn(L, nkv, hd, generator=g).to(torch.bfloat16)
+        mine = perm[used:used + n_pages_each[e]]
+        used += n_pages_each[e]
+        table[e, :len(mine)] = mine.to(torch.int32)
+        # the unwritten tail of the last page holds NaN: nothing of it may leak
+        pool[mine[-1], 0] = float("nan")
+        vt[mine[-1]] = float("nan")
+        for t in range(L):
+            pool[mine[t // P], 0, :, t % P] = k[t]
+            vt[mine[t // P], :, :, t % P] = v[t]
+        ref = ref_attention(q, k, v, 1.0 / math.sqrt(hd), window)
+        qs.append(q[start:])
+        refs.append(ref[start:])
+    qd = dev(torch.cat(qs).reshape(-1, nh * hd))
+    out = torch.zeros_like(qd)
+    ctx = FakeCtx(entries_tokens)
+    ok = attention_bf16.run(ops, ctx, View(dev(table)), qd, dev(pool), out, nh, nkv, hd, 1.0 / math.sqrt(hd), window)
+    assert ok
+    return f64(out), torch.cat(refs).reshape(-1, nh * hd)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,P,window", [
+    (4, 2, 64, 16, None), (6, 2, 32, 16, None), (16, 8, 128, 16, None), (3, 1, 128, 32, None),
+    (4, 4, 64, 16, 40), (20, 1, 32, 16, None), (8, 2, 128, 16, 300)])
+def test_attention_bf16_decode_rows(ops, nh, nkv, hd, P, window):
+    """Single-token entries at many context lengths, page edges included, split over the context."""
+    if not ops.use_fast_attention:
+        pytest.skip("bfloat16 attention kernels are switched off")
+    entries = [(1, s) for s in (0, 1, 15, 16, 17, 31, 32, 100, 511, 512, 777, 1500)]
+    got, want = fast_attention_case(ops, entries, nh, nkv, hd, P, window, seed=nh * 100 + hd)
+    assert torch.isfinite(got).all()
+    assert (got - want).abs().max() < 2e-2
+
+
+@pytest.mark.parametrize("nh,nkv,hd,P,window", [
+    (4, 2, 64, 16, None), (6, 2, 32, 16, None), (4, 2, 128, 16, None), (2, 1, 128, 32, None),
+    (4, 4, 64, 16, 40), (2, 2, 32, 16, 7)])
+def test_attention_bf16_portions_and_mixed(ops, nh, nkv, hd, P, window):
+    """Portions of every size, starting anywhere (a page's edge, the middle of a
+    page, the start of a request), beside decode rows."""
+    if not ops.use_fast_attention:
+        pytest.skip("bfloat16 attention kernels are switched off")
+    entries = [(2, 0), (7, 30), (1, 99), (16, 16), (17, 15), (64, 0), (65, 63), (130, 41), (1, 0), (3, 300), (200, 5)]
+    got, want = fast_attention_case(ops, entries, nh, nkv, hd, P, window, seed=nh * 10 + hd)
+    assert torch.isfinite(got).all()
+    assert (got - want).abs().max() < 2e-2
+
+
+def test_attention_bf16_far_key(ops):
+    """One key far back carries the weight, for a decode row and for a row inside a portion."""
+    if not ops.use_fast_attention:
+        pytest.skip("bfloat16 attention kernels are switched off")
+    from tinyinfer_amd.ops import attention_bf16
+    T, hd, P = 1000, 64, 16
+    g = torch.Generator().manual_seed(21)
+    k = (torch.randn(T, 1, hd, generator=g) * 0.1).to(torch.bfloat16)
+    v = torch.randn(T, 1, hd, generator=g).to(torch.bfloat16)
+    far = 17
+    k[far, 0] = 0
+    k[far, 0, 3] = 30.0
+    n_pages = -(-T // P)
+    pool = torch.zeros(n_pages, 2, 1, P, hd, dtype=torch.bfloat16)
+    vt = pool[:, 1].reshape(n_pages, 1, hd, P)
+    for t in range(T):
+        pool[t // P, 0, 0, t % P] = k[t, 0]
+        vt[t // P, 0, :, t % P] = v[t, 0]
+    table = torch.arange(n_pages, dtype=torch.int32)[None, :].repeat(2, 1).contiguous()
+    for entries in ([(1, T - 1)], [(100, T - 100)]):
+        n = entries[0][0]
+        q = torch.zeros(n, hd, dtype=torch.bfloat16)
+        q[-1, 3] = 30.0
+        out = torch.zeros(n, hd, dtype=torch.bfloat16, device="cuda")
+        ctx = FakeCtx(entries)
+        assert attention_bf16.run(ops, ctx, View(dev(table)), dev(q), dev(pool), out, 1, 1, hd, 1.0 / 8, None)
+        assert (f64(out[-1]) - f64(v[far, 0])).abs().max() < 2e-2

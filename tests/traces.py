@@ -98,6 +98,19 @@ def max_tokens(trace) -> int:
     return worst
 
 
+def max_pages(trace, page_size: int) -> int:
+    """The fewest pages that hold the trace: the most pages live requests need at any time."""
+    held: Dict[str, int] = {}
+    worst = 0
+    for step in trace:
+        for rid, toks, _ in step["entries"]:
+            held[rid] = held.get(rid, 0) + len(toks)
+        worst = max(worst, sum(-(-n // page_size) for n in held.values()))
+        for rid in step["end"]:
+            held.pop(rid, None)
+    return worst
+
+
 def to_jsonl(trace) -> str:
     import json
     lines = []

@@ -1,6 +1,10 @@
 """The device tensors behind the cache manager: one pool of pages per paged
-group, laid out `[cache layer][page][K|V][kv head][row in page][head_dim]`, and
-one block of state per state group, `[cache layer][slot][...]`.
+group, `[cache layer][page][K|V][kv head][...]`, and one block of state per
+state group, `[cache layer][slot][...]`.  Within a page the keys of a kv head lie
+`[row in page][head_dim]` (a score sums over head_dim) and the values transposed,
+`[head_dim][row in page]` (the mix sums over rows): each is contiguous along the
+dimension the matrix cores reduce over.  The tensor's nominal shape is
+`[..., P, head_dim]` for both halves.
 
 A page id addresses the same slot in every cache layer of its group.  At
 Qwen3-0.6B sizes (8 kv heads x 128, 16 rows) a page is 64 KiB per layer in

@@ -45,7 +45,7 @@ attention_rows_kernel(const T* __restrict__ q, const T* __restrict__ pool, const
     const int page = tab[p / P];
     if (page < 0) continue;   // never happens for a reserved request; never read astray
     const T* kp = pool + (size_t)page * page_elems + k_off + (size_t)(p % P) * HD;
-    const T* vp = pool + (size_t)page * page_elems + v_off + (size_t)(p % P) * HD;
+    const T* vp = pool + (size_t)page * page_elems + v_off + (p % P);   // values lie transposed: [d][row]
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < DPL; ++i) s = fmaf(qv[i], ld<T>(kp + lane + i * AG_LANES), s);
@@ -55,7 +55,7 @@ attention_rows_kernel(const T* __restrict__ q, const T* __restrict__ pool, const
     const float w = expf(s - m_new);
     l = l * alpha + w;
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) o[i] = o[i] * alpha + w * ld<T>(vp + lane + i * AG_LANES);
+    for (int i = 0; i < DPL; ++i) o[i] = o[i] * alpha + w * ld<T>(vp + (size_t)(lane + i * AG_LANES) * P);
     mx = m_new;
   }
 #pragma unroll
@@ -101,7 +101,8 @@ static int launch_rows(int dpl, dim3 grid, const void* q, const void* pool, cons
   return 0;
 }
 
-// q, out: [M, n_head, hd] in T; pool: [pages][2][n_kv][P][hd] in T; table: [slots][table_stride];
+// q, out: [M, n_head, hd] in T; pool: [pages][K: [n_kv][P][hd] | V: [n_kv][hd][P]] in T;
+// table: [slots][table_stride];
 // pos, slot: [M].  window <= 0: all keys up to the row's own position.
 extern "C" int ti_attention_rows(int dtype, const void* q, const void* pool, const int* table, int table_stride,
                                  const int* pos, const int* slot, void* out, int M, int n_head, int n_kv,

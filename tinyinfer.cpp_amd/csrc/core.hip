@@ -102,8 +102,11 @@ extern "C" int ti_rope_neox(float* x, const int* pos, const float* inv_freq, int
 // One workgroup per token; each wave takes whole heads in turn.  For q heads and
 // k heads: RMS-norm over head_dim (if a weight is given), then the half-split
 // rotation (if inv_freq is given).  q goes to q_out (T), k and v into the cache
-// page of the token's position:
-//   pool[page][0 = K | 1 = V][kv head][pos % P][:] with page = table[slot][pos / P].
+// page of the token's position, page = table[slot][pos / P]:
+//   keys   pool[page][0][kv head][pos % P][d]   (a key's dims are contiguous: the
+//                                                 score sums over d)
+//   values pool[page][1][kv head][d][pos % P]   (transposed: the mix sums over
+//                                                 positions, so these are contiguous)
 // v is copied unchanged.  n_kv == 0: only q is handled (the layer reads another
 // layer's keys and values).
 template <typename T>
@@ -139,10 +142,10 @@ __global__ void qk_norm_rope_kv_write_kernel(
     } else {
       if (!page_ok) continue;   // the host reserves pages first; never write astray
       const int kvh = is_v ? u - n_head - n_kv : u - n_head;
-      dst = pool + page_base + ((size_t)(is_v ? 1 : 0) * n_kv + kvh) * P * hd + (size_t)prow * hd;
+      dst = pool + page_base + ((size_t)(is_v ? 1 : 0) * n_kv + kvh) * P * hd + (is_v ? (size_t)prow : (size_t)prow * hd);
     }
     if (is_v) {
-      for (int i = lane; i < hd; i += TI_WAVE) st<T>(dst + i, src[i]);
+      for (int i = lane; i < hd; i += TI_WAVE) st<T>(dst + (size_t)i * P, src[i]);
       continue;
     }
     const float* w = is_q ? q_w : k_w;

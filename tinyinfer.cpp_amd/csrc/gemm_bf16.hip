@@ -1,0 +1,315 @@
+// bfloat16 matrix products C = A W^T on the matrix cores of gfx950, 32-bit
+// accumulation.  A is [M, K] (row stride lda), W is [N, K], both bfloat16 with K
+// contiguous, which is the natural operand layout of MFMA for both sides.
+//
+// Two kernels:
+//  * skinny (M <= 64, decode and small portions): every weight element is read
+//    from memory exactly once per call.  A workgroup of four wavefronts owns 16
+//    weight rows; the wavefronts split K between them in interleaved 128-byte
+//    pieces and reduce through LDS in a fixed order.  The weights are the "A"
+//    operand of v_mfma_f32_16x16x32_bf16, the tokens are the 16 columns.
+//  * tiled (M > 64, prefill): 128 x 128 x 32 tiles through double-buffered LDS,
+//    four wavefronts in 2 x 2, each 64 x 64 out of v_mfma_f32_32x32x16_bf16.
+//
+// Epilogues: store float, add into a float residual, store bfloat16, or SwiGLU
+// over a stacked [gate; up] weight.  The reduction order of an output element
+// never depends on M within one kernel.  (The reference's two products are
+// /root/reference/src/cuda/gemm.cu:37-85 and 152-261; it reads the weights once
+// per row of A for M <= 32.)
+#include "common.h"
+
+TI_ERROR_API
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+
+union Frag {
+  uint4 u;
+  bf16x8 v;
+};
+
+__device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
+
+// ============================================================== skinny kernel
+// grid.x = ceil(N / 16) (SwiGLU: ceil(F / 8): 8 gate rows and their 8 up rows)
+template <int MT, int EPI>
+__global__ void __launch_bounds__(256)
+gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_,
+                   int M, int N, int K, long lda) {
+  constexpr bool SW = (EPI == TI_EPI_SWIGLU);
+  __shared__ float red[4][MT][16][17];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 15, j = lane >> 4;   // MFMA row / column, and k group
+  const int rows_total = SW ? 2 * N : N;
+  // the weight row this lane feeds
+  int wrow;
+  if (SW) {
+    const int n = blockIdx.x * 8 + (r & 7);
+    wrow = (r < 8 ? 0 : N) + (n < N ? n : N - 1);
+  } else {
+    const int n = blockIdx.x * 16 + r;
+    wrow = n < N ? n : N - 1;
+  }
+  (void)rows_total;
+  const bf16_t* wp = W + (size_t)wrow * K + j * 16;
+  const bf16_t* ap[MT];
+  bool aok[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + r;
+    aok[t] = m < M;
+    ap[t] = A + (size_t)(aok[t] ? m : 0) * lda + j * 16;
+  }
+  floatx4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  // chunk c covers k in [64 c, 64 c + 64); lane group j takes [64 c + 16 j, +16)
+  const int chunks = (K + 63) / 64;
+  constexpr int UN = 4;
+  for (int c0 = wave; c0 < chunks; c0 += 4 * UN) {
+    Frag w0[UN], w1[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int k = (c0 + 4 * u) * 64 + j * 16;
+      w0[u].u = (k + 8 <= K) ? ld16(wp + (size_t)(c0 + 4 * u) * 64) : zero;
+      w1[u].u = (k + 16 <= K) ? ld16(wp + (size_t)(c0 + 4 * u) * 64 + 8) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int k = (c0 + 4 * u) * 64 + j * 16;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        Frag a0, a1;
+        a0.u = (aok[t] && k + 8 <= K) ? ld16(ap[t] + (size_t)(c0 + 4 * u) * 64) : zero;
+        a1.u = (aok[t] && k + 16 <= K) ? ld16(ap[t] + (size_t)(c0 + 4 * u) * 64 + 8) : zero;
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u].v, a0.v, acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, a1.v, acc[t], 0, 0, 0);
+      }
+    }
+  }
+  // acc[t][i]: weight row 4 j + i, token 16 t + r
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][t][r][4 * j + i] = acc[t][i];
+  __syncthreads();
+  // thread -> (token = tid / 16, row = tid % 16): consecutive threads, consecutive columns
+  const int tok = threadIdx.x >> 4, row = threadIdx.x & 15;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + tok;
+    if (m >= M) continue;
+    if (SW) {
+      if (row >= 8) continue;
+      const int n = blockIdx.x * 8 + row;
+      if (n >= N) continue;
+      float g = 0.f, u = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        g += red[w][t][tok][row];
+        u += red[w][t][tok][row + 8];
+      }
+      ((bf16_t*)out_)[(size_t)m * N + n] = f2bf(silu_mul(g, u));
+    } else {
+      const int n = blockIdx.x * 16 + row;
+      if (n >= N) continue;
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) s += red[w][t][tok][row];
+      const size_t o = (size_t)m * N + n;
+      if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = s;
+      if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] += s;
+      if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(s);
+    }
+  }
+}
+
+// =============================================================== tiled kernel
+#define TBM 128
+#define TBN 128
+#define TBK 32
+#define TLD (TBK + 8)   // LDS row stride in bfloat16: 80 bytes, keeps 16-byte reads off the same banks
+#define TPIECES (TBM * TBK / 8 / 256)   // 16-byte pieces per thread and operand tile
+#define TKP (TBK / 8)                   // pieces per row
+
+// SwiGLU: the workgroup covers 64 output columns; LDS row b of the weight tile is
+// global row (b & 32 ? F : 0) + n0 + (b >> 6) * 32 + (b & 31), so that in every
+// wavefront MFMA tile 0 holds gate columns and tile 1 the matching up columns.
+template <int EPI>
+__global__ void __launch_bounds__(256)
+gemm_tiled_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_,
+                  int M, int N, int K, long lda) {
+  constexpr bool SW = (EPI == TI_EPI_SWIGLU);
+  __shared__ __attribute__((aligned(16))) bf16_t sA[2][TBM * TLD];
+  __shared__ __attribute__((aligned(16))) bf16_t sB[2][TBN * TLD];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * TBM;
+  const int n0 = blockIdx.x * (SW ? TBN / 2 : TBN);
+  const int w_rows = SW ? 2 * N : N;
+
+  // global -> LDS in pieces of 16 bytes, TPIECES per thread and operand tile
+  constexpr int RSTEP = 256 / TKP;   // rows covered by one round of the workgroup
+  const int lrow = tid / TKP, lkc = (tid % TKP) * 8;
+  const bf16_t* gA[TPIECES];
+  const bf16_t* gB[TPIECES];
+  bool okA[TPIECES], okB[TPIECES];
+#pragma unroll
+  for (int i = 0; i < TPIECES; ++i) {
+    const int row = lrow + RSTEP * i;
+    const int am = m0 + row;
+    okA[i] = am < M;
+    gA[i] = A + (size_t)(okA[i] ? am : 0) * lda + lkc;
+    int wr;
+    if (SW) {
+      const int n = n0 + (row >> 6) * 32 + (row & 31);
+      okB[i] = n < N;
+      wr = ((row & 32) ? N : 0) + (okB[i] ? n : 0);
+    } else {
+      wr = n0 + row;
+      okB[i] = wr < N;
+      if (!okB[i]) wr = 0;
+    }
+    (void)w_rows;
+    gB[i] = W + (size_t)wr * K + lkc;
+  }
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  uint4 ra[TPIECES], rb[TPIECES];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < TPIECES; ++i) {
+      const bool kin = k0 + lkc + 8 <= K;
+      ra[i] = (okA[i] && kin) ? ld16(gA[i] + k0) : zero;
+      rb[i] = (okB[i] && kin) ? ld16(gB[i] + k0) : zero;
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TPIECES; ++i) {
+      *reinterpret_cast<uint4*>(&sA[buf][(lrow + RSTEP * i) * TLD + lkc]) = ra[i];
+      *reinterpret_cast<uint4*>(&sB[buf][(lrow + RSTEP * i) * TLD + lkc]) = rb[i];
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+
+  const int fr = lane & 31, fk = (lane >> 5) * 8;
+  const int n_k = (K + TBK - 1) / TBK;
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  for (int kt = 0; kt < n_k; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < n_k) fetch((kt + 1) * TBK);
+#pragma unroll
+    for (int ks = 0; ks < TBK; ks += 16) {
+      Frag fa[2], fb[2];
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+        fa[a].u = *reinterpret_cast<const uint4*>(&sA[buf][(wm * 64 + a * 32 + fr) * TLD + ks + fk]);
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+        fb[b].u = *reinterpret_cast<const uint4*>(&sB[buf][(wn * 64 + b * 32 + fr) * TLD + ks + fk]);
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a].v, fb[b].v, acc[a][b], 0, 0, 0);
+    }
+    if (kt + 1 < n_k) stash(buf ^ 1);
+    __syncthreads();
+  }
+
+  // acc[a][b][i]: row wm*64 + a*32 + 8*(i/4) + 4*(lane/32) + i%4, column wn*64 + b*32 + lane%32
+  const int ccol = lane & 31, crow = (lane >> 5) * 4;
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int m = m0 + wm * 64 + a * 32 + (i >> 2) * 8 + crow + (i & 3);
+      if (m >= M) continue;
+      if (SW) {
+        const int n = n0 + wn * 32 + ccol;
+        if (n < N) ((bf16_t*)out_)[(size_t)m * N + n] = f2bf(silu_mul(acc[a][0][i], acc[a][1][i]));
+      } else {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const int n = n0 + wn * 64 + b * 32 + ccol;
+          if (n >= N) continue;
+          const size_t o = (size_t)m * N + n;
+          const float s = acc[a][b][i];
+          if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = s;
+          if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] += s;
+          if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(s);
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------- dispatch
+template <int EPI>
+static void launch_skinny(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
+                          hipStream_t s) {
+  const int grid = (EPI == TI_EPI_SWIGLU) ? (N + 7) / 8 : (N + 15) / 16;
+  const int mt = (M + 15) / 16;
+  if (mt == 1) gemm_skinny_kernel<1, EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
+  if (mt == 2) gemm_skinny_kernel<2, EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
+  if (mt == 3) gemm_skinny_kernel<3, EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
+  if (mt == 4) gemm_skinny_kernel<4, EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
+}
+
+template <int EPI>
+static void launch_tiled(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
+                         hipStream_t s) {
+  const int bn = (EPI == TI_EPI_SWIGLU) ? TBN / 2 : TBN;
+  dim3 grid((N + bn - 1) / bn, (M + TBM - 1) / TBM);
+  gemm_tiled_kernel<EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
+}
+
+// N: output columns (SwiGLU: F, with W holding 2F rows).  Returns 3 for a shape
+// these kernels do not serve (the caller takes the generic kernel then).
+extern "C" int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
+                            hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K, "gemm_bf16: bad sizes M=%d N=%d K=%d lda=%ld", M, N, K, lda);
+  if (K % 8 != 0 || lda % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) {
+    ti_set_error("gemm_bf16: K=%d / lda=%ld not multiples of 8 or operands not 16-byte aligned", K, lda);
+    return 3;
+  }
+  if ((M + TBM - 1) / TBM > 65535) {
+    ti_set_error("gemm_bf16: M=%d too large for one launch", M);
+    return 3;
+  }
+  if (M == 0) return 0;
+  const bf16_t* a = (const bf16_t*)A;
+  const bf16_t* w = (const bf16_t*)W;
+  const bool skinny = M <= 64;
+#define TI_GO(E)                                                  \
+  case E:                                                         \
+    if (skinny)                                                   \
+      launch_skinny<E>(a, w, out, M, N, K, lda, stream);          \
+    else                                                          \
+      launch_tiled<E>(a, w, out, M, N, K, lda, stream);           \
+    break;
+  switch (epi) {
+    TI_GO(TI_EPI_STORE_F32)
+    TI_GO(TI_EPI_ADD_F32)
+    TI_GO(TI_EPI_STORE_ACT)
+    TI_GO(TI_EPI_SWIGLU)
+    default:
+      TI_REQUIRE(false, "gemm_bf16: unknown epilogue %d", epi);
+  }
+#undef TI_GO
+  TI_LAUNCH_CHECK();
+  return 0;
+}

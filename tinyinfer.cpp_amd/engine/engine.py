@@ -68,7 +68,10 @@ class StepContext:
         self.tiles = None                 # int32 [n_tiles, 2]: (entry, first row) of each query tile
         self.n_tiles = 0
         self.decode_only = False
+        self.decode_rows = None           # int32: rows of single-token entries (None if decode_only)
+        self.n_decode_rows = 0
         self.max_context = 0              # longest context (tokens) any row reads in this step
+        self.split_context = 0            # the context length the decode kernel's split count is sized for
         self.run = 0                      # index into the model's run order
         self._views: Dict[int, CacheView] = {}
 
@@ -246,6 +249,7 @@ class Engine:
         paged = cache.paged_groups()
         W = self.table_width
         tiles: List[Tuple[int, int]] = []
+        dec_rows: List[int] = []
         row0 = 0
         for i, e in enumerate(entries):
             n = len(e.tokens)
@@ -255,16 +259,23 @@ class Engine:
             if n > 1:
                 for q0 in range(0, n, PREFILL_TILE_Q):
                     tiles.append((i, row0 + q0))
+            else:
+                dec_rows.append(row0)
             row0 += n
-        ctx.decode_only = all(n == 1 for _, n, _, _ in ctx.entries)
+        ctx.decode_only = not tiles
+        if ctx.decode_only:
+            dec_rows = []
         ctx.n_tiles = len(tiles)
+        ctx.n_decode_rows = len(dec_rows)
+        ctx.split_context = ctx.max_context
 
-        # layout: tokens | positions | slots | out_rows | entries [R,4] | tiles [n_tiles,2] | tables
+        # layout: tokens | positions | slots | out_rows | entries [R,4] | tiles [n_tiles,2] | decode rows | tables
         o_tok, o_pos, o_slot = 0, M, 2 * M
         o_out = 3 * M
         o_ent = o_out + n_want
         o_tile = o_ent + 4 * R
-        o_tab = o_tile + 2 * len(tiles)
+        o_dec = o_tile + 2 * len(tiles)
+        o_tab = o_dec + len(dec_rows)
         total = o_tab + len(paged) * R * W
         turn, host, dev = self._meta_buffers(total)
         h = host.numpy()
@@ -280,6 +291,8 @@ class Engine:
         for j, (ei, q0) in enumerate(tiles):
             h[o_tile + 2 * j] = ei
             h[o_tile + 2 * j + 1] = q0
+        if dec_rows:
+            h[o_dec:o_dec + len(dec_rows)] = dec_rows
         for k, (gi, g) in enumerate(paged):
             base = o_tab + k * R * W
             h[base:base + R * W] = -1
@@ -297,6 +310,7 @@ class Engine:
         ctx.out_rows = dev[o_out:o_out + n_want] if n_want else None
         ctx.entry_meta = dev[o_ent:o_ent + 4 * R].view(R, 4)
         ctx.tiles = dev[o_tile:o_tile + 2 * len(tiles)].view(-1, 2) if tiles else None
+        ctx.decode_rows = dev[o_dec:o_dec + len(dec_rows)] if dec_rows else None
         for k, (gi, g) in enumerate(paged):
             base = o_tab + k * R * W
             ctx._views[gi] = CacheView(dev[base:base + R * W].view(R, W), self.page_size)

@@ -1,0 +1,61 @@
+"""How a step's rows are handed to the bfloat16 matrix-core attention kernels:
+rows of single-token entries go to the flash-decoding kernel (split over the
+context so that the launch fills the chip), rows of longer entries to the tiled
+prefill kernel.  Head sizes or page sizes the kernels do not serve are left to
+the generic kernel (`run` returns False)."""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+SERVED_HEAD_DIMS = (32, 64, 128)
+TARGET_WORKGROUPS = 1024      # a few per compute unit (256 of them)
+MAX_SPLITS = 64
+MIN_BLOCKS_PER_SPLIT = 4      # one 16-key block per wavefront at least
+
+
+def decode_splits(n_rows: int, kv_heads: int, heads: int, context: int) -> int:
+    parts = (heads // kv_heads + 15) // 16
+    base = max(1, n_rows * kv_heads * parts)
+    want = -(-TARGET_WORKGROUPS // base)
+    blocks = -(-max(1, context) // 16)
+    return max(1, min(want, blocks // MIN_BLOCKS_PER_SPLIT, MAX_SPLITS))
+
+
+def _ptr(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) -> bool:
+    P = pool.shape[3]
+    if head_dim not in SERVED_HEAD_DIMS or P % 16 != 0:
+        return False
+    lib = ops.lib("attention_bf16")
+    stream = ops._stream()
+    table = view.table
+    win = int(window or 0)
+    n_dec = ctx.M if ctx.decode_only else ctx.n_decode_rows
+    if n_dec:
+        rows = None if ctx.decode_only else ctx.decode_rows
+        context = ctx.split_context if win == 0 else min(ctx.split_context, win + 16)
+        S = decode_splits(n_dec, kv_heads, heads, context)
+        part_o = part_ml = None
+        if S > 1:
+            part_o = ctx.buf("attn.part_o", (n_dec, heads, S, head_dim), torch.float32)
+            part_ml = ctx.buf("attn.part_ml", (n_dec, heads, S, 2), torch.float32)
+        rc = lib.ti_attention_decode_bf16(
+            _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.positions), _ptr(ctx.slots), _ptr(rows),
+            _ptr(out), _ptr(part_o), _ptr(part_ml), n_dec, heads, kv_heads, head_dim, P, ctypes.c_float(scale),
+            win, S, stream)
+        if rc == 3:
+            return False
+        ops._check(lib, rc, "attention(decode)")
+    if ctx.n_tiles:
+        rc = lib.ti_attention_prefill_bf16(
+            _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.tiles), _ptr(ctx.entry_meta), _ptr(out),
+            ctx.n_tiles, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, stream)
+        if rc == 3:
+            return False
+        ops._check(lib, rc, "attention(prefill)")
+    return True
