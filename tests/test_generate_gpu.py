@@ -1,0 +1,159 @@
+"""Generation through the entry points: scheduler, step function, device sampler,
+decode graphs, preemption, command line."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import CONFIGS, random_tokens, read_folder
+from plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def plain_generate(cfg, w, prompt, n, number=0, temperature=0.0, top_k=0, top_p=1.0, seed=42):
+    from tinyinfer_amd.sampling import uniform, DEFAULT_TOP_K
+    toks = list(prompt)
+    out = []
+    for i in range(n):
+        logits = plain.forward(w, cfg, toks)[-1]
+        if temperature <= 0:
+            t = plain.argmax_lowest(logits)
+        else:
+            p = plain.sample_distribution(logits, temperature, top_k or DEFAULT_TOP_K, top_p)
+            t = plain.draw(p, uniform(seed, number, i))
+        toks.append(t)
+        out.append(t)
+    return out
+
+
+def test_config_a_greedy_eight_tokens(model_folders):
+    """One request, an 8-token prompt, greedy decoding of 8 tokens, in 32-bit."""
+    import tinyinfer_amd as ti
+    d = model_folders("A", "float32")
+    cfg, w = read_folder(d)
+    prompt = random_tokens(8, 256, 0)
+    llm = ti.LLM(d, dtype="float32", max_seq=64, max_requests=1)
+    got = llm.generate([prompt], max_new_tokens=8)[0]
+    assert got == plain_generate(cfg, w, prompt, 8)
+
+
+def test_config_b_mixed_batch_with_temperature(model_folders):
+    """Three requests with prompts of 5, 17 and 33 tokens, prefilled in portions of
+    7 beside decoding requests, pages of 4 tokens, temperature 0.8, a fixed seed, 6
+    tokens each, in 32-bit."""
+    import tinyinfer_amd as ti
+    d = model_folders("B", "float32")
+    cfg, w = read_folder(d)
+    prompts = [random_tokens(n, 1000, 10 + n) for n in (5, 17, 33)]
+    engine = ti.Engine.from_folder(d, "float32", page_size=4, max_tokens=192, max_requests=3, max_seq=64)
+    stats = ti.GenerationStats()
+    got = ti.generate_ids(engine, prompts, max_new_tokens=6, temperature=0.8, seed=123, chunk_size=7,
+                          max_batched_tokens=12, stats=stats)
+    want = [plain_generate(cfg, w, p, 6, number=i, temperature=0.8, seed=123) for i, p in enumerate(prompts)]
+    assert got == want
+    # every prompt token and all but the last generated token of each request was fed once
+    assert stats.prefill_tokens + stats.decode_tokens == 55 + 3 * 5 and stats.steps > 6
+    # what a request draws does not depend on its company: alone it gets the same tokens
+    engine2 = ti.Engine.from_folder(d, "float32", page_size=16, max_tokens=64, max_requests=1, max_seq=64)
+    sched = ti.Scheduler(engine2.cache)
+    for i, p in enumerate(prompts):
+        sched._submitted = i
+        r = sched.add(p, 6, ti.SamplingParams(0.8, 0, 1.0, 123))
+        from tinyinfer_amd.api import run_requests
+        run_requests(engine2, sched)
+        assert r.generated == want[i]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_with_graphs_equals_eager(model_folders, dtype):
+    """Decode steps replayed from captured graphs give the same logits bit for bit
+    as eager steps, replay after replay, with eager steps in between (the
+    reference checks the same: /root/reference/src/inference.cu:297-341)."""
+    import tinyinfer_amd as ti
+    d = model_folders("D", "bfloat16", True)
+    prompts = [random_tokens(n, 333, 40 + n) for n in (21, 3, 50)]
+    outs = {}
+    for graph in (False, True):
+        engine = ti.Engine.from_folder(d, dtype, page_size=16, max_tokens=384, max_requests=3, max_seq=128)
+        outs[graph] = ti.generate_ids(engine, prompts, max_new_tokens=40, use_graph=graph, chunk_size=16,
+                                      max_batched_tokens=24)
+        if graph:
+            assert engine._graphs, "no graph was captured"
+    assert outs[True] == outs[False]
+    # logits bit for bit, several replays, eager work between them
+    e1 = ti.Engine.from_folder(d, dtype, page_size=16, max_tokens=256, max_requests=2, max_seq=128)
+    e2 = ti.Engine.from_folder(d, dtype, page_size=16, max_tokens=256, max_requests=2, max_seq=128)
+    toks = {"x": random_tokens(70, 333, 1), "y": random_tokens(70, 333, 2)}
+    for e in (e1, e2):
+        e.step([ti.StepEntry("x", toks["x"][:30], [29]), ti.StepEntry("y", toks["y"][:9], [8])])
+    fed = {"x": 30, "y": 9}
+    for i in range(30):
+        entries = [ti.StepEntry(r, [toks[r][fed[r]]], [0]) for r in ("x", "y")]
+        a = e1.step(entries).clone()
+        if i % 7 == 3:                         # an eager step through the graph engine as well
+            b = e2.step(entries).clone()
+        else:
+            b = e2.step_graph(entries).clone()
+        assert torch.equal(a, b), i
+        for r in fed:
+            fed[r] += 1
+
+
+def test_preemption_recomputes_and_changes_nothing(model_folders):
+    """With too few pages the youngest request gives way and is fed again later;
+    in 32-bit the tokens are the ones a roomy pool gives."""
+    import tinyinfer_amd as ti
+    d = model_folders("B", "bfloat16", True)
+    prompts = [random_tokens(n, 1000, 70 + n) for n in (12, 12, 9)]
+    roomy = ti.Engine.from_folder(d, "float32", page_size=4, max_tokens=256, max_requests=3, max_seq=48)
+    want = ti.generate_ids(roomy, prompts, max_new_tokens=20, temperature=0.7, seed=5)
+    tight = ti.Engine.from_folder(d, "float32", page_size=4, max_tokens=64, max_requests=3, max_seq=48)
+    stats = ti.GenerationStats()
+    got = ti.generate_ids(tight, prompts, max_new_tokens=20, temperature=0.7, seed=5, stats=stats)
+    assert stats.preemptions > 0
+    assert got == want
+    assert not tight.cache.live_requests()
+    tight.cache.check()
+
+
+def test_eos_and_length(model_folders):
+    import tinyinfer_amd as ti
+    d = model_folders("A", "float32")
+    prompt = random_tokens(6, 256, 3)
+    engine = ti.Engine.from_folder(d, "float32", max_tokens=64, max_requests=1)
+    full = ti.generate_ids(engine, [prompt], max_new_tokens=10)[0]
+    assert len(full) == 10
+    cut = ti.generate_ids(engine, [prompt], max_new_tokens=10, eos_token_ids=[full[4]])[0]
+    assert cut == full[:full.index(full[4])]              # the end token itself is not emitted
+
+
+def test_command_line(model_folders, tmp_path):
+    d = model_folders("A", "float32")
+    cfg, w = read_folder(d)
+    p1, p2 = random_tokens(5, 256, 1), random_tokens(9, 256, 2)
+    f = tmp_path / "prompts.txt"
+    f.write_text(" ".join(map(str, p2)) + "\r\n\n")
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "tinyinfer"), "-m", d, "-n", "5",
+                          "-p", ",".join(map(str, p1)), "-f", str(f), "--dtype", "float32", "--max-seq", "64"],
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    lines = run.stdout.strip().split("\n")
+    assert lines[0] == "==================== prompt 0 ===================="
+    assert lines[1] == "[prompt] " + ",".join(map(str, p1))
+    assert lines[2] == "[output] " + " ".join(map(str, plain_generate(cfg, w, p1, 5)))
+    assert lines[5] == "[output] " + " ".join(map(str, plain_generate(cfg, w, p2, 5)))
+    assert "main: prefill:" in run.stderr and "tok/s" in run.stderr
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "tinyinfer"), "-m", d, "--nonsense"],
+                         capture_output=True, text=True, timeout=120)
+    assert bad.returncode == 1 and "usage:" in bad.stderr
+
+
+def test_smoke_entry():
+    sys.path.insert(0, ROOT)
+    import __graft_entry__
+    __graft_entry__.smoke()

@@ -8,7 +8,12 @@ from .parts.registry import register_part, build_part
 from . import parts as _parts          # noqa: F401  registers the built-in parts
 from . import models as _models        # noqa: F401  registers the built-in architecture
 from .models import Model, ModelSpec, LayerSpec, PartSpec
+from .engine import Engine, StepEntry
+from .engine.scheduler import Scheduler, Request
+from .sampling import SamplingParams
+from .api import LLM, generate_ids, GenerationStats
 
 __all__ = ["ConfigError", "read_config_json", "Qwen3Config", "register_architecture",
            "registered_architectures", "config_and_spec", "register_part", "build_part",
-           "Model", "ModelSpec", "LayerSpec", "PartSpec"]
+           "Model", "ModelSpec", "LayerSpec", "PartSpec", "Engine", "StepEntry", "Scheduler", "Request",
+           "SamplingParams", "LLM", "generate_ids", "GenerationStats"]

@@ -125,6 +125,7 @@ class Engine:
         self._meta_events: List[Optional[torch.cuda.Event]] = []
         self._meta_turn = 0
         self.steps_run = 0
+        self._graphs: Dict[int, "_DecodeGraph"] = {}
 
     # ------------------------------------------------------------- construction
     @classmethod
@@ -169,8 +170,11 @@ class Engine:
             self._ws[key] = t
         return t[:n].view(*shape)
 
-    def _meta_buffers(self, n_ints: int):
-        """A pinned host buffer (two take turns) and the device buffer, both >= n_ints."""
+    def _meta_buffers(self, n_ints: int, dev_fixed: Optional[torch.Tensor] = None):
+        """A pinned host buffer (two take turns) and the device buffer, both >= n_ints.
+        `dev_fixed`: use this device buffer (a captured graph reads its address)."""
+        if dev_fixed is not None and dev_fixed.numel() < n_ints:
+            raise EngineError("the fixed metadata buffer is too small for this step")
         if self._meta_dev is None or self._meta_dev.numel() < n_ints:
             cap = max(4096, int(n_ints * 1.5))
             self._meta_dev = torch.empty(cap, dtype=torch.int32, device=self.device)
@@ -181,7 +185,7 @@ class Engine:
         ev = self._meta_events[i]
         if ev is not None:
             ev.synchronize()          # the copy that last read this buffer has finished
-        return i, self._meta_host[i], self._meta_dev
+        return i, self._meta_host[i], (self._meta_dev if dev_fixed is None else dev_fixed)
 
     # --------------------------------------------------------------------- step
     def release(self, request: Hashable) -> None:
@@ -197,7 +201,7 @@ class Engine:
         self.finish(ctx)
         return logits
 
-    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
+    def prepare(self, entries: Sequence[StepEntry], meta_dev: Optional[torch.Tensor] = None) -> StepContext:
         """Check the batch, reserve pages, build and upload the step's metadata."""
         if not entries:
             raise EngineError("a step needs at least one entry")
@@ -277,7 +281,7 @@ class Engine:
         o_dec = o_tile + 2 * len(tiles)
         o_tab = o_dec + len(dec_rows)
         total = o_tab + len(paged) * R * W
-        turn, host, dev = self._meta_buffers(total)
+        turn, host, dev = self._meta_buffers(total, meta_dev)
         h = host.numpy()
         out_i = o_out
         for i, (e, (r0, n, start, sslot)) in enumerate(zip(entries, ctx.entries)):
@@ -335,6 +339,73 @@ class Engine:
         for e in ctx._entries_in:
             self.cache.commit(e.request, len(e.tokens))
         self.steps_run += 1
+
+    # ------------------------------------------------------------ decode graphs
+    def step_graph(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """`step` for a batch of single tokens that each want their logits, replayed
+        from a HIP graph captured once per batch size (the reference keys its CUDA
+        graphs the same way: /root/reference/src/inference.cu:267-295).  Anything
+        else runs through `step`.
+
+        What a replay reads is at fixed addresses: the graph has its own metadata
+        buffer (tokens, positions, block-table rows: refreshed by one copy before
+        each replay) and its own workspace; loop bounds are read on the device,
+        and the number of context splits is sized for `max_seq`, not for the
+        step.  Sampling stays outside the graph."""
+        if not all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries):
+            return self.step(entries)
+        R = len(entries)
+        rec = self._graphs.get(R)
+        if rec is None:
+            return self._capture(entries)
+        saved = self._ws
+        self._ws = rec.workspace
+        try:
+            ctx = self.prepare(entries, meta_dev=rec.meta)
+        finally:
+            self._ws = saved
+        rec.graph.replay()
+        self.finish(ctx)
+        return rec.logits
+
+    def _capture(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        R = len(entries)
+        paged = len(self.cache.paged_groups())
+        rec = _DecodeGraph()
+        rec.meta = torch.empty(8 * R + paged * R * self.table_width + 64, dtype=torch.int32, device=self.device)
+        saved = self._ws
+        self._ws = rec.workspace
+        try:
+            ctx = self.prepare(entries, meta_dev=rec.meta)
+            ctx.split_context = self.max_seq
+            # a first run outside the graph: it computes this step's result and makes every
+            # workspace buffer the graph will use
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                self.run(ctx)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            rec.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(rec.graph):
+                rec.logits = self.run(ctx)
+        finally:
+            self._ws = saved
+        # capture records, it does not run: the first run above already wrote this step's
+        # keys, values and logits, and a replay would write the same again
+        self.finish(ctx)
+        self._graphs[R] = rec
+        return rec.logits
+
+
+class _DecodeGraph:
+    """A captured decode step for one batch size, with the buffers it reads and writes."""
+
+    def __init__(self):
+        self.graph = None
+        self.meta: Optional[torch.Tensor] = None
+        self.workspace: Dict[str, torch.Tensor] = {}
+        self.logits: Optional[torch.Tensor] = None
 
 
 def required_libraries(dtype: str):

@@ -1,0 +1,1 @@
+from .sampler import SamplingParams, Sampler, uniform, DEFAULT_TOP_K
