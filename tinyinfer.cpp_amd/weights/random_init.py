@@ -65,3 +65,27 @@ def write_model_folder(path: str, config: Mapping, seed: int, dtype: str = "bflo
     write_safetensors(os.path.join(path, "model.safetensors"), tensors,
                       {"format": "pt", "seed": str(seed)})
     return tensors
+
+
+def main(argv=None) -> int:
+    """python -m tinyinfer_amd.weights.random_init CONFIG.json OUT_DIR [--seed S] [--dtype bfloat16|float32]"""
+    import argparse
+    ap = argparse.ArgumentParser(description="write a model folder (config.json, model.safetensors) with random "
+                                             "weights from a configuration and a seed")
+    ap.add_argument("config", help="a config.json of a registered architecture")
+    ap.add_argument("out", help="folder to write")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16",
+                    help="how matrices are stored (norm weights are stored in float32)")
+    args = ap.parse_args(argv)
+    with open(args.config, "r", encoding="utf-8") as f:
+        config = json.load(f)
+    tensors = write_model_folder(args.out, config, args.seed, args.dtype)
+    n = sum(t.numel() for t in tensors.values())
+    print(f"wrote {args.out}: {len(tensors)} tensors, {n} parameters, seed {args.seed}, matrices in {args.dtype}")
+    return 0
+
+
+if __name__ == "__main__":
+    import sys
+    sys.exit(main())
