@@ -124,8 +124,10 @@ class View:
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("hd,nh,nkv,P", [(48, 3, 3, 4), (128, 4, 2, 16), (16, 6, 2, 8)])
-def test_qk_norm_rope_kv_write(ops, dtype, hd, nh, nkv, P):
+@pytest.mark.parametrize("table_len", [None, 7, 64])
+@pytest.mark.parametrize("hd,nh,nkv,P", [(48, 3, 3, 4), (128, 4, 2, 16), (16, 6, 2, 8), (256, 1, 1, 16)])
+def test_qk_norm_rope_kv_write(ops, dtype, hd, nh, nkv, P, table_len):
+    """With a sin/cos table that covers all, some (positions 0..6) or none of the positions."""
     g = torch.Generator().manual_seed(11)
     M, pages, W = 7, 9, 5
     eps, theta = 1e-5, 3e4
@@ -143,8 +145,10 @@ def test_qk_norm_rope_kv_write(ops, dtype, hd, nh, nkv, P):
     assert need0 <= 3
     pool = torch.zeros(pages, 2, nkv, P, hd, dtype=DT[dtype], device="cuda")
     q_out = torch.empty(M, nh * hd, dtype=DT[dtype], device="cuda")
-    ops.qk_norm_rope_kv_write(dev(qkv), dev(qw), dev(kw), eps, dev(inv_freq(hd, theta)), dev(pos), dev(slot),
-                              View(dev(table)), pool, q_out, nh, nkv, hd)
+    freqs = dev(inv_freq(hd, theta))
+    rope_table = None if table_len is None else ops.rope_table(freqs, table_len)
+    ops.qk_norm_rope_kv_write(dev(qkv), dev(qw), dev(kw), eps, freqs, dev(pos), dev(slot),
+                              View(dev(table)), pool, q_out, nh, nkv, hd, rope_table)
     q = qkv[:, :nh * hd].reshape(M, nh, hd)
     k = qkv[:, nh * hd:(nh + nkv) * hd].reshape(M, nkv, hd)
     v = qkv[:, (nh + nkv) * hd:].reshape(M, nkv, hd)
@@ -401,7 +405,8 @@ def test_sample_frequencies(ops):
 # ------------------------------------------------- bfloat16 matrix-core products
 @pytest.mark.parametrize("M,N,K", [
     (1, 48, 64), (5, 261, 1024), (8, 1000, 96), (16, 17, 200), (17, 130, 72), (33, 64, 3072), (64, 151, 256),
-    (65, 130, 96), (128, 128, 32), (200, 261, 1024), (300, 520, 104), (77, 1000, 1032)])
+    (65, 130, 96), (128, 128, 32), (200, 261, 1024), (300, 520, 104), (77, 1000, 1032),
+    (300, 520, 128), (257, 384, 192), (513, 200, 64), (1000, 1100, 320), (2048, 96, 1024)])
 def test_linear_bf16_matrix_cores(ops, M, N, K):
     """The skinny (M <= 64) and tiled (M > 64) MFMA kernels against float64, every
     epilogue, at sizes that are no multiples of their tiles.  (5, 261, 1024) is the

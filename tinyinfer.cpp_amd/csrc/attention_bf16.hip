@@ -48,75 +48,168 @@ struct PagedKV {
   int kvh;
 };
 
-// One block of 16 keys [key0, key0 + 16) for this wavefront's 16 columns.
+// The fragments of two blocks of 16 keys each, [keyA, keyA + 16) and [keyB, keyB + 16),
+// for the two products.  The pair is what one turn of the walk handles: one softmax
+// update and one rescaling of the output for 32 keys, and the second product as
+// v_mfma_f32_16x16x32_bf16 over both blocks at once.
+template <int HD>
+struct KVPair {
+  Frag8 k[2][HD / 32];   // K:   row lane % 16, dims 32 s + 8 (lane / 16) .. + 7
+  Frag8 v[HD / 16];      // V^T: row (dim) 16 d + lane % 16; elements 0..3: keys 4 (lane / 16) .. + 3 of
+                         //      block A, elements 4..7: the same keys of block B
+};
+
+// Issue the loads of a pair.  They are unconditional (the caller passes pages that
+// exist, whatever they hold) so that the compiler can count them and let the
+// arithmetic of the pair before run while they are in flight.
+template <int HD>
+__device__ __forceinline__ void load_pair(const PagedKV& kv, int pageA, int keyA, int pageB, int keyB,
+                                          KVPair<HD>& f) {
+  const int lane = threadIdx.x & 63;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const size_t page_elems = (size_t)2 * kv.n_kv * kv.P * HD;
+  const size_t k_off = (size_t)kv.kvh * kv.P * HD, v_off = (size_t)(kv.n_kv + kv.kvh) * kv.P * HD;
+  const bf16_t* pa = kv.pool + (size_t)pageA * page_elems;
+  const bf16_t* pb = kv.pool + (size_t)pageB * page_elems;
+  const int rowA = keyA % kv.P, rowB = keyB % kv.P;
+  const bf16_t* ka = pa + k_off + (size_t)(rowA + r16) * HD + quad * 8;
+  const bf16_t* kb = pb + k_off + (size_t)(rowB + r16) * HD + quad * 8;
+  const bf16_t* va = pa + v_off + (size_t)r16 * kv.P + rowA + quad * 4;
+  const bf16_t* vb = pb + v_off + (size_t)r16 * kv.P + rowB + quad * 4;
+#pragma unroll
+  for (int s = 0; s < HD / 32; ++s) {
+    f.k[0][s].u = *reinterpret_cast<const uint4*>(ka + s * 32);
+    f.k[1][s].u = *reinterpret_cast<const uint4*>(kb + s * 32);
+  }
+#pragma unroll
+  for (int d = 0; d < HD / 16; ++d) {
+    const uint2 a = *reinterpret_cast<const uint2*>(va + (size_t)d * 16 * kv.P);
+    const uint2 b = *reinterpret_cast<const uint2*>(vb + (size_t)d * 16 * kv.P);
+    f.v[d].u = make_uint4(a.x, a.y, b.x, b.y);
+  }
+}
+
+// What the walk knows of one block.
+struct BlockInfo {
+  int key0;     // first key
+  bool valid;   // false: the block does not count (a stand-in loaded to keep the loads
+                // unconditional, or a page that was given back)
+  bool check;   // true: some key of it may be hidden from some column, or not written yet
+};
+
+// One pair of blocks for this wavefront's 16 columns.
 //   qf       Q^T fragments: column lane % 16, dims 32 * step + 8 * (lane / 16) .. + 7
 //   lo, hi   the keys this lane's column may see: lo <= key <= hi
 //   kv_last  last position of the request that has been written (rows after it hold rubbish)
-//   check    false if every key of the block is visible to every column and written
 template <int HD>
-__device__ __forceinline__ void attend_block(const PagedKV& kv, const Frag8* qf, int key0, int lo, int hi,
-                                             int kv_last, bool check, float scale, float& m, float& l,
-                                             floatx4* o) {
+__device__ __forceinline__ void attend_pair(KVPair<HD>& f, const Frag8* qf, BlockInfo A, BlockInfo B, int lo,
+                                            int hi, int kv_last, float scale, float& m, float& l, floatx4* o) {
   const int lane = threadIdx.x & 63;
-  const int r16 = lane & 15, quad = lane >> 4;
-  const int page = kv.table[key0 / kv.P];
-  if (page < 0) return;   // given back or never taken: nothing visible lies there
-  const int prow = key0 % kv.P;
-  const size_t page_elems = (size_t)2 * kv.n_kv * kv.P * HD;
-  const bf16_t* kbase = kv.pool + (size_t)page * page_elems + (size_t)kv.kvh * kv.P * HD + (size_t)prow * HD;
-  const bf16_t* vbase = kv.pool + (size_t)page * page_elems + (size_t)(kv.n_kv + kv.kvh) * kv.P * HD + prow;
-
-  // S^T = K . Q^T
-  Frag8 kf[HD / 32];
+  const int quad = lane >> 4;
+  // S^T = K . Q^T, both blocks
+  floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int s = 0; s < HD / 32; ++s)
-    kf[s].u = *reinterpret_cast<const uint4*>(kbase + (size_t)r16 * HD + s * 32 + quad * 8);
-  // the value fragments do not depend on the scores: issue their loads now
-  Frag4 vf[HD / 16];
-#pragma unroll
-  for (int d = 0; d < HD / 16; ++d)
-    vf[d].u = *reinterpret_cast<const uint2*>(vbase + (size_t)(d * 16 + r16) * kv.P + quad * 4);
-  floatx4 sc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int s = 0; s < HD / 32; ++s) sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s].v, qf[s].v, sc, 0, 0, 0);
-
-  // this lane: keys key0 + 4 quad + i of column r16
-  float sv[4];
-  float bm = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int key = key0 + quad * 4 + i;
-    sv[i] = (!check || (key >= lo && key <= hi)) ? sc[i] * scale : -INFINITY;
-    bm = fmaxf(bm, sv[i]);
+  for (int s = 0; s < HD / 32; ++s) {
+    sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[0][s].v, qf[s].v, sa, 0, 0, 0);
+    sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[1][s].v, qf[s].v, sb, 0, 0, 0);
   }
+  // this lane: keys key0 + 4 quad + i of column lane % 16, in each block
+  float sv[8];
+  const bool plain = A.valid && B.valid && !A.check && !B.check;   // the same in every lane
+  if (plain) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sv[i] = sa[i] * scale;
+      sv[4 + i] = sb[i] * scale;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ka = A.key0 + quad * 4 + i, kb = B.key0 + quad * 4 + i;
+      const bool see_a = A.valid && (!A.check || (ka >= lo && ka <= hi));
+      const bool see_b = B.valid && (!B.check || (kb >= lo && kb <= hi));
+      sv[i] = see_a ? sa[i] * scale : -INFINITY;
+      sv[4 + i] = see_b ? sb[i] * scale : -INFINITY;
+      // rows never written may hold anything, NaN included, and 0 * NaN is NaN
+      const bool zero_a = !A.valid || ka > kv_last, zero_b = !B.valid || kb > kv_last;
+      if (zero_a || zero_b) {
+#pragma unroll
+        for (int d = 0; d < HD / 16; ++d) {
+          bf16_t* h = reinterpret_cast<bf16_t*>(&f.v[d].u);
+          if (zero_a) h[i] = 0;
+          if (zero_b) h[4 + i] = 0;
+        }
+      }
+    }
+  }
+  float bm = sv[0];
+#pragma unroll
+  for (int i = 1; i < 8; ++i) bm = fmaxf(bm, sv[i]);
   bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
   bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
   const float m_new = fmaxf(m, bm);
   const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-  const float alpha = __expf(m - m_safe);
-  Frag4 pf;
+  Frag8 pf;
+  bf16_t* ph = reinterpret_cast<bf16_t*>(&pf.u);
   float ps = 0.f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < 8; ++i) {
     const float p = __expf(sv[i] - m_safe);
     ps += p;
-    pf.h[i] = f2bf(p);
+    ph[i] = f2bf(p);
   }
-  l = l * alpha + ps;
-  m = m_new;
-  if (check) {
-    // rows never written may hold anything, NaN included, and 0 * NaN is NaN
+  // the running maximum settles after a few blocks; then nothing needs rescaling
+  if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+    const float alpha = __expf(m - m_safe);
+    l *= alpha;
 #pragma unroll
     for (int d = 0; d < HD / 16; ++d)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (key0 + quad * 4 + i > kv_last) vf[d].h[i] = 0;
+      for (int i = 0; i < 4; ++i) o[d][i] *= alpha;
+    m = m_new;
   }
+  l += ps;
 #pragma unroll
-  for (int d = 0; d < HD / 16; ++d) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) o[d][i] *= alpha;
-    o[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[d].v, pf.v, o[d], 0, 0, 0);
+  for (int d = 0; d < HD / 16; ++d)
+    o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[d].v, pf.v, o[d], 0, 0, 0);
+}
+
+// Walk blocks first, first + stride, ... (n of them) of one request, two at a time.
+// The page ids of 64 blocks are fetched at once, one per lane, so that the walk waits
+// for the block table once per 1024 positions and not once per block; within such a
+// run the loads of the next pair are in flight while a pair is computed (two fragment
+// sets take turns; loads past the end repeat the last block and are not used).
+// `check(block)` tells whether a block needs masks.
+template <int HD, typename Check>
+__device__ __forceinline__ void walk_blocks(const PagedKV& kv, const Frag8* qf, int first, int stride, int n,
+                                            int lo, int hi, int kv_last, float scale, Check check, float& m,
+                                            float& l, floatx4* o) {
+  const int lane = threadIdx.x & 63;
+  for (int c0 = 0; c0 < n; c0 += 64) {
+    const int nc = min(64, n - c0);
+    const int mine = (lane < nc) ? kv.table[((first + (c0 + lane) * stride) * 16) / kv.P] : -1;
+    KVPair<HD> f0, f1;
+    BlockInfo a0, b0, a1, b1;
+    // block j of this run, clamped to the run's last block
+    auto info = [&](int j, int& page) {
+      const int jc = min(j, nc - 1);
+      const int blk = first + (c0 + jc) * stride;
+      page = __builtin_amdgcn_readlane(mine, jc);
+      return BlockInfo{blk * 16, j < nc && page >= 0, check(blk)};
+    };
+    auto issue = [&](int j, KVPair<HD>& f, BlockInfo& A, BlockInfo& B) {
+      int pa, pb;
+      A = info(j, pa);
+      B = info(j + 1, pb);
+      load_pair<HD>(kv, max(pa, 0), A.key0, max(pb, 0), B.key0, f);
+    };
+    issue(0, f0, a0, b0);
+    for (int i = 0; i < nc; i += 4) {
+      issue(i + 2, f1, a1, b1);
+      attend_pair<HD>(f0, qf, a0, b0, lo, hi, kv_last, scale, m, l, o);
+      issue(i + 4, f0, a0, b0);
+      if (i + 2 < nc) attend_pair<HD>(f1, qf, a1, b1, lo, hi, kv_last, scale, m, l, o);
+    }
   }
 }
 
@@ -164,9 +257,10 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
 #pragma unroll
   for (int d = 0; d < HD / 16; ++d) o[d] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  for (int b = b0 + wave; b < b1; b += 4) {
-    const bool check = (b == blk_lo) || (b == blk_hi);
-    attend_block<HD>(kv, qf, b * 16, lo, p_q, p_q, check, scale, mx, l, o);
+  {
+    const int mine = (b1 - (b0 + wave) + 3) / 4;   // blocks b0 + wave, + 4, ... below b1
+    walk_blocks<HD>(kv, qf, b0 + wave, 4, mine, lo, p_q, p_q, scale,
+                    [=](int b) { return b == blk_lo || b == blk_hi; }, mx, l, o);
   }
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -219,24 +313,44 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
   }
 }
 
-// grid (rows, n_head), HD threads: out = sum_s w_s o_s / sum_s w_s l_s, w_s = exp(m_s - max m)
+// grid (rows, n_head), max(HD, 64) threads: out = sum_s w_s o_s / sum_s w_s l_s, w_s = exp(m_s - max m).
+// The statistics of all splits are fetched at once into LDS and the partial outputs
+// in batches of eight independent loads: the kernel waits for memory a few times,
+// not once per split.
+#define MERGE_MAX_SPLITS 64
 template <int HD>
-__global__ void __launch_bounds__(HD)
+__global__ void __launch_bounds__(HD < 64 ? 64 : HD)
 attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                   const int* __restrict__ rows, bf16_t* __restrict__ out, int n_head, int n_splits) {
+  __shared__ float s_w[MERGE_MAX_SPLITS];
+  __shared__ float s_inv;
   const int ridx = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
   const int m_row = rows ? rows[ridx] : ridx;
   const float* pm = part_ml + ((size_t)ridx * n_head + head) * n_splits * 2;
   const float* po = part_o + ((size_t)ridx * n_head + head) * n_splits * HD;
-  float mm = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, pm[2 * s]);
-  float lt = 0.f, acc = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float w = (pm[2 * s] == -INFINITY) ? 0.f : __expf(pm[2 * s] - mm);
-    lt += pm[2 * s + 1] * w;
-    acc += po[(size_t)s * HD + d] * w;
+  // one wavefront fetches (max, sum) of every split and turns them into weights
+  if (d < 64) {
+    const float ms = (d < n_splits) ? pm[2 * d] : -INFINITY;
+    const float ls = (d < n_splits) ? pm[2 * d + 1] : 0.f;
+    const float mm = group_max<64>(ms);
+    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - mm);
+    const float lt = group_sum<64>(ls * w);
+    s_w[d] = w;
+    if (d == 0) s_inv = 1.0f / lt;
   }
-  out[((size_t)m_row * n_head + head) * HD + d] = f2bf(acc / lt);
+  __syncthreads();
+  if (d >= HD) return;
+  float acc = 0.f;
+  int s = 0;
+  for (; s + 8 <= n_splits; s += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = po[(size_t)(s + j) * HD + d];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc += v[j] * s_w[s + j];
+  }
+  for (; s < n_splits; ++s) acc += po[(size_t)s * HD + d] * s_w[s];
+  out[((size_t)m_row * n_head + head) * HD + d] = f2bf(acc * s_inv);
 }
 
 // ================================================================== prefill
@@ -281,12 +395,14 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ poo
   // a block is free of checks if every column sees all of it: it ends at or before the
   // tile's first position and (with a window) starts inside the last column's window
   const int hi_col = col_ok ? my_pos : -1;          // columns beyond the portion see nothing
-  for (int b = blk_lo; b <= blk_hi; ++b) {
-    const int key0 = b * 16;
-    const bool inside = (key0 + 15 <= pos_first) && (w_rows == 16) &&
-                        (window <= 0 || key0 >= pos_last - window + 1) && (key0 >= tile_lo);
-    attend_block<HD>(kv, qf, key0, my_lo, hi_col, kv_last, !inside, scale, mx, l, o);
-  }
+  walk_blocks<HD>(kv, qf, blk_lo, 1, blk_hi - blk_lo + 1, my_lo, hi_col, kv_last, scale,
+                  [=](int b) {
+                    const int key0 = b * 16;
+                    const bool inside = (key0 + 15 <= pos_first) && (w_rows == 16) &&
+                                        (window <= 0 || key0 >= pos_last - window + 1) && (key0 >= tile_lo);
+                    return !inside;
+                  },
+                  mx, l, o);
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!col_ok) return;
@@ -327,7 +443,7 @@ extern "C" int ti_attention_decode_bf16(const void* q, const void* pool, const i
                                         hipStream_t stream) {
   int rc = check_common("attention_decode", n_head, n_kv, hd, page_size, table_stride);
   if (rc) return rc;
-  TI_REQUIRE(n_splits >= 1 && n_splits <= 65535, "attention_decode: bad split count %d", n_splits);
+  TI_REQUIRE(n_splits >= 1 && n_splits <= MERGE_MAX_SPLITS, "attention_decode: bad split count %d (1..%d)", n_splits, MERGE_MAX_SPLITS);
   TI_REQUIRE(n_splits == 1 || (part_o && part_ml), "attention_decode: splits need partial buffers");
   if (n_rows == 0) return 0;
   const int parts = (n_head / n_kv + 15) / 16;
@@ -340,7 +456,8 @@ extern "C" int ti_attention_decode_bf16(const void* q, const void* pool, const i
                                                     part_ml, n_head, n_kv, page_size, scale, window,        \
                                                     n_splits);                                              \
     if (n_splits > 1)                                                                                       \
-      attn_merge_kernel<H><<<dim3(n_rows, n_head), H, 0, stream>>>(part_o, part_ml, rows, (bf16_t*)out,     \
+      attn_merge_kernel<H><<<dim3(n_rows, n_head), (H < 64 ? 64 : H), 0, stream>>>(part_o, part_ml, rows,   \
+                                                                                  (bf16_t*)out,            \
                                                                    n_head, n_splits);                       \
     break;
   switch (hd) {

@@ -98,11 +98,34 @@ extern "C" int ti_rope_neox(float* x, const int* pos, const float* inv_freq, int
   return 0;
 }
 
+// ---------------------------------------------------------- sin/cos table
+// table[p][k] = (cos, sin)(float(p) * inv_freq[k]) for p < n_pos: the same 32-bit
+// angle and the same precise sincosf the kernels would compute on the fly.
+__global__ void rope_table_kernel(float2* __restrict__ table, const float* __restrict__ inv_freq, int half,
+                                  int n_pos) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_pos * half) return;
+  const int p = i / half, k = i % half;
+  float s, c;
+  sincosf((float)p * inv_freq[k], &s, &c);
+  table[i] = make_float2(c, s);
+}
+
+extern "C" int ti_rope_table(float* table, const float* inv_freq, int half, int n_pos, hipStream_t stream) {
+  TI_REQUIRE(half > 0 && n_pos > 0, "rope_table: bad sizes half=%d positions=%d", half, n_pos);
+  const long n = (long)half * n_pos;
+  rope_table_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>((float2*)table, inv_freq, half, n_pos);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
 // ------------------------------------- per-head norm + rotation + cache write
-// One workgroup per token; each wave takes whole heads in turn.  For q heads and
-// k heads: RMS-norm over head_dim (if a weight is given), then the half-split
-// rotation (if inv_freq is given).  q goes to q_out (T), k and v into the cache
-// page of the token's position, page = table[slot][pos / P]:
+// One wavefront per (token, head): grid (M, ceil(units / 4)), units = q heads +
+// k heads + v heads.  For q heads and k heads: RMS-norm over head_dim (if a weight
+// is given), then the half-split rotation (if inv_freq is given; cos and sin come
+// from `rope_table` for positions below `table_len`, else they are computed).  q
+// goes to q_out (T), k and v into the cache page of the token's position,
+// page = table[slot][pos / P]:
 //   keys   pool[page][0][kv head][pos % P][d]   (a key's dims are contiguous: the
 //                                                 score sums over d)
 //   values pool[page][1][kv head][d][pos % P]   (transposed: the mix sums over
@@ -110,76 +133,78 @@ extern "C" int ti_rope_neox(float* x, const int* pos, const float* inv_freq, int
 // v is copied unchanged.  n_kv == 0: only q is handled (the layer reads another
 // layer's keys and values).
 template <typename T>
-__global__ void qk_norm_rope_kv_write_kernel(
+__global__ void __launch_bounds__(256)
+qk_norm_rope_kv_write_kernel(
     const float* __restrict__ qkv, const float* __restrict__ q_w, const float* __restrict__ k_w,
-    const float* __restrict__ inv_freq, const int* __restrict__ pos, const int* __restrict__ slot,
+    const float* __restrict__ inv_freq, const float2* __restrict__ rope_table, int table_len,
+    const int* __restrict__ pos, const int* __restrict__ slot,
     const int* __restrict__ table, int table_stride, T* __restrict__ pool, T* __restrict__ q_out,
     int n_head, int n_kv, int hd, int P, float eps) {
   const int m = blockIdx.x;
   const int wave = threadIdx.x / TI_WAVE, lane = threadIdx.x % TI_WAVE;
-  const int n_waves = blockDim.x / TI_WAVE;
+  const int u = blockIdx.y * (blockDim.x / TI_WAVE) + wave;
+  if (u >= n_head + 2 * n_kv) return;
   const int half = hd / 2;
   const int nq = n_head * hd, nk = n_kv * hd;
   const float* row = qkv + (size_t)m * (nq + 2 * nk);
   const int p = pos[m];
-  const float fp = (float)p;
-  size_t page_base = 0;
-  int prow = 0;
-  bool page_ok = false;
-  if (n_kv > 0) {
+  const bool is_q = u < n_head;
+  const bool is_v = u >= n_head + n_kv;
+  const float* src = row + (size_t)u * hd;
+  T* dst;
+  if (is_q) {
+    dst = q_out + (size_t)m * nq + (size_t)u * hd;
+  } else {
     const int page = table[(size_t)slot[m] * table_stride + p / P];
-    page_ok = page >= 0;
-    page_base = (size_t)(page_ok ? page : 0) * 2 * n_kv * P * hd;
-    prow = p % P;
+    if (page < 0) return;   // the host reserves pages first; never write astray
+    const int prow = p % P;
+    const int kvh = is_v ? u - n_head - n_kv : u - n_head;
+    dst = pool + (size_t)page * 2 * n_kv * P * hd + ((size_t)(is_v ? 1 : 0) * n_kv + kvh) * P * hd +
+          (is_v ? (size_t)prow : (size_t)prow * hd);
   }
-  for (int u = wave; u < n_head + 2 * n_kv; u += n_waves) {
-    const bool is_q = u < n_head;
-    const bool is_v = u >= n_head + n_kv;
-    const float* src = row + (size_t)u * hd;
-    T* dst;
-    if (is_q) {
-      dst = q_out + (size_t)m * nq + (size_t)u * hd;
-    } else {
-      if (!page_ok) continue;   // the host reserves pages first; never write astray
-      const int kvh = is_v ? u - n_head - n_kv : u - n_head;
-      dst = pool + page_base + ((size_t)(is_v ? 1 : 0) * n_kv + kvh) * P * hd + (is_v ? (size_t)prow : (size_t)prow * hd);
-    }
-    if (is_v) {
-      for (int i = lane; i < hd; i += TI_WAVE) st<T>(dst + (size_t)i * P, src[i]);
-      continue;
-    }
-    const float* w = is_q ? q_w : k_w;
+  if (is_v) {
+    for (int i = lane; i < hd; i += TI_WAVE) st<T>(dst + (size_t)i * P, src[i]);
+    return;
+  }
+  const float* w = is_q ? q_w : k_w;
+  float scale = 1.f;
+  if (w) {
     float ss = 0.f;
     for (int i = lane; i < half; i += TI_WAVE) {
       const float lo = src[i], hi = src[i + half];
       ss += lo * lo + hi * hi;
     }
-    float scale = 1.f;
+    ss = group_sum<TI_WAVE>(ss);
+    scale = 1.0f / sqrtf(ss / (float)hd + eps);
+  }
+  const float fp = (float)p;
+  for (int i = lane; i < half; i += TI_WAVE) {
+    float lo = src[i] * scale, hi = src[i + half] * scale;
     if (w) {
-      ss = group_sum<TI_WAVE>(ss);
-      scale = 1.0f / sqrtf(ss / (float)hd + eps);
+      lo *= w[i];
+      hi *= w[i + half];
     }
-    for (int i = lane; i < half; i += TI_WAVE) {
-      float lo = src[i] * scale, hi = src[i + half] * scale;
-      if (w) {
-        lo *= w[i];
-        hi *= w[i + half];
-      }
-      if (inv_freq) {
-        float s, c;
+    if (inv_freq) {
+      float s, c;
+      if (rope_table && p < table_len) {
+        const float2 cs = rope_table[(size_t)p * half + i];
+        c = cs.x;
+        s = cs.y;
+      } else {
         sincosf(fp * inv_freq[i], &s, &c);
-        const float a = lo * c - hi * s, b = lo * s + hi * c;
-        lo = a;
-        hi = b;
       }
-      st<T>(dst + i, lo);
-      st<T>(dst + i + half, hi);
+      const float a = lo * c - hi * s, b = lo * s + hi * c;
+      lo = a;
+      hi = b;
     }
+    st<T>(dst + i, lo);
+    st<T>(dst + i + half, hi);
   }
 }
 
 extern "C" int ti_qk_norm_rope_kv_write(int dtype, const float* qkv, const float* q_w, const float* k_w,
-                                        const float* inv_freq, const int* pos, const int* slot,
+                                        const float* inv_freq, const float* rope_table, int table_len,
+                                        const int* pos, const int* slot,
                                         const int* table, int table_stride, void* pool, void* q_out,
                                         int M, int n_head, int n_kv, int hd, int page_size, float eps,
                                         hipStream_t stream) {
@@ -188,14 +213,17 @@ extern "C" int ti_qk_norm_rope_kv_write(int dtype, const float* qkv, const float
              "qk_norm_rope_kv_write: bad sizes heads=%d kv_heads=%d page=%d table_stride=%d", n_head, n_kv,
              page_size, table_stride);
   if (M == 0) return 0;
+  const int units = n_head + 2 * n_kv;
+  TI_REQUIRE((units + 3) / 4 <= 65535, "qk_norm_rope_kv_write: too many heads");
+  dim3 grid(M, (units + 3) / 4);
   if (dtype == TI_F32)
-    qk_norm_rope_kv_write_kernel<float><<<M, 256, 0, stream>>>(qkv, q_w, k_w, inv_freq, pos, slot, table,
-                                                              table_stride, (float*)pool, (float*)q_out,
-                                                              n_head, n_kv, hd, page_size, eps);
+    qk_norm_rope_kv_write_kernel<float><<<grid, 256, 0, stream>>>(
+        qkv, q_w, k_w, inv_freq, (const float2*)rope_table, table_len, pos, slot, table, table_stride,
+        (float*)pool, (float*)q_out, n_head, n_kv, hd, page_size, eps);
   else if (dtype == TI_BF16)
-    qk_norm_rope_kv_write_kernel<bf16_t><<<M, 256, 0, stream>>>(qkv, q_w, k_w, inv_freq, pos, slot, table,
-                                                               table_stride, (bf16_t*)pool, (bf16_t*)q_out,
-                                                               n_head, n_kv, hd, page_size, eps);
+    qk_norm_rope_kv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>(
+        qkv, q_w, k_w, inv_freq, (const float2*)rope_table, table_len, pos, slot, table, table_stride,
+        (bf16_t*)pool, (bf16_t*)q_out, n_head, n_kv, hd, page_size, eps);
   else
     TI_REQUIRE(false, "qk_norm_rope_kv_write: unknown dtype %d", dtype);
   TI_LAUNCH_CHECK();

@@ -24,6 +24,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
 union Frag {
   uint4 u;
   bf16x8 v;
@@ -257,6 +259,222 @@ gemm_tiled_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, vo
   }
 }
 
+// ====================================================== tiled kernel, pipelined
+// The same product with the tiles brought in by direct global-to-LDS loads
+// (global_load_lds_dwordx4: each lane fetches 16 bytes, the wavefront's 64 pieces
+// land in 1 KiB of LDS in lane order) three stages deep, so that two k-tiles are in
+// flight while one is multiplied (K must be a multiple of 64; other K take the plain
+// tiled kernel).  BK = 64: a tile row is 128 bytes = 8 pieces.  Rows
+// are stored unpadded, and piece c of row r sits in slot c ^ ((r >> 1) & 7): the 16
+// rows that one phase of a 16-byte LDS read touches then fall on all 64 banks once.
+// The lane that fills slot (r, c) simply fetches piece c ^ ((r >> 1) & 7) of row r.
+//
+// WG tile BM x BN, four wavefronts as WAVES_M x WAVES_N, each (BM / WAVES_M) x
+// (BN / WAVES_N) out of 32 x 32 x 16 MFMAs.  SwiGLU needs two 32-column tiles per
+// wavefront: tile 0 holds gate columns, tile 1 the matching up columns.
+#define PBK 64
+#define PSTAGES 3
+
+__device__ __forceinline__ void wait_vmcnt(int n) {
+  // s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
+  switch (n) {
+    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+#define TI_W(N) case N: __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | (((N) >> 4) << 14)); break;
+    TI_W(1) TI_W(2) TI_W(3) TI_W(4) TI_W(5) TI_W(6) TI_W(7) TI_W(8) TI_W(9) TI_W(10) TI_W(11) TI_W(12)
+    TI_W(13) TI_W(14) TI_W(15) TI_W(16) TI_W(20) TI_W(24)
+#undef TI_W
+    default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+  }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+__global__ void __launch_bounds__(256)
+gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_,
+                      int M, int N, int K, long lda) {
+  constexpr bool SW = (EPI == TI_EPI_SWIGLU);
+  constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
+  static_assert(WAVES_M * WAVES_N == 4, "four wavefronts");
+  static_assert(!SW || TN == 2, "SwiGLU pairs two column tiles per wavefront");
+  constexpr int STAGE_BYTES = (BM + BN) * PBK * 2;
+  constexpr int GROUPS_A = BM / 8, GROUPS_B = BN / 8;        // 8 rows = 1 KiB = one wavefront load
+  constexpr int LOADS = (GROUPS_A + GROUPS_B) / 4;           // per wavefront and k-tile
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int m0 = blockIdx.y * BM;
+  const int n0 = blockIdx.x * (SW ? BN / 2 : BN);
+  const int lr = lane >> 3, lc = lane & 7;                   // row within a group of 8, slot within the row
+
+  // the global row each of this lane's loads reads (clamped into the matrix: rows
+  // beyond it are computed and thrown away), as a pointer to its first element
+  const bf16_t* gsrc[LOADS];
+  int gpiece[LOADS];                                         // which 8-element piece of the row this lane fetches
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int g = wave + 4 * i;                              // groups 0..GROUPS_A-1: A, then B
+    if (g < GROUPS_A) {
+      const int row = g * 8 + lr;
+      const int gm = min(m0 + row, M - 1);
+      gsrc[i] = A + (size_t)gm * lda;
+      gpiece[i] = lc ^ ((row >> 1) & 7);
+    } else {
+      const int row = (g - GROUPS_A) * 8 + lr;
+      int wr;
+      if (SW) {
+        const int span = BN / WAVES_N;                       // 64: LDS rows of one wavefront's columns
+        const int n = n0 + (row / span) * 32 + (row & 31);
+        wr = ((row & 32) ? N : 0) + min(n, N - 1);
+      } else {
+        wr = min(n0 + row, N - 1);
+      }
+      gsrc[i] = W + (size_t)wr * K;
+      gpiece[i] = lc ^ ((row >> 1) & 7);
+    }
+  }
+
+  auto issue = [&](int kt) {
+    unsigned char* stage = smem + (kt % PSTAGES) * STAGE_BYTES;
+    const int k0 = kt * PBK;
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int g = wave + 4 * i;
+      unsigned char* dst = stage + g * 1024;                 // the same in every lane
+      // K is a multiple of 64 here (the dispatcher sees to it): no piece lies past the end
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(gsrc[i] + k0 + gpiece[i] * 8),
+          (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    }
+  };
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int a = 0; a < TM; ++a)
+#pragma unroll
+    for (int b = 0; b < TN; ++b)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+
+  // The multiply loop is scheduled by hand.  The compiler does not know which LDS
+  // bytes a direct load will write, so before any LDS read it can see, and at every
+  // fence, it waits for all of them, the two k-tiles in flight included; that would
+  // undo the pipeline.  So LDS is read with ds_read_b128 in inline assembly, the
+  // barrier is the bare instruction, and the waits are written out: vmcnt before the
+  // barrier (the tile about to be multiplied has landed), lgkmcnt before each group of
+  // MFMAs (its fragments have arrived; those of the next k-step are still in flight).
+  const int fr = lane & 31, fh = lane >> 5;                  // fragment row, and which half of a 16-wide k-step
+  const unsigned lds0 = (unsigned)(size_t)smem;              // LDS byte address of the first stage
+  const unsigned rowA = lds0 + (wm * (BM / WAVES_M) + fr) * 128;
+  const unsigned rowB = lds0 + BM * PBK * 2 + (wn * (BN / WAVES_N) + fr) * 128;
+  unsigned xo[PBK / 16];                                     // swizzled byte offset of this lane's piece, per k-step
+#pragma unroll
+  for (int ks = 0; ks < PBK / 16; ++ks) xo[ks] = ((ks * 2 + fh) ^ ((fr >> 1) & 7)) << 4;
+
+  const int n_k = K / PBK;
+  issue(0);
+  if (n_k > 1) issue(1);
+  for (int kt = 0; kt < n_k; ++kt) {
+    // tile kt has landed (its loads are older than those of tile kt + 1), in every wavefront,
+    // and every wavefront has finished with the stage that tile kt + 2 goes into
+    if (kt + 1 < n_k) wait_vmcnt(LOADS); else wait_vmcnt(0);
+    __builtin_amdgcn_s_barrier();
+    if (kt + 2 < n_k) issue(kt + 2);
+    const unsigned st = (kt % PSTAGES) * STAGE_BYTES;
+    v4u fa[2][TM], fb[2][TN];
+    auto read_step = [&](int ks, int set) {
+      const unsigned pa = rowA + st + xo[ks], pb = rowB + st + xo[ks];
+#pragma unroll
+      for (int a = 0; a < TM; ++a)
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[set][a]) : "v"(pa), "n"(a * 32 * 128));
+#pragma unroll
+      for (int b = 0; b < TN; ++b)
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[set][b]) : "v"(pb), "n"(b * 32 * 128));
+    };
+    read_step(0, 0);
+#pragma unroll
+    for (int ks = 0; ks < PBK / 16; ++ks) {
+      const int set = ks & 1;
+      if (ks + 1 < PBK / 16) {
+        read_step(ks + 1, set ^ 1);
+        // all but the TM + TN reads just issued are done: this k-step's fragments are there
+        if (TM + TN == 6) asm volatile("s_waitcnt lgkmcnt(6)" ::: "memory");
+        if (TM + TN == 4) asm volatile("s_waitcnt lgkmcnt(4)" ::: "memory");
+        if (TM + TN == 3) asm volatile("s_waitcnt lgkmcnt(3)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
+      // tie the fragments to the wait, so that no MFMA is moved above it
+#pragma unroll
+      for (int a = 0; a < TM; ++a) asm volatile("" : "+v"(fa[set][a]));
+#pragma unroll
+      for (int b = 0; b < TN; ++b) asm volatile("" : "+v"(fb[set][b]));
+#pragma unroll
+      for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[set][a]),
+                                                              __builtin_bit_cast(bf16x8, fb[set][b]), acc[a][b],
+                                                              0, 0, 0);
+    }
+  }
+
+  // acc[a][b][i]: row wm*(BM/WAVES_M) + a*32 + 8*(i/4) + 4*(lane/32) + i%4, column wn*(BN/WAVES_N) + b*32 + lane%32
+  const int ccol = lane & 31, crow = (lane >> 5) * 4;
+#pragma unroll
+  for (int a = 0; a < TM; ++a) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int m = m0 + wm * (BM / WAVES_M) + a * 32 + (i >> 2) * 8 + crow + (i & 3);
+      if (m >= M) continue;
+      if (SW) {
+        const int n = n0 + wn * 32 + ccol;
+        if (n < N) ((bf16_t*)out_)[(size_t)m * N + n] = f2bf(silu_mul(acc[a][0][i], acc[a][TN - 1][i]));
+      } else {
+#pragma unroll
+        for (int b = 0; b < TN; ++b) {
+          const int n = n0 + wn * (BN / WAVES_N) + b * 32 + ccol;
+          if (n >= N) continue;
+          const size_t o = (size_t)m * N + n;
+          const float v = acc[a][b][i];
+          if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = v;
+          if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] += v;
+          if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(v);
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
+                            hipStream_t s) {
+  constexpr int bytes = PSTAGES * (BM + BN) * PBK * 2;
+  auto kernel = gemm_pipelined_kernel<BM, BN, WAVES_M, WAVES_N, EPI>;
+  static bool ready = false;          // per instantiation: allow more than 64 KiB of dynamic LDS
+  if (!ready) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+      ti_set_error("gemm_bf16: cannot reserve %d bytes of LDS", bytes);
+      return 2;
+    }
+    ready = true;
+  }
+  const int bn = (EPI == TI_EPI_SWIGLU) ? BN / 2 : BN;
+  dim3 grid((N + bn - 1) / bn, (M + BM - 1) / BM);
+  kernel<<<grid, 256, bytes, s>>>(A, W, out, M, N, K, lda);
+  return 0;
+}
+
+// the largest tile that still gives every compute unit a workgroup
+template <int EPI>
+static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
+                             hipStream_t s) {
+  const int cols = (EPI == TI_EPI_SWIGLU) ? 2 : 1;   // a SwiGLU workgroup covers BN / 2 output columns
+  auto count = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N * cols + bn - 1) / bn); };
+  if (count(256, 128) >= 256) return launch_pipelined<256, 128, 2, 2, EPI>(A, W, out, M, N, K, lda, s);
+  if (count(128, 128) >= 256) return launch_pipelined<128, 128, 2, 2, EPI>(A, W, out, M, N, K, lda, s);
+  return launch_pipelined<128, 64, 4, 1, EPI>(A, W, out, M, N, K, lda, s);
+}
+
 // ------------------------------------------------------------------- dispatch
 template <int EPI>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
@@ -276,6 +494,10 @@ static void launch_tiled(const bf16_t* A, const bf16_t* W, void* out, int M, int
   dim3 grid((N + bn - 1) / bn, (M + TBM - 1) / TBM);
   gemm_tiled_kernel<EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
 }
+
+static int g_use_pipelined = 1;
+// 1: the pipelined tiled kernel for M > 64 (default); 0: the plain tiled kernel (for comparison)
+extern "C" void ti_gemm_bf16_use_pipelined(int on) { g_use_pipelined = on; }
 
 // N: output columns (SwiGLU: F, with W holding 2F rows).  Returns 3 for a shape
 // these kernels do not serve (the caller takes the generic kernel then).
@@ -298,7 +520,10 @@ extern "C" int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int 
   case E:                                                         \
     if (skinny)                                                   \
       launch_skinny<E>(a, w, out, M, N, K, lda, stream);          \
-    else                                                          \
+    else if (g_use_pipelined && K % PBK == 0) {                   \
+      int rc_ = launch_tiled_best<E>(a, w, out, M, N, K, lda, stream); \
+      if (rc_) return rc_;                                        \
+    } else                                                        \
       launch_tiled<E>(a, w, out, M, N, K, lda, stream);           \
     break;
   switch (epi) {

@@ -80,6 +80,73 @@ argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
   if (threadIdx.x == 0) out[r] = best;
 }
 
+// Greedy choice of a long row in two steps, so that a row is read by many
+// workgroups at once: grid (rows, ARG_PARTS) finds the best of each slice, then
+// one wavefront per row picks among the ARG_PARTS winners (lowest index on ties).
+#define ARG_PARTS 64
+__global__ void __launch_bounds__(256)
+argmax_part_kernel(const float* __restrict__ logits, float* __restrict__ part_val, int* __restrict__ part_idx,
+                   int V) {
+  __shared__ float s_val[4];
+  __shared__ int s_idx[4];
+  const int r = blockIdx.x, c = blockIdx.y;
+  const int chunk = (V + ARG_PARTS - 1) / ARG_PARTS;
+  const int b = c * chunk, e = min(V, b + chunk);
+  const float* row = logits + (size_t)r * V;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = b + threadIdx.x; i < e; i += 256) {
+    const float v = row[i];
+    if (v > bv || (bi == 0x7fffffff && v == v)) {
+      bv = v;
+      bi = i;
+    }
+  }
+#pragma unroll
+  for (int o = TI_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, TI_WAVE);
+    const int oi = __shfl_xor(bi, o, TI_WAVE);
+    if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) {
+      bv = ov;
+      bi = oi;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_val[threadIdx.x >> 6] = bv;
+    s_idx[threadIdx.x >> 6] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) {
+      const float ov = s_val[w];
+      const int oi = s_idx[w];
+      if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    part_val[r * ARG_PARTS + c] = bv;
+    part_idx[r * ARG_PARTS + c] = bi;
+  }
+}
+
+__global__ void __launch_bounds__(64)
+argmax_final_kernel(const float* __restrict__ part_val, const int* __restrict__ part_idx, int* __restrict__ out) {
+  const int r = blockIdx.x;
+  float bv = part_val[r * ARG_PARTS + threadIdx.x];
+  int bi = part_idx[r * ARG_PARTS + threadIdx.x];
+#pragma unroll
+  for (int o = TI_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, TI_WAVE);
+    const int oi = __shfl_xor(bi, o, TI_WAVE);
+    if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) {
+      bv = ov;
+      bi = oi;
+    }
+  }
+  if (threadIdx.x == 0) out[r] = bi == 0x7fffffff ? 0 : bi;
+}
+
 // temp[r] <= 0: greedy.  top_k[r] <= 0 or >= V: no top-k cut.  top_p[r] >= 1: no top-p cut.
 __global__ void __launch_bounds__(SNT)
 sample_kernel(const float* __restrict__ logits, const float* __restrict__ temp, const int* __restrict__ top_k,
@@ -185,10 +252,18 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temp, 
   if (threadIdx.x == 0) out[r] = s_pick;
 }
 
-extern "C" int ti_argmax(const float* logits, int* out, int n_rows, int V, hipStream_t stream) {
+// scratch: 2 * n_rows * 64 four-byte words, or nullptr (then one workgroup reads a whole row)
+extern "C" int ti_argmax(const float* logits, int* out, void* scratch, int n_rows, int V, hipStream_t stream) {
   TI_REQUIRE(n_rows >= 0 && V > 0, "argmax: bad sizes rows=%d V=%d", n_rows, V);
   if (n_rows == 0) return 0;
-  argmax_kernel<<<n_rows, SNT, 0, stream>>>(logits, out, V);
+  if (scratch && V >= 16384) {
+    float* pv = (float*)scratch;
+    int* pi = (int*)scratch + (size_t)n_rows * ARG_PARTS;
+    argmax_part_kernel<<<dim3(n_rows, ARG_PARTS), 256, 0, stream>>>(logits, pv, pi, V);
+    argmax_final_kernel<<<n_rows, 64, 0, stream>>>(pv, pi, out);
+  } else {
+    argmax_kernel<<<n_rows, SNT, 0, stream>>>(logits, out, V);
+  }
   TI_LAUNCH_CHECK();
   return 0;
 }

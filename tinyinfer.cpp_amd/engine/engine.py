@@ -119,6 +119,9 @@ class Engine:
         self.cache = CacheManager(model.cache_groups, self.page_size, self.num_pages, max_requests, self.max_seq)
         self.storage = CacheStorage(self.cache, self.act_dtype, self.device)
         self.table_width = self.cache.max_pages_per_request
+        for part in model.parts():
+            if hasattr(part, "prepare"):
+                part.prepare(self.ops, self.max_seq)      # tables that depend on the longest sequence
         self._ws: Dict[str, torch.Tensor] = {}
         self._meta_dev = None
         self._meta_host: List[torch.Tensor] = []

@@ -10,9 +10,9 @@ import ctypes
 import torch
 
 SERVED_HEAD_DIMS = (32, 64, 128)
-TARGET_WORKGROUPS = 1024      # a few per compute unit (256 of them)
-MAX_SPLITS = 64
-MIN_BLOCKS_PER_SPLIT = 4      # one 16-key block per wavefront at least
+TARGET_WORKGROUPS = 256       # one per compute unit: a unit streams about as fast with 4 wavefronts as with 8
+MAX_SPLITS = 64               # the merge kernel's limit
+MIN_BLOCKS_PER_SPLIT = 8      # two 16-key blocks per wavefront at least
 
 
 def decode_splits(n_rows: int, kv_heads: int, heads: int, context: int) -> int:

@@ -124,8 +124,18 @@ class Ops:
                               ctypes.c_long(x.stride(0)), self._stream())
         self._check(lib, rc, "rope")
 
+    def rope_table(self, inv_freq, n_pos):
+        """float32 [n_pos, hd/2, 2] = (cos, sin)(float(p) * inv_freq[k]), computed on the device."""
+        self._dev(inv_freq)
+        half = inv_freq.shape[0]
+        table = torch.empty((n_pos, half, 2), dtype=torch.float32, device=inv_freq.device)
+        lib = self.lib("core")
+        rc = lib.ti_rope_table(_ptr(table), _ptr(inv_freq), half, n_pos, self._stream())
+        self._check(lib, rc, "rope_table")
+        return table
+
     def qk_norm_rope_kv_write(self, qkv, q_w, k_w, eps, inv_freq, positions, slots, view, pool, q_out,
-                              heads, kv_heads, head_dim):
+                              heads, kv_heads, head_dim, rope_table=None):
         """qkv f32 [M, (heads + 2 kv_heads) hd] -> q_out T [M, heads hd] and the cache pages.
         kv_heads = 0: only q (nothing is written to the cache)."""
         M = qkv.shape[0]
@@ -146,8 +156,12 @@ class Ops:
                 raise KernelError(f"qk_norm_rope_kv_write: pool {tuple(pool.shape)} {pool.dtype} does not fit "
                                   f"[pages,2,{kv_heads},P,{head_dim}] of {q_out.dtype}")
         lib = self.lib("core")
+        if rope_table is not None and (rope_table.dtype != torch.float32 or not rope_table.is_contiguous()
+                                       or rope_table.shape[1:] != (head_dim // 2, 2)):
+            raise KernelError("qk_norm_rope_kv_write: the sin/cos table must be float32 [positions, head_dim/2, 2]")
         rc = lib.ti_qk_norm_rope_kv_write(
-            _code(q_out.dtype), _ptr(qkv), _ptr(q_w), _ptr(k_w), _ptr(inv_freq), _ptr(positions), _ptr(slots),
+            _code(q_out.dtype), _ptr(qkv), _ptr(q_w), _ptr(k_w), _ptr(inv_freq), _ptr(rope_table),
+            0 if rope_table is None else rope_table.shape[0], _ptr(positions), _ptr(slots),
             _ptr(view.table), view.table.shape[1], _ptr(pool), _ptr(q_out), M, heads, kv_heads, head_dim,
             pool.shape[3], ctypes.c_float(eps), self._stream())
         self._check(lib, rc, "qk_norm_rope_kv_write")
@@ -221,8 +235,11 @@ class Ops:
         self._dev(logits, out)
         if logits.dtype != torch.float32 or not logits.is_contiguous() or out.dtype != torch.int32 or out.shape[0] < n:
             raise KernelError("argmax: logits must be contiguous float32 [n, V], out int32 [n]")
+        scratch = getattr(self, "_argmax_scratch", None)
+        if scratch is None or scratch.numel() < 2 * 64 * n:
+            scratch = self._argmax_scratch = torch.empty(2 * 64 * max(n, 64), dtype=torch.int32, device=logits.device)
         lib = self.lib("sampling")
-        rc = lib.ti_argmax(_ptr(logits), _ptr(out), n, V, self._stream())
+        rc = lib.ti_argmax(_ptr(logits), _ptr(out), _ptr(scratch), n, V, self._stream())
         self._check(lib, rc, "argmax")
 
     def sample(self, logits, temperature, top_k, top_p, uniform, out):

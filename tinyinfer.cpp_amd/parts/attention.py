@@ -97,7 +97,8 @@ class Attention(Part):
             qkv, self.q_norm_w, self.k_norm_w, self.eps,
             None if rot is None else rot["inv_freq"],
             ctx.positions, ctx.slots, view, pool, q,
-            self.heads, 0 if self.shares_kv else self.kv_heads, self.head_dim)
+            self.heads, 0 if self.shares_kv else self.kv_heads, self.head_dim,
+            None if rot is None else rot.get("table"))
         a = ctx.buf("attn.out", (M, self.nq), ctx.act_dtype)
         ctx.ops.attention(ctx, view, q, pool, a, self.heads, self.kv_heads, self.head_dim,
                           self.scale, self.window)

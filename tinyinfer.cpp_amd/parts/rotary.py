@@ -5,7 +5,8 @@ adjacent-pair variant is the mistake listed in docs/report.md:91).
 
 The inverse frequencies are built once on the host in double precision and
 rounded to float; the angle pos * inv_freq[k] and its sine and cosine are 32-bit
-on the device.
+on the device.  `prepare(n)` tabulates them for positions below n (with the same
+device function a kernel would call for a position beyond the table).
 """
 from __future__ import annotations
 
@@ -29,14 +30,21 @@ class RotaryNeox(Part):
         self._inv_freq_host = torch.pow(
             torch.tensor(self.theta, dtype=torch.float64), -2.0 * k / self.head_dim).to(torch.float32)
         self.inv_freq = None
+        self.table = None
 
     def to(self, device):
         self.inv_freq = self._inv_freq_host.to(device)
+        self.table = None
         return self
+
+    def prepare(self, ops, max_positions: int):
+        """Tabulate cos and sin for positions [0, max_positions)."""
+        if self.inv_freq is not None and (self.table is None or self.table.shape[0] < max_positions):
+            self.table = ops.rope_table(self.inv_freq, int(max_positions))
 
     def fused_rotation(self):
         """Arguments for the fused norm/rotate/cache-write kernel."""
-        return {"inv_freq": self.inv_freq}
+        return {"inv_freq": self.inv_freq, "table": self.table}
 
     def apply(self, ctx, q, k):
         """In place on f32 [M, heads, hd] views (strided rows allowed)."""
