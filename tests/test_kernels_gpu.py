@@ -471,7 +471,7 @@ class FakeCtx:
             pos += list(range(start, start + n))
             slot += [e] * n
             if n > 1:
-                tiles += [[e, row0 + q0] for q0 in range(0, n, 64)]
+                tiles += [[e, row0 + q0] for q0 in range(0, n, 128)]
             else:
                 dec.append(row0)
             row0 += n

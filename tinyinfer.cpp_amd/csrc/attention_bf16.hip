@@ -126,19 +126,19 @@ __device__ __forceinline__ void attend_pair(KVPair<HD>& f, const Frag8* qf, Bloc
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int ka = A.key0 + quad * 4 + i, kb = B.key0 + quad * 4 + i;
-      const bool see_a = A.valid && (!A.check || (ka >= lo && ka <= hi));
-      const bool see_b = B.valid && (!B.check || (kb >= lo && kb <= hi));
+      const bool see_a = A.valid & (!A.check | ((ka >= lo) & (ka <= hi)));   // bitwise: selects, no branches
+      const bool see_b = B.valid & (!B.check | ((kb >= lo) & (kb <= hi)));
       sv[i] = see_a ? sa[i] * scale : -INFINITY;
       sv[4 + i] = see_b ? sb[i] * scale : -INFINITY;
       // rows never written may hold anything, NaN included, and 0 * NaN is NaN
-      const bool zero_a = !A.valid || ka > kv_last, zero_b = !B.valid || kb > kv_last;
-      if (zero_a || zero_b) {
+      const bool zero_a = !A.valid | (ka > kv_last), zero_b = !B.valid | (kb > kv_last);
+      const unsigned keep_a = zero_a ? ((i & 1) ? 0x0000FFFFu : 0xFFFF0000u) : 0xFFFFFFFFu;
+      const unsigned keep_b = zero_b ? ((i & 1) ? 0x0000FFFFu : 0xFFFF0000u) : 0xFFFFFFFFu;
 #pragma unroll
-        for (int d = 0; d < HD / 16; ++d) {
-          bf16_t* h = reinterpret_cast<bf16_t*>(&f.v[d].u);
-          if (zero_a) h[i] = 0;
-          if (zero_b) h[4 + i] = 0;
-        }
+      for (int d = 0; d < HD / 16; ++d) {
+        unsigned* wv = reinterpret_cast<unsigned*>(&f.v[d].u);
+        wv[i >> 1] &= keep_a;             // element i of block A
+        wv[2 + (i >> 1)] &= keep_b;       // element 4 + i: block B
       }
     }
   }
@@ -354,11 +354,11 @@ attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ pa
 }
 
 // ================================================================== prefill
-// grid (tiles, n_head), 256 threads.  tiles[t] = (entry, first row); entries[e] =
-// (row0, n_tokens, start_pos, -).  A tile is 64 rows; wavefront w takes rows
+// grid (tiles, n_head), 512 threads.  tiles[t] = (entry, first row); entries[e] =
+// (row0, n_tokens, start_pos, -).  A tile is 128 rows; wavefront w takes rows
 // first + 16 w .. + 15 as its columns.
 template <int HD>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool, const int* __restrict__ table,
                     int table_stride, const int* __restrict__ tiles, const int* __restrict__ entries,
                     bf16_t* __restrict__ out, int n_head, int n_kv, int P, float scale, int window) {
@@ -416,6 +416,349 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ poo
   }
 }
 
+// ======================================================= prefill, through LDS
+// The prefill kernel for head sizes 64 and 128.  A workgroup takes 128 consecutive
+// tokens of one q head; a wavefront's tokens are column blocks of 32 of
+// v_mfma_f32_32x32x16_bf16 (one block each for four wavefronts, or two each for two).  Keys and values come in turns of 32 keys by direct
+// global-to-LDS loads, several turns deep, and are shared by the wavefronts.
+//
+//   S^T (32 keys x 32 tokens) = K (32 x hd) . Q^T          8 (hd=128) MFMAs per column block
+//   O^T (hd x 32 tokens)     += V^T (hd x 32 keys) . P^T   hd/32 x 2 MFMAs per column block
+//
+// LDS rows of K are not in key order: row r of a 16-row group holds the key whose
+// bits 2 and 3 are those of r swapped.  The score tile then leaves a lane with eight
+// keys that are contiguous in memory (8h .. 8h+7 of each 16), so that the matching
+// V^T fragment is one 16-byte read.  Pieces are XOR-swizzled against bank conflicts.
+#define PF_ROWS 128
+#define PF_KEYS 32
+#define PF_STAGES 4      // LDS stages: PF_STAGES - 1 turns are in flight while one is computed
+
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+
+__device__ __forceinline__ void lgkm_wait(int n) {
+  switch (n) {
+    case 0: asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); break;
+    case 1: asm volatile("s_waitcnt lgkmcnt(1)" ::: "memory"); break;
+    case 2: asm volatile("s_waitcnt lgkmcnt(2)" ::: "memory"); break;
+    case 3: asm volatile("s_waitcnt lgkmcnt(3)" ::: "memory"); break;
+    case 4: asm volatile("s_waitcnt lgkmcnt(4)" ::: "memory"); break;
+    case 5: asm volatile("s_waitcnt lgkmcnt(5)" ::: "memory"); break;
+    case 6: asm volatile("s_waitcnt lgkmcnt(6)" ::: "memory"); break;
+    case 7: asm volatile("s_waitcnt lgkmcnt(7)" ::: "memory"); break;
+    default: asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); break;
+  }
+}
+// wait until at most k * LOADS vector-memory operations are outstanding
+// (s_waitcnt with only vmcnt set: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
+template <int LOADS>
+__device__ __forceinline__ void vm_wait_turns(int k) {
+#define TI_VM(N) __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | ((((N) >> 4) & 3) << 14))
+  static_assert(LOADS * (PF_STAGES - 2) <= 63, "vmcnt has six bits");
+  switch (k) {
+    case 0: TI_VM(0); break;
+    case 1: TI_VM(LOADS); break;
+    case 2: TI_VM(2 * LOADS); break;
+    case 3: TI_VM(3 * LOADS); break;
+    case 4: TI_VM(4 * LOADS); break;
+    case 5: TI_VM(5 * LOADS); break;
+    case 6: TI_VM(6 * LOADS); break;
+    default: TI_VM(0); break;
+  }
+#undef TI_VM
+}
+
+// CB: column blocks (of 32 tokens) per wavefront; the workgroup has 4 / CB wavefronts.
+template <int HD, int CB>
+__global__ void __launch_bounds__(256 / CB)
+attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool,
+                        const int* __restrict__ table, int table_stride, const int* __restrict__ tiles,
+                        const int* __restrict__ entries, bf16_t* __restrict__ out, int n_head, int n_kv, int P,
+                        float scale, int window) {
+  constexpr int NW = 4 / CB;                          // wavefronts
+  constexpr int WROWS = 32 * CB;                      // tokens per wavefront
+  constexpr int NP = HD / 8;                          // 16-byte pieces per K row
+  constexpr int K_BYTES = PF_KEYS * HD * 2;
+  constexpr int STAGE = 2 * K_BYTES;                  // K tile + V^T tile
+  constexpr int K_ROWS = 1024 / (HD * 2);             // K rows per wavefront load
+  constexpr int K_LOADS = PF_KEYS / K_ROWS;
+  constexpr int V_LOADS = HD / 16;                    // 16 dims (64 bytes each) per wavefront load
+  static_assert(K_LOADS % NW == 0 && V_LOADS % NW == 0, "every wavefront takes the same kinds of loads");
+  constexpr int MY_K = K_LOADS / NW, MY_LOADS = (K_LOADS + V_LOADS) / NW;   // per wavefront and turn
+  constexpr int KS = HD / 16;                         // k-steps of the first product
+  constexpr int DB = HD / 32;                         // 32-dim blocks of the output
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  const int entry = tiles[2 * blockIdx.x], first = tiles[2 * blockIdx.x + 1];
+  const int row0 = entries[4 * entry], n_tok = entries[4 * entry + 1], start = entries[4 * entry + 2];
+  const int head = blockIdx.y;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r32 = lane & 31, h = lane >> 5;
+  const int row_end = row0 + n_tok;
+  const int kv_last = start + n_tok - 1;
+  const int kvh = head / (n_head / n_kv);
+  const size_t page_elems = (size_t)2 * n_kv * P * HD;
+  const bf16_t* kpool = pool + (size_t)kvh * P * HD;
+  const bf16_t* vpool = pool + (size_t)(n_kv + kvh) * P * HD;
+  const int* tab = table + (size_t)entry * table_stride;
+
+  // this wavefront: rows w_first .. w_first + WROWS - 1, in column blocks of 32
+  const int w_first = first + wave * WROWS;
+  const int w_rows = max(0, min(WROWS, row_end - w_first));
+  const int w_pos_first = start + (w_first - row0), w_pos_last = w_pos_first + w_rows - 1;
+  const int w_lo = (window > 0 && w_pos_first - window + 1 > 0) ? w_pos_first - window + 1 : 0;
+  // the workgroup: rows first .. first + 127
+  const int g_rows = min(PF_ROWS, row_end - first);
+  const int g_pos_first = start + (first - row0), g_pos_last = g_pos_first + g_rows - 1;
+  const int g_lo = (window > 0 && g_pos_first - window + 1 > 0) ? g_pos_first - window + 1 : 0;
+
+  // scores are kept in units of log 2: softmax weights are then bare exp2
+  const float scale2 = scale * 1.4426950408889634f;
+
+  v4u qf[CB][KS];
+  int my_pos[CB];
+  bool col_ok[CB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) {
+    const int row = w_first + cb * 32 + r32;
+    col_ok[cb] = row < row_end;
+    my_pos[cb] = start + (row - row0);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[cb][ks] = v4u{0, 0, 0, 0};
+      if (col_ok[cb]) {
+        const uint4 t = *reinterpret_cast<const uint4*>(q + ((size_t)row * n_head + head) * HD + ks * 16 + h * 8);
+        qf[cb][ks] = v4u{t.x, t.y, t.z, t.w};
+      }
+    }
+  }
+  float mx[CB], l[CB];
+  floatx16 o[CB][DB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) {
+    mx[cb] = -INFINITY;
+    l[cb] = 0.f;
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[cb][d][i] = 0.f;
+  }
+
+  // what this lane fetches in each of its loads of a turn
+  //  K load g: LDS rows K_ROWS g .. + K_ROWS - 1; lane i -> row r = K_ROWS g + i / NP, slot c = i % NP,
+  //            holds piece c ^ (r & (NP - 1)) of key 16 (r / 16) + swap23(r % 16)
+  //  V load g: dims 16 g .. 16 g + 15, 64 bytes each; lane i -> dim d = 16 g + i / 4, slot c = i % 4,
+  //            holds piece c ^ ((d >> 2) & 3): keys 16 (piece / 2) + 8 (piece % 2) .. + 7
+  // packed per load: (element offset inside the page, without the row of the block's first
+  // key) * 2 + (which 16-key block of the turn).  Loads j < MY_K are K loads.
+  int ld_desc[MY_LOADS];
+#pragma unroll
+  for (int j = 0; j < MY_LOADS; ++j) {
+    if (j < MY_K) {
+      const int g = wave + NW * j;
+      const int r = K_ROWS * g + lane / NP, c = lane % NP;
+      const int r16 = r & 15;
+      const int key16 = ((r16 & 4) << 1) | ((r16 & 8) >> 1) | (r16 & 3);
+      ld_desc[j] = (key16 * HD + (c ^ (r & (NP - 1))) * 8) * 2 + (r >> 4);
+    } else {
+      const int gv = wave + NW * (j - MY_K);
+      const int d = 16 * gv + (lane >> 2), c = lane & 3;
+      const int piece = c ^ ((d >> 2) & 3);
+      ld_desc[j] = (d * P + (piece & 1) * 8) * 2 + (piece >> 1);
+    }
+  }
+
+  const unsigned lds0 = (unsigned)(size_t)smem;
+  // LDS addresses of this lane's fragments (without stage and k-step)
+  const unsigned k_row = lds0 + r32 * (HD * 2);                     // K row r32
+  const unsigned v_row = lds0 + K_BYTES + r32 * 64;                 // V^T row (dim) r32 of a 32-dim block
+
+  const int blk_lo = (g_lo / PF_KEYS) * 2, blk_hi = g_pos_last / 16;   // 16-key blocks, starting on a turn
+  const int v_limit = min(kv_last, blk_hi * 16 + 15);               // last key whose value row is real
+  int turn_count = 0;                                               // turns so far: picks the stage
+  for (int c0 = blk_lo; c0 <= blk_hi; c0 += 64) {
+    const int nblk = min(64, blk_hi + 1 - c0);
+    const int n_turns = (nblk + 1) / 2;
+    // the page ids of this run's blocks, one per lane; blocks past the end repeat page 0
+    int ids = (lane < nblk) ? tab[((c0 + lane) * 16) / P] : 0;
+    if (ids < 0) ids = 0;                                           // given back: all its keys are masked
+    auto issue = [&](int t) {
+      const unsigned stage = lds0 + ((turn_count + t) % PF_STAGES) * STAGE;
+      const int pa = __builtin_amdgcn_readlane(ids, min(2 * t, 63));
+      const int pb = __builtin_amdgcn_readlane(ids, min(2 * t + 1, 63));
+      const int key0 = (c0 + 2 * t) * 16;
+#pragma unroll
+      for (int j = 0; j < MY_LOADS; ++j) {
+        const int blk = ld_desc[j] & 1, off = ld_desc[j] >> 1;
+        const int page = blk ? pb : pa;
+        const int prow = (key0 + 16 * blk) % P;                    // row of the block's first key in its page
+        const bf16_t* src;
+        unsigned dst;
+        if (j < MY_K) {
+          src = kpool + (size_t)page * page_elems + (size_t)prow * HD + off;
+          dst = (wave + NW * j) * 1024;
+        } else {
+          src = vpool + (size_t)page * page_elems + off + prow;
+          dst = K_BYTES + (wave + NW * (j - MY_K)) * 1024;
+        }
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)(size_t)(stage + dst), 16, 0, 0);
+      }
+    };
+    constexpr int AHEAD = PF_STAGES - 1;
+#pragma unroll
+    for (int t = 0; t < AHEAD; ++t)
+      if (t < n_turns) issue(t);
+    for (int t = 0; t < n_turns; ++t) {
+      // turn t has landed: only the turns issued after it (at most AHEAD - 1) may be outstanding
+      vm_wait_turns<MY_LOADS>(min(AHEAD - 1, n_turns - 1 - t));
+      __builtin_amdgcn_s_barrier();
+      if (t + AHEAD < n_turns) issue(t + AHEAD);                   // into the stage that turn t - 1 has left
+      const int key0 = (c0 + 2 * t) * 16;
+      // nothing of this turn is visible to this wavefront: it only helps loading
+      if (w_rows == 0 || key0 > w_pos_last || key0 + PF_KEYS - 1 < w_lo) continue;
+      const unsigned st = ((turn_count + t) % PF_STAGES) * STAGE;
+
+      // ---- the fragments of both tiles: keys now, values right behind them
+      v4u kf[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const unsigned a = k_row + st + (((ks * 2 + h) ^ (r32 & (NP - 1))) << 4);
+        asm volatile("ds_read_b128 %0, %1" : "=v"(kf[ks]) : "v"(a));
+      }
+      // ---- S^T = K . Q^T, one column block after the other, so that the softmax of a
+      //      block can run while the matrix core is busy with the next one
+      floatx16 sc[CB];
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[cb][i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          if (cb == 0) {
+            lgkm_wait(KS - 1 - ks);        // the first ks + 1 of the KS reads have arrived
+            asm volatile("" : "+v"(kf[ks]));
+          }
+          sc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[ks]),
+                                                           __builtin_bit_cast(bf16x8, qf[cb][ks]), sc[cb], 0, 0, 0);
+        }
+      }
+      // the value fragments are asked for now and waited for after the softmax
+      v4u vf[DB][2];
+#pragma unroll
+      for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+          const unsigned a = v_row + st + d * 32 * 64 + (((tt * 2 + h) ^ ((r32 >> 2) & 3)) << 4);
+          asm volatile("ds_read_b128 %0, %1" : "=v"(vf[d][tt]) : "v"(a));
+        }
+
+      // ---- masks and the online softmax, per column block
+      // element i of a lane: key key0 + 16 (i / 8) + 8 h + 4 ((i / 4) % 2) + i % 4
+      const bool plain = (key0 + PF_KEYS - 1 <= w_pos_first) && (w_rows == WROWS) &&
+                         (window <= 0 || key0 >= w_pos_last - window + 1);
+      v4u pf[CB][2];
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+        float sv[16];
+        if (plain) {                       // the same in every lane: no compare at all
+#pragma unroll
+          for (int i = 0; i < 16; ++i) sv[i] = sc[cb][i] * scale2;
+        } else {
+          const int hi = col_ok[cb] ? my_pos[cb] : -1;
+          const int lo = (window > 0) ? my_pos[cb] - window + 1 : 0;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = key0 + 16 * (i >> 3) + 8 * h + 4 * ((i >> 2) & 1) + (i & 3);
+            const bool see = (key <= hi) & (key >= lo);      // bitwise on purpose: selects, no branches
+            sv[i] = see ? sc[cb][i] * scale2 : -INFINITY;
+          }
+        }
+        float bm = sv[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) bm = fmaxf(bm, sv[i]);
+        bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+        const float m_new = fmaxf(mx[cb], bm);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        float ps = 0.f;
+        float pv[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          pv[i] = __builtin_amdgcn_exp2f(sv[i] - m_safe);
+          ps += pv[i];
+        }
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+          pf[cb][tt] = v4u{pack_bf16x2(pv[8 * tt], pv[8 * tt + 1]), pack_bf16x2(pv[8 * tt + 2], pv[8 * tt + 3]),
+                           pack_bf16x2(pv[8 * tt + 4], pv[8 * tt + 5]), pack_bf16x2(pv[8 * tt + 6], pv[8 * tt + 7])};
+        // the running maximum settles after a few turns; then nothing needs rescaling
+        if (__builtin_amdgcn_ballot_w64(m_new != mx[cb]) != 0) {
+          const float alpha = __builtin_amdgcn_exp2f(mx[cb] - m_safe);
+          l[cb] *= alpha;
+#pragma unroll
+          for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[cb][d][i] *= alpha;
+          mx[cb] = m_new;
+        }
+        l[cb] += ps;
+      }
+
+      // ---- O^T += V^T . P^T
+      lgkm_wait(0);
+#pragma unroll
+      for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) asm volatile("" : "+v"(vf[d][tt]));
+      if (key0 + PF_KEYS - 1 > v_limit || key0 < g_lo) {
+        // rows never written, and the stand-in page read for a block that was given back or
+        // lies past the end, may hold anything, NaN included, and 0 * NaN is NaN
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const int key = key0 + 16 * tt + 8 * h + e;
+              const bool drop = (key > v_limit) | (key < g_lo);
+              const unsigned keep = drop ? ((e & 1) ? 0x0000FFFFu : 0xFFFF0000u) : 0xFFFFFFFFu;
+              vf[d][tt][e >> 1] &= keep;
+            }
+      }
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt)
+            o[cb][d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[d][tt]),
+                                                               __builtin_bit_cast(bf16x8, pf[cb][tt]), o[cb][d],
+                                                               0, 0, 0);
+    }
+    turn_count += n_turns;
+    // every wavefront is done with this run's stages before the next run refills them
+    __builtin_amdgcn_s_barrier();
+  }
+
+  // o[cb][d][i]: dim 32 d + 8 (i / 4) + 4 h + i % 4 of token (column) r32 of block cb
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) {
+    const float lt = l[cb] + __shfl_xor(l[cb], 32, 64);
+    if (!col_ok[cb]) continue;
+    const float inv = 1.0f / lt;
+    const int row = w_first + cb * 32 + r32;
+    bf16_t* dst = out + ((size_t)row * n_head + head) * HD;
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const uint2 r = make_uint2(pack_bf16x2(o[cb][d][4 * g4] * inv, o[cb][d][4 * g4 + 1] * inv),
+                                   pack_bf16x2(o[cb][d][4 * g4 + 2] * inv, o[cb][d][4 * g4 + 3] * inv));
+        *reinterpret_cast<uint2*>(dst + 32 * d + 8 * g4 + 4 * h) = r;
+      }
+  }
+}
+
 // ------------------------------------------------------------------ dispatch
 static int check_common(const char* what, int n_head, int n_kv, int hd, int P, int table_stride) {
   if (!(hd == 32 || hd == 64 || hd == 128)) {
@@ -468,7 +811,12 @@ extern "C" int ti_attention_decode_bf16(const void* q, const void* pool, const i
   return 0;
 }
 
-// Portions of prompts.  tiles: int [n_tiles, 2] = (entry, first row), each tile 64 rows;
+static int g_prefill_lds = 1;
+// 1: head sizes 64 and 128 take the kernel that shares keys and values through LDS
+// (default); 0: every head size takes the kernel that reads them per wavefront
+extern "C" void ti_attention_prefill_use_lds(int on) { g_prefill_lds = on; }
+
+// Portions of prompts.  tiles: int [n_tiles, 2] = (entry, first row), each tile 128 rows;
 // entries: int [n_entries, 4] = (row0, n_tokens, start_pos, -); table row e belongs to entry e.
 extern "C" int ti_attention_prefill_bf16(const void* q, const void* pool, const int* table, int table_stride,
                                          const int* tiles, const int* entries, void* out, int n_tiles,
@@ -479,9 +827,35 @@ extern "C" int ti_attention_prefill_bf16(const void* q, const void* pool, const 
   TI_REQUIRE(n_head <= 65535, "attention_prefill: too many heads");
   if (n_tiles == 0) return 0;
   dim3 grid(n_tiles, n_head);
+  if (g_prefill_lds && (hd == 64 || hd == 128)) {
+    const int lds = PF_STAGES * 2 * PF_KEYS * hd * 2;
+    static bool ready = false;          // allow more than 64 KiB of dynamic LDS, once
+    if (!ready) {
+      if (hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<128, 1>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              PF_STAGES * 2 * PF_KEYS * 128 * 2) != hipSuccess ||
+          hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<64, 1>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              PF_STAGES * 2 * PF_KEYS * 64 * 2) != hipSuccess) {
+        ti_set_error("attention_prefill: cannot reserve %d bytes of LDS", lds);
+        return 2;
+      }
+      ready = true;
+    }
+    if (hd == 128)
+      attn_prefill_lds_kernel<128, 1><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,
+                                                                  table_stride, tiles, entries, (bf16_t*)out,
+                                                                  n_head, n_kv, page_size, scale, window);
+    else
+      attn_prefill_lds_kernel<64, 1><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,
+                                                                 table_stride, tiles, entries, (bf16_t*)out,
+                                                                 n_head, n_kv, page_size, scale, window);
+    TI_LAUNCH_CHECK();
+    return 0;
+  }
 #define TI_PRE(H)                                                                                          \
   case H:                                                                                                  \
-    attn_prefill_kernel<H><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,          \
+    attn_prefill_kernel<H><<<grid, 512, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,          \
                                                      table_stride, tiles, entries, (bf16_t*)out, n_head,    \
                                                      n_kv, page_size, scale, window);                       \
     break;

@@ -28,6 +28,12 @@ FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-shared",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]
 HEADERS = ["common.h"]
+# flags of single libraries.  The attention kernels rescale their MFMA accumulators with
+# vector instructions; kept in the accumulation registers they would be copied out and back
+# on every turn of the loop, so their MFMAs are told to work on ordinary vector registers.
+EXTRA_FLAGS: Dict[str, List[str]] = {
+    "attention_bf16": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
 
 # library name -> source file
 SOURCES: Dict[str, str] = {
@@ -57,7 +63,7 @@ def _digest(name: str) -> str:
     for f in [SOURCES[name]] + HEADERS:
         with open(os.path.join(HERE, f), "rb") as fh:
             h.update(fh.read())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + EXTRA_FLAGS.get(name, [])).encode())
     return h.hexdigest()[:12]
 
 
@@ -108,7 +114,7 @@ def _compile(name: str, out_dir: str) -> str:
         env["HOME"] = tempfile.gettempdir()
     t0 = time.time()
     _say(f"compiling {SOURCES[name]} for {ARCH} ...")
-    proc = subprocess.run([_hipcc()] + FLAGS + [src, "-o", part], cwd=HERE, env=env,
+    proc = subprocess.run([_hipcc()] + FLAGS + EXTRA_FLAGS.get(name, []) + [src, "-o", part], cwd=HERE, env=env,
                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if proc.returncode != 0:
         if os.path.exists(part):

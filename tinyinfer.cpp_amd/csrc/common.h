@@ -24,10 +24,19 @@ __device__ __forceinline__ float bf2f(bf16_t v) { return __uint_as_float(((uint3
 
 // round to nearest, ties to even; NaN stays NaN
 __device__ __forceinline__ bf16_t f2bf(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  const uint32_t u = __float_as_uint(f);
+  const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  const uint32_t quiet = (u >> 16) | 0x40u;
+  return (bf16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? quiet : rounded);   // a select, not a branch
+}
+
+// two floats -> two bfloat16 in one word (first in the low half), round to nearest even:
+// gfx950 has an instruction for it (v_cvt_pk_bf16_f32)
+typedef float ti_float2v __attribute__((ext_vector_type(2)));
+typedef __bf16 ti_bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  const ti_float2v v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, ti_bf16x2));
 }
 
 template <typename T> __device__ __forceinline__ float ld(const T* p);

@@ -24,7 +24,7 @@ from ..models.model import Model
 from ..ops.kernels import get_ops
 from ..weights.loader import DTYPES
 
-PREFILL_TILE_Q = 64     # query rows per work item of the tiled attention kernels
+PREFILL_TILE_Q = 128    # query rows per work item of the tiled attention kernels
 
 
 class EngineError(RuntimeError):
