@@ -171,6 +171,27 @@ def test_cuts_agree_bitwise_in_float32(model_folders):
         assert np.array_equal(results[0][r], results[2][r]), r
 
 
+def test_norm_inside_the_product_changes_no_bit(model_folders):
+    """Steps of few tokens run the norm before a projection inside the projection's
+    kernel.  With that switched off the same steps give the same bits."""
+    from tinyinfer_amd.ops.kernels import get_ops
+    folder = model_folders("A", "bfloat16")
+    requests = {r: t for r, t in make_requests(CONFIGS["A"]["vocab_size"]).items() if r in ("a", "b")}
+    trace = traces.tail_one_by_one(requests, 32)
+    ops = get_ops()
+    results = []
+    try:
+        for fused in (True, False):
+            ops.use_fused_norm = fused
+            engine = build_engine(folder, "bfloat16", traces.max_tokens(trace))
+            assert engine.ops.can_fuse_norm(1, torch.bfloat16) == fused
+            results.append(replay(engine, trace))
+    finally:
+        ops.use_fused_norm = True
+    for r in requests:
+        assert np.array_equal(results[0][r], results[1][r]), r
+
+
 def test_step_refuses_what_it_cannot_run(model_folders):
     from tinyinfer_amd.engine import StepEntry, EngineError
     from tinyinfer_amd.cache import OutOfPages

@@ -457,6 +457,83 @@ def test_linear_bf16_rows_do_not_depend_on_the_batch(ops):
         assert torch.equal(one[0], small[m])
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 48, 1024), (7, 1000, 1096), (40, 130, 2048), (64, 2048, 1032)])
+def test_linear_bf16_few_columns_many_wavefronts(ops, M, N, K):
+    """Few output columns and a long K: the skinny kernel runs with eight wavefronts
+    that split K.  Same result as float64, and a row alone has the bits it has in a batch."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    g = torch.Generator().manual_seed(M + N)
+    a = (torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16)
+    w = (torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16)
+    ref = ref_linear(a, w)
+    base = torch.randn(M, N, generator=g)
+    out = dev(base.clone())
+    ops.linear(dev(a), dev(w), out, "add")
+    assert (f64(out) - (ref + f64(base))).abs().max() < 2e-5 * K
+    full = torch.empty(M, N, device="cuda")
+    ops.linear(dev(a), dev(w), full, "store")
+    one = torch.empty(1, N, device="cuda")
+    m = M - 1
+    ops.linear(dev(a[m:m + 1].contiguous()), dev(w), one, "store")
+    assert torch.equal(one[0], full[m])
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 48, 64), (5, 261, 1024), (16, 40, 192), (3, 130, 1280), (8, 64, 2304),
+                                   (2, 18, 4096)])
+def test_linear_with_the_norm_inside(ops, M, N, K):
+    """rmsnorm and product in one kernel (few tokens) give the bits of the norm kernel
+    followed by the product kernel, for every epilogue; and both agree with float64."""
+    from tinyinfer_amd.ops.kernels import NormedRows
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    g = torch.Generator().manual_seed(M * 3 + N)
+    x = dev(torch.randn(M, K, generator=g) * 3.0)
+    nw = dev(1 + 0.1 * torch.randn(K, generator=g))
+    w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    eps = 1e-3
+    h = torch.empty(M, K, device="cuda", dtype=torch.bfloat16)
+    ops.rmsnorm(x, nw, eps, h)
+    xd = f64(x)
+    ref = f64((xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + eps) * f64(nw)).to(torch.bfloat16)) @ f64(w).T
+    assert ops.can_fuse_norm(M, torch.bfloat16)
+    for epi, dt in (("store", torch.float32), ("add", torch.float32), ("store_act", torch.bfloat16),
+                    ("swiglu", torch.bfloat16)):
+        if epi == "swiglu" and N % 2:
+            continue
+        cols = N // 2 if epi == "swiglu" else N
+        base = torch.randn(M, cols, generator=g).to(dt)
+        two, one = dev(base.clone()), dev(base.clone())
+        ops.linear(h, w, two, epi)
+        lazy = NormedRows(x, nw, eps, torch.empty_like(h))
+        assert ops._linear_normed(lazy, w, one, epi), "the fused kernel refused a size it should serve"
+        assert torch.equal(one, two), epi
+        if epi == "store":
+            # the norm kernel rounds its rows exactly where the float64 reference does, up to
+            # a last bit of the 32-bit scale: allow one bfloat16 step on a few operands
+            assert (f64(one) - ref).abs().max() < 2e-5 * K + 0.01 * ref.abs().max()
+
+
+def test_linear_with_the_norm_inside_refuses_what_it_does_not_serve(ops):
+    """More rows than the kernel holds, or a K that is no multiple of 64: `linear` computes
+    the norm first and the result is still right."""
+    from tinyinfer_amd.ops.kernels import NormedRows
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    g = torch.Generator().manual_seed(9)
+    for M, N, K in ((17, 32, 128), (4, 32, 72)):
+        x = dev(torch.randn(M, K, generator=g))
+        nw = dev(1 + 0.1 * torch.randn(K, generator=g))
+        w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+        h = torch.empty(M, K, device="cuda", dtype=torch.bfloat16)
+        ops.rmsnorm(x, nw, 1e-6, h)
+        two = torch.empty(M, N, device="cuda")
+        ops.linear(h, w, two, "store")
+        one = torch.empty(M, N, device="cuda")
+        ops.linear(NormedRows(x, nw, 1e-6, torch.empty_like(h)), w, one, "store")
+        assert torch.equal(one, two)
+
+
 # ---------------------------------------------- bfloat16 matrix-core attention
 class FakeCtx:
     """The fields of a step context that the attention dispatch reads."""

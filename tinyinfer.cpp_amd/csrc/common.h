@@ -59,6 +59,19 @@ template <int WIDTH> __device__ __forceinline__ float group_max(float v) {
   return v;
 }
 
+// The RMSNorm of a row by one wavefront, in pieces of four floats: lane l holds the pieces
+// l, l + 64, ...  Every kernel that norms a row this way goes through these two functions,
+// so they all produce the same bits.
+__device__ __forceinline__ float rms_accumulate(float acc, float4 v) {
+  acc = fmaf(v.x, v.x, acc);
+  acc = fmaf(v.y, v.y, acc);
+  acc = fmaf(v.z, v.z, acc);
+  return fmaf(v.w, v.w, acc);
+}
+__device__ __forceinline__ float rms_scale(float lane_acc, int width, float eps) {
+  return 1.0f / sqrtf(group_sum<TI_WAVE>(lane_acc) / (float)width + eps);
+}
+
 // sum over a workgroup of NT threads (NT multiple of 64, <= 1024); `red` holds
 // NT/64 floats of LDS.  Every thread gets the total.  Fixed order: deterministic.
 template <int NT> __device__ __forceinline__ float block_sum(float v, float* red) {

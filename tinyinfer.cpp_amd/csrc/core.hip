@@ -55,10 +55,42 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
   for (int i = threadIdx.x; i < H; i += 256) st<T>(dst + i, src[i] * scale * w[i]);
 }
 
+// the same for widths that are multiples of four: a wavefront per row, four rows a workgroup
+template <typename T>
+__global__ void __launch_bounds__(256)
+rmsnorm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w, const int* __restrict__ rows,
+                    T* __restrict__ out, int n_rows, int H, float eps) {
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (r >= n_rows) return;
+  const float* src = x + (size_t)(rows ? rows[r] : r) * H;
+  float ss = 0.f;
+  for (int k = lane * 4; k < H; k += 256) ss = rms_accumulate(ss, *reinterpret_cast<const float4*>(src + k));
+  const float scale = rms_scale(ss, H, eps);
+  T* dst = out + (size_t)r * H;
+  for (int k = lane * 4; k < H; k += 256) {
+    const float4 v = *reinterpret_cast<const float4*>(src + k);
+    const float4 g = *reinterpret_cast<const float4*>(w + k);
+    st<T>(dst + k, v.x * scale * g.x);
+    st<T>(dst + k + 1, v.y * scale * g.y);
+    st<T>(dst + k + 2, v.z * scale * g.z);
+    st<T>(dst + k + 3, v.w * scale * g.w);
+  }
+}
+
 extern "C" int ti_rmsnorm(int out_dtype, const float* x, const float* w, const int* rows, void* out,
                           int n_rows, int H, float eps, hipStream_t stream) {
   TI_REQUIRE(n_rows >= 0 && H > 0, "rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
+  TI_REQUIRE(out_dtype == TI_F32 || out_dtype == TI_BF16, "rmsnorm: unknown dtype %d", out_dtype);
   if (n_rows == 0) return 0;
+  if (H % 4 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0) {
+    const int grid = (n_rows + 3) / 4;
+    if (out_dtype == TI_F32)
+      rmsnorm_wave_kernel<float><<<grid, 256, 0, stream>>>(x, w, rows, (float*)out, n_rows, H, eps);
+    else
+      rmsnorm_wave_kernel<bf16_t><<<grid, 256, 0, stream>>>(x, w, rows, (bf16_t*)out, n_rows, H, eps);
+    TI_LAUNCH_CHECK();
+    return 0;
+  }
   if (out_dtype == TI_F32)
     rmsnorm_kernel<float><<<n_rows, 256, 0, stream>>>(x, w, rows, (float*)out, H, eps);
   else if (out_dtype == TI_BF16)

@@ -35,13 +35,14 @@ __device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *reinterpret_cas
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
 
 // ============================================================== skinny kernel
-// grid.x = ceil(N / 16) (SwiGLU: ceil(F / 8): 8 gate rows and their 8 up rows)
-template <int MT, int EPI>
-__global__ void __launch_bounds__(256)
+// grid.x = ceil(N / 16) (SwiGLU: ceil(F / 8): 8 gate rows and their 8 up rows).
+// NW wavefronts split K between them.
+template <int MT, int EPI, int NW = 4>
+__global__ void __launch_bounds__(NW * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_,
                    int M, int N, int K, long lda) {
   constexpr bool SW = (EPI == TI_EPI_SWIGLU);
-  __shared__ float red[4][MT][16][17];
+  __shared__ float red[NW][MT][16][17];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, j = lane >> 4;   // MFMA row / column, and k group
   const int rows_total = SW ? 2 * N : N;
@@ -72,22 +73,24 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, v
   // chunk c covers k in [64 c, 64 c + 64); lane group j takes [64 c + 16 j, +16)
   const int chunks = (K + 63) / 64;
   constexpr int UN = 4;
-  for (int c0 = wave; c0 < chunks; c0 += 4 * UN) {
+  for (int c0 = wave; c0 < chunks; c0 += NW * UN) {
     Frag w0[UN], w1[UN];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int k = (c0 + 4 * u) * 64 + j * 16;
-      w0[u].u = (k + 8 <= K) ? ld16(wp + (size_t)(c0 + 4 * u) * 64) : zero;
-      w1[u].u = (k + 16 <= K) ? ld16(wp + (size_t)(c0 + 4 * u) * 64 + 8) : zero;
+      const int k = (c0 + NW * u) * 64 + j * 16;
+      const bool mine = c0 + NW * u < chunks;
+      w0[u].u = (mine && k + 8 <= K) ? ld16(wp + (size_t)(c0 + NW * u) * 64) : zero;
+      w1[u].u = (mine && k + 16 <= K) ? ld16(wp + (size_t)(c0 + NW * u) * 64 + 8) : zero;
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int k = (c0 + 4 * u) * 64 + j * 16;
+      const int k = (c0 + NW * u) * 64 + j * 16;
+      const bool mine = c0 + NW * u < chunks;
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         Frag a0, a1;
-        a0.u = (aok[t] && k + 8 <= K) ? ld16(ap[t] + (size_t)(c0 + 4 * u) * 64) : zero;
-        a1.u = (aok[t] && k + 16 <= K) ? ld16(ap[t] + (size_t)(c0 + 4 * u) * 64 + 8) : zero;
+        a0.u = (mine && aok[t] && k + 8 <= K) ? ld16(ap[t] + (size_t)(c0 + NW * u) * 64) : zero;
+        a1.u = (mine && aok[t] && k + 16 <= K) ? ld16(ap[t] + (size_t)(c0 + NW * u) * 64 + 8) : zero;
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u].v, a0.v, acc[t], 0, 0, 0);
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, a1.v, acc[t], 0, 0, 0);
       }
@@ -100,6 +103,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, v
     for (int i = 0; i < 4; ++i) red[wave][t][r][4 * j + i] = acc[t][i];
   __syncthreads();
   // thread -> (token = tid / 16, row = tid % 16): consecutive threads, consecutive columns
+  if (NW > 4 && threadIdx.x >= 256) return;
   const int tok = threadIdx.x >> 4, row = threadIdx.x & 15;
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -111,7 +115,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, v
       if (n >= N) continue;
       float g = 0.f, u = 0.f;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
+      for (int w = 0; w < NW; ++w) {
         g += red[w][t][tok][row];
         u += red[w][t][tok][row + 8];
       }
@@ -121,12 +125,140 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, v
       if (n >= N) continue;
       float s = 0.f;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) s += red[w][t][tok][row];
+      for (int w = 0; w < NW; ++w) s += red[w][t][tok][row];
       const size_t o = (size_t)m * N + n;
       if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = s;
       if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] += s;
       if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(s);
     }
+  }
+}
+
+// ============================================= skinny kernel with an RMSNorm in front
+// out = rmsnorm(x; nw, eps) W^T for M <= 16 tokens.  The norm that stands before a
+// projection is computed by every workgroup for itself: the rows are few and lie in the
+// cache, the first weight loads are already under way while it runs, and it costs no
+// launch of its own.  x: float [M, K]; nw: norm weight [K].  The normed rows go to LDS as
+// bfloat16 (the rounding every product operand gets, so the result equals that of the
+// norm kernel followed by the plain product) and the main loop reads its token fragments
+// from there.  KC: float4 pieces of a row each lane holds (K <= 256 KC).
+template <int EPI, int KC, int NW>
+__global__ void __launch_bounds__(NW * 64)
+gemm_skinny_normed_kernel(const float* __restrict__ X, const float* __restrict__ Gw, float eps,
+                          const bf16_t* __restrict__ W, void* __restrict__ out_, int M, int N, int K) {
+  constexpr bool SW = (EPI == TI_EPI_SWIGLU);
+  extern __shared__ __attribute__((aligned(16))) unsigned char dyn_smem[];
+  bf16_t* sA = reinterpret_cast<bf16_t*>(dyn_smem);          // [M][K + 8]
+  __shared__ float red[NW][16][17];
+  const int lda = K + 8;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 15, j = lane >> 4;
+  int wrow;
+  if (SW) {
+    const int n = blockIdx.x * 8 + (r & 7);
+    wrow = (r < 8 ? 0 : N) + (n < N ? n : N - 1);
+  } else {
+    const int n = blockIdx.x * 16 + r;
+    wrow = n < N ? n : N - 1;
+  }
+  const bf16_t* wp = W + (size_t)wrow * K + j * 16;
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  const int chunks = K / 64;
+  constexpr int UN = 4;
+
+  // the first weights of this wavefront: on their way while the norm is computed
+  Frag w0[UN], w1[UN];
+#pragma unroll
+  for (int u = 0; u < UN; ++u) {
+    const bool mine = wave + NW * u < chunks;
+    w0[u].u = mine ? ld16(wp + (size_t)(wave + NW * u) * 64) : zero;
+    w1[u].u = mine ? ld16(wp + (size_t)(wave + NW * u) * 64 + 8) : zero;
+  }
+
+  // ---- the norm: wavefront w takes rows w, w + NW, ...; a lane holds KC float4 of a row
+  float4 g[KC];
+#pragma unroll
+  for (int c = 0; c < KC; ++c) {
+    const int k = lane * 4 + 256 * c;
+    g[c] = k < K ? *reinterpret_cast<const float4*>(Gw + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+#pragma unroll
+  for (int rr = 0; rr < 16 / NW; ++rr) {
+    const int m = wave + NW * rr;
+    if (m >= M) break;
+    const float* xr = X + (size_t)m * K;
+    float4 v[KC];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int k = lane * 4 + 256 * c;
+      v[c] = k < K ? *reinterpret_cast<const float4*>(xr + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int c = 0; c < KC; ++c)
+      if (lane * 4 + 256 * c < K) ss = rms_accumulate(ss, v[c]);
+    const float scale = rms_scale(ss, K, eps);
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int k = lane * 4 + 256 * c;
+      if (k < K) {
+        const uint2 hb = make_uint2(pack_bf16x2(v[c].x * scale * g[c].x, v[c].y * scale * g[c].y),
+                                    pack_bf16x2(v[c].z * scale * g[c].z, v[c].w * scale * g[c].w));
+        *reinterpret_cast<uint2*>(sA + (size_t)m * lda + k) = hb;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- the product, as in the plain skinny kernel with the token fragments from LDS
+  const bool aok = r < M;
+  const bf16_t* ap = sA + (size_t)(aok ? r : 0) * lda + j * 16;
+  floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int c0 = wave; c0 < chunks; c0 += NW * UN) {
+    if (c0 != wave) {
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const bool mine = c0 + NW * u < chunks;
+        w0[u].u = mine ? ld16(wp + (size_t)(c0 + NW * u) * 64) : zero;
+        w1[u].u = mine ? ld16(wp + (size_t)(c0 + NW * u) * 64 + 8) : zero;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const bool mine = aok && (c0 + NW * u < chunks);
+      Frag a0, a1;
+      a0.u = mine ? ld16(ap + (size_t)(c0 + NW * u) * 64) : zero;
+      a1.u = mine ? ld16(ap + (size_t)(c0 + NW * u) * 64 + 8) : zero;
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u].v, a0.v, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, a1.v, acc, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) red[wave][r][4 * j + i] = acc[i];
+  __syncthreads();
+  const int tok = threadIdx.x >> 4, row = threadIdx.x & 15;   // tok >= 16 for the wavefronts beyond four
+  if (tok >= M) return;
+  if (SW) {
+    if (row >= 8) return;
+    const int n = blockIdx.x * 8 + row;
+    if (n >= N) return;
+    float gt = 0.f, up = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      gt += red[w][tok][row];
+      up += red[w][tok][row + 8];
+    }
+    ((bf16_t*)out_)[(size_t)tok * N + n] = f2bf(silu_mul(gt, up));
+  } else {
+    const int n = blockIdx.x * 16 + row;
+    if (n >= N) return;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) sum += red[w][tok][row];
+    const size_t o = (size_t)tok * N + n;
+    if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = sum;
+    if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] += sum;
+    if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(sum);
   }
 }
 
@@ -476,15 +608,32 @@ static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M,
 }
 
 // ------------------------------------------------------------------- dispatch
+// Wavefronts per workgroup of the skinny kernel (4 or 8).  A product with few output columns
+// has few workgroups (one per 16 columns); more wavefronts in each, splitting K further, keep
+// more loads in flight.  0 = choose by the shape.
+static int g_skinny_waves = 0;
+extern "C" void ti_gemm_bf16_skinny_waves(int waves) { g_skinny_waves = waves; }
+
 template <int EPI>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
                           hipStream_t s) {
   const int grid = (EPI == TI_EPI_SWIGLU) ? (N + 7) / 8 : (N + 15) / 16;
   const int mt = (M + 15) / 16;
-  if (mt == 1) gemm_skinny_kernel<1, EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
-  if (mt == 2) gemm_skinny_kernel<2, EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
-  if (mt == 3) gemm_skinny_kernel<3, EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
-  if (mt == 4) gemm_skinny_kernel<4, EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
+  int waves = g_skinny_waves;
+  // by the weight's shape only, so that a row's bits do not depend on the rows beside it
+  if (waves == 0) waves = (grid <= 128 && K >= 1024) ? 8 : 4;
+#define TI_SKINNY(MTV)                                                               \
+  if (mt == MTV) {                                                                   \
+    if (waves == 8)                                                                  \
+      gemm_skinny_kernel<MTV, EPI, 8><<<grid, 512, 0, s>>>(A, W, out, M, N, K, lda); \
+    else                                                                             \
+      gemm_skinny_kernel<MTV, EPI, 4><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda); \
+  }
+  TI_SKINNY(1)
+  TI_SKINNY(2)
+  TI_SKINNY(3)
+  TI_SKINNY(4)
+#undef TI_SKINNY
 }
 
 template <int EPI>
@@ -493,6 +642,57 @@ static void launch_tiled(const bf16_t* A, const bf16_t* W, void* out, int M, int
   const int bn = (EPI == TI_EPI_SWIGLU) ? TBN / 2 : TBN;
   dim3 grid((N + bn - 1) / bn, (M + TBM - 1) / TBM);
   gemm_tiled_kernel<EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
+}
+
+// out = rmsnorm(x; nw, eps) W^T for M <= 16 (see gemm_skinny_normed_kernel).  Returns 3 for
+// sizes it does not serve (M > 16, K not a multiple of 64 or above 4096).
+extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, const void* W, void* out,
+                                   int M, int N, int K, int epi, hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16_normed: bad sizes M=%d N=%d K=%d", M, N, K);
+  if (M > 16 || K % 64 != 0 || K > 4096 || ((uintptr_t)W & 15) || ((uintptr_t)x & 15) || ((uintptr_t)nw & 15)) {
+    ti_set_error("gemm_bf16_normed: M=%d K=%d is not served (M <= 16, K %% 64 == 0, K <= 4096)", M, K);
+    return 3;
+  }
+  if (M == 0) return 0;
+  const size_t lds = (size_t)M * (K + 8) * 2;
+  const bf16_t* w = (const bf16_t*)W;
+  const int grid = (epi == TI_EPI_SWIGLU) ? (N + 7) / 8 : (N + 15) / 16;
+  const int kc = (K + 255) / 256;
+  // the same number of wavefronts as the plain skinny kernel takes for this weight: same bits
+  int waves = g_skinny_waves;
+  if (waves == 0) waves = (grid <= 128 && K >= 1024) ? 8 : 4;
+#define TI_GNW(E, KCV, NWV)                                                                                 \
+  {                                                                                                         \
+    auto kern = gemm_skinny_normed_kernel<E, KCV, NWV>;                                                     \
+    if (lds > 48 * 1024)                                                                                    \
+      TI_REQUIRE(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,         \
+                                     (int)lds) == hipSuccess, "gemm_bf16_normed: LDS size refused");        \
+    kern<<<grid, NWV * 64, lds, stream>>>(x, nw, eps, w, out, M, N, K);                                     \
+  }
+#define TI_GNK(E, KCV)                \
+  {                                   \
+    if (waves == 8) TI_GNW(E, KCV, 8) \
+    else TI_GNW(E, KCV, 4)            \
+  }
+#define TI_GN(E)                        \
+  case E:                               \
+    if (kc <= 4) TI_GNK(E, 4)           \
+    else if (kc <= 8) TI_GNK(E, 8)      \
+    else TI_GNK(E, 16)                  \
+    break;
+  switch (epi) {
+    TI_GN(TI_EPI_STORE_F32)
+    TI_GN(TI_EPI_ADD_F32)
+    TI_GN(TI_EPI_STORE_ACT)
+    TI_GN(TI_EPI_SWIGLU)
+    default:
+      TI_REQUIRE(false, "gemm_bf16_normed: unknown epilogue %d", epi);
+  }
+#undef TI_GN
+#undef TI_GNK
+#undef TI_GNW
+  TI_LAUNCH_CHECK();
+  return 0;
 }
 
 static int g_use_pipelined = 1;

@@ -35,6 +35,25 @@ def _ptr(t: Optional[torch.Tensor]):
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
 
+class NormedRows:
+    """rmsnorm(x; weight, eps) that has not been computed yet.  A norm hands this to a
+    consumer that said it can take it; `Ops.linear` accepts it in place of the activation
+    and runs the norm inside the product's kernel where a kernel for that exists, else
+    it computes the rows first (`materialize`)."""
+
+    def __init__(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor):
+        self.x, self.weight, self.eps, self.out = x, weight, eps, out
+        self.shape = out.shape
+        self.dtype = out.dtype
+        self._done = False
+
+    def materialize(self, ops: "Ops") -> torch.Tensor:
+        if not self._done:
+            ops.rmsnorm(self.x, self.weight, self.eps, self.out)
+            self._done = True
+        return self.out
+
+
 class Ops:
     """Loads kernel libraries on first use and exposes one method per op."""
 
@@ -45,6 +64,7 @@ class Ops:
         have = lambda n: os.path.isfile(os.path.join(_build.HERE, _build.SOURCES[n]))
         self.use_fast_gemm = have("gemm_bf16")
         self.use_fast_attention = have("attention_bf16")
+        self.use_fused_norm = True       # the norm before a product inside the product's kernel (few tokens)
 
     # ------------------------------------------------------------------ loading
     def lib(self, name: str) -> ctypes.CDLL:
@@ -172,6 +192,10 @@ class Ops:
         epilogue: "store" f32 out = ; "add" f32 out += ; "store_act" T out = ;
         "swiglu": w is [2F, K] = [gate; up], T out [M, F] = silu(gate) * up."""
         epi = EPI[epilogue]
+        if isinstance(a, NormedRows):
+            if self._linear_normed(a, w, out, epilogue):
+                return
+            a = a.materialize(self)
         M, K = a.shape
         rows = w.shape[0]
         N = rows // 2 if epilogue == "swiglu" else rows
@@ -192,6 +216,37 @@ class Ops:
         rc = lib.ti_gemm_generic(code, _ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi,
                                  self._stream())
         self._check(lib, rc, "linear")
+
+    NORMED_MAX_ROWS = 16
+
+    def can_fuse_norm(self, n_rows: int, dtype: torch.dtype) -> bool:
+        """Whether `linear` has a kernel that takes the norm of this many rows in."""
+        return (self.use_fused_norm and self.use_fast_gemm and dtype == torch.bfloat16
+                and 0 < n_rows <= self.NORMED_MAX_ROWS)
+
+    def _linear_normed(self, a: NormedRows, w, out, epilogue) -> bool:
+        """rmsnorm and product in one kernel; False if no kernel serves the shape."""
+        M, K = a.shape
+        if not self.can_fuse_norm(M, a.dtype) or w.dtype != torch.bfloat16:
+            return False
+        rows = w.shape[0]
+        N = rows // 2 if epilogue == "swiglu" else rows
+        self._dev(a.x, a.weight, w, out)
+        if w.dim() != 2 or w.shape[1] != K or not w.is_contiguous() or (epilogue == "swiglu" and rows % 2):
+            raise KernelError(f"linear: normed rows {tuple(a.shape)} and w {tuple(w.shape)} do not fit")
+        if a.x.shape != (M, K) or a.x.dtype != torch.float32 or not a.x.is_contiguous() \
+                or a.weight.shape != (K,) or a.weight.dtype != torch.float32:
+            raise KernelError("linear: the rows to norm must be float32 [M, K] with a float32 weight [K]")
+        want = torch.float32 if epilogue in ("store", "add") else torch.bfloat16
+        if out.shape != (M, N) or out.dtype != want or not out.is_contiguous():
+            raise KernelError(f"linear[{epilogue}]: out {tuple(out.shape)} {out.dtype} does not fit [{M},{N}] {want}")
+        lib = self.lib("gemm_bf16")
+        rc = lib.ti_gemm_bf16_normed(_ptr(a.x), _ptr(a.weight), ctypes.c_float(a.eps), _ptr(w), _ptr(out),
+                                     M, N, K, EPI[epilogue], self._stream())
+        if rc == 3:
+            return False
+        self._check(lib, rc, "linear(normed)")
+        return True
 
     def _linear_bf16(self, a, w, out, epi, M, N, K) -> bool:
         """The MFMA kernels; False if they refuse the shape (the generic kernel takes it)."""

@@ -23,6 +23,7 @@ from ..spec import TensorNeed, PagedKVNeed
 
 class Attention(Part):
     family = "mixer"
+    takes_lazy_norm = True      # h goes into one product and nowhere else
 
     def __init__(self, prefix: str, hidden: int, heads: int, kv_heads: int, head_dim: int,
                  qk_norm: bool = True, eps: float = 1e-6, window: Optional[int] = None,

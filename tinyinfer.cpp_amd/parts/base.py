@@ -14,6 +14,12 @@ Interfaces by family (M tokens in the step, H the residual width; `x` is the
   ffn        forward(ctx, h, x)                         adds its output into x
   block      forward(ctx, x)                            arranges its parts around x
   head       forward(ctx, h_rows) -> logits f32 [N, V]
+
+Optional, for fewer kernels when a step has few tokens: a norm with the class
+attribute `can_be_lazy` takes `forward(..., lazy=True)` and may then return its
+rows not yet computed (`ops.kernels.NormedRows`); a block passes `lazy=True` only
+for a consumer with the class attribute `takes_lazy_norm`, which promises to hand
+h to exactly one `ctx.ops.linear` and to use nothing of it but its `shape`.
 """
 from __future__ import annotations
 

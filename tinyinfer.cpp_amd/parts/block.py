@@ -22,10 +22,18 @@ class PreNormBlock(Part):
     def children(self):
         return [self.norm1, self.mixer, self.norm2, self.ffn]
 
+    @staticmethod
+    def _normed(ctx, norm, consumer, x):
+        # a consumer that feeds h to exactly one `ops.linear` says so (`takes_lazy_norm`);
+        # a norm that can hand its rows over uncomputed takes the `lazy` argument
+        if getattr(consumer, "takes_lazy_norm", False) and getattr(norm, "can_be_lazy", False):
+            return norm.forward(ctx, x, lazy=True)
+        return norm.forward(ctx, x)
+
     def forward(self, ctx, x):
-        h = self.norm1.forward(ctx, x)
+        h = self._normed(ctx, self.norm1, self.mixer, x)
         self.mixer.forward(ctx, h, x)
-        h = self.norm2.forward(ctx, x)
+        h = self._normed(ctx, self.norm2, self.ffn, x)
         self.ffn.forward(ctx, h, x)
 
 

@@ -13,6 +13,7 @@ from ..spec import TensorNeed
 
 class SwiGLU(Part):
     family = "ffn"
+    takes_lazy_norm = True      # h goes into one product and nowhere else
 
     def __init__(self, prefix: str, hidden: int, intermediate: int):
         super().__init__(prefix)
