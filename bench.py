@@ -121,6 +121,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiles of decoding)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not served (this engine runs on a single GPU)")
@@ -145,8 +146,10 @@ def main() -> int:
     sampler = Sampler(engine.ops, engine.device)
     nums = model_numbers(cfg)
 
-    say(f"prefill of {PREFILL_TOKENS} tokens ...")
-    p_s = measure_prefill(engine, rng)
+    p_s = None
+    if not args.no_prefill:
+        say(f"prefill of {PREFILL_TOKENS} tokens ...")
+        p_s = measure_prefill(engine, rng)
     say(f"decode at batch {args.batch} ...")
     tps, ms = measure_decode(engine, sampler, args.batch, args.steps, args.warmup, rng, "m")
     points = {}
@@ -169,8 +172,9 @@ def main() -> int:
                    "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"], "tied_head": True,
                    "global_batch": args.batch, "cached_tokens": CONTEXT, "seq_len": MAX_SEQ, "page_size": PAGE,
                    "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU", "decode_graph": True},
-        "prefill": {"value": round(PREFILL_TOKENS / p_s, 1), "tokens": PREFILL_TOKENS, "ms": round(p_s * 1e3, 3),
-                    "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / p_s / PEAK_BF16, 4)},
+        "prefill": None if p_s is None else
+        {"value": round(PREFILL_TOKENS / p_s, 1), "tokens": PREFILL_TOKENS, "ms": round(p_s * 1e3, 3),
+         "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / p_s / PEAK_BF16, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM, 4)},
         "points": points,

@@ -192,6 +192,29 @@ def test_norm_inside_the_product_changes_no_bit(model_folders):
         assert np.array_equal(results[0][r], results[1][r]), r
 
 
+def test_prepared_decode_attention_changes_only_rounding(model_folders):
+    """Steps of single tokens norm, rotate and cache inside the attention kernel.  With that
+    switched off the same steps give the same logits up to the rounding of a different order
+    of summation (config D: head size 64, one kv head, a window)."""
+    from tinyinfer_amd.ops.kernels import get_ops
+    folder = model_folders("D", "bfloat16", True)
+    requests = {r: t for r, t in make_requests(CONFIGS["D"]["vocab_size"]).items() if r in ("a", "c")}
+    trace = traces.tail_one_by_one(requests, 48)
+    ops = get_ops()
+    results = []
+    try:
+        for fused in (True, False):
+            ops.use_fused_qk_decode = fused
+            engine = build_engine(folder, "bfloat16", traces.max_tokens(trace))
+            results.append(replay(engine, trace))
+    finally:
+        ops.use_fused_qk_decode = True
+    _, tol = plain_logits(folder, make_requests(CONFIGS["D"]["vocab_size"]), "bfloat16")
+    for r in requests:
+        assert np.abs(results[0][r] - results[1][r]).max() < tol, r
+        assert not np.array_equal(results[0][r][:1], results[0][r][1:2])
+
+
 def test_step_refuses_what_it_cannot_run(model_folders):
     from tinyinfer_amd.engine import StepEntry, EngineError
     from tinyinfer_amd.cache import OutOfPages

@@ -637,6 +637,68 @@ def test_attention_bf16_portions_and_mixed(ops, nh, nkv, hd, P, window):
     assert (got - want).abs().max() < 2e-2
 
 
+@pytest.mark.parametrize("nh,nkv,hd,P,window,norm,rope", [
+    (16, 8, 128, 16, None, True, "table"), (4, 2, 64, 16, None, True, "table"), (3, 1, 128, 32, 50, True, "computed"),
+    (4, 4, 64, 16, 40, False, "table"), (16, 1, 64, 16, None, True, None), (8, 2, 128, 16, None, False, None)])
+def test_attention_bf16_decode_from_projections(ops, nh, nkv, hd, P, window, norm, rope):
+    """The decode kernel that norms and rotates its own queries and writes the row's key and
+    value, against the two kernels it stands for, at context lengths around page edges and
+    split over the context: the same bits in the cache; the same output up to the last
+    bfloat16 bit (the row's own key enters the softmax last instead of in its block)."""
+    if not ops.use_fast_attention:
+        pytest.skip("bfloat16 attention kernels are switched off")
+    g = torch.Generator().manual_seed(nh * 31 + hd)
+    starts = (0, 1, 15, 16, 17, 31, 32, 100, 511, 512, 777, 1500)
+    entries = [(1, s) for s in starts]
+    n_pages_each = [-(-(s + 1) // P) for s in starts]
+    pages = sum(n_pages_each) + 5
+    perm = torch.randperm(pages, generator=g)
+    pool = (torch.randn(pages, 2, nkv, P, hd, generator=g)).to(torch.bfloat16)
+    W = max(n_pages_each) + 1
+    table = torch.full((len(starts), W), -1, dtype=torch.int32)
+    used = 0
+    for e, n in enumerate(n_pages_each):
+        table[e, :n] = perm[used:used + n].to(torch.int32)
+        used += n
+    M = len(starts)
+    qkv = dev(torch.randn(M, (nh + 2 * nkv) * hd, generator=g) * 2.0)
+    q_w = dev(1 + 0.1 * torch.randn(hd, generator=g)) if norm else None
+    k_w = dev(1 + 0.1 * torch.randn(hd, generator=g)) if norm else None
+    inv_freq = tab = None
+    if rope:
+        inv_freq = dev((10000.0 ** (-torch.arange(hd // 2, dtype=torch.float64) * 2 / hd)).float())
+        if rope == "table":
+            tab = ops.rope_table(inv_freq, 600)          # positions beyond the table are computed
+    scale = 1.0 / math.sqrt(hd)
+    ctx = FakeCtx(entries)
+    view = View(dev(table))
+    # the two kernels
+    pool_a = dev(pool.clone())
+    q = torch.empty(M, nh * hd, device="cuda", dtype=torch.bfloat16)
+    ops.qk_norm_rope_kv_write(qkv, q_w, k_w, 1e-5, inv_freq, ctx.positions, ctx.slots, view, pool_a, q, nh, nkv, hd, tab)
+    out_a = torch.zeros_like(q)
+    ops.attention(ctx, view, q, pool_a, out_a, nh, nkv, hd, scale, window)
+    # the one kernel
+    pool_b = dev(pool.clone())
+    out_b = torch.zeros_like(q)
+    assert ops.attention_from_projections(ctx, view, qkv, q_w, k_w, 1e-5, inv_freq, tab, pool_b, True, out_b,
+                                          nh, nkv, hd, scale, window)
+    assert torch.equal(pool_a.view(torch.int16), pool_b.view(torch.int16))
+    assert torch.isfinite(out_b.float()).all()
+
+    def same_up_to_one_step(x, y):
+        x, y = x.float(), y.float()
+        return bool(((x - y).abs() <= 2.0 ** -7 * torch.maximum(x.abs(), y.abs()) + 1e-3 * x.abs().max()).all())
+    assert same_up_to_one_step(out_a, out_b)
+    # and without the write (a layer that reads another layer's keys and values): the cache stays as it is
+    pool_c = pool_a.clone()
+    out_c = torch.zeros_like(q)
+    assert ops.attention_from_projections(ctx, view, qkv[:, :nh * hd].contiguous(), q_w, None, 1e-5, inv_freq, tab,
+                                          pool_c, False, out_c, nh, nkv, hd, scale, window)
+    assert torch.equal(pool_c.view(torch.int16), pool_a.view(torch.int16))
+    assert torch.equal(out_c.view(torch.int16), out_a.view(torch.int16))     # nothing of its own: the same walk
+
+
 def test_attention_bf16_far_key(ops):
     """One key far back carries the weight, for a decode row and for a row inside a portion."""
     if not ops.use_fast_attention:

@@ -23,6 +23,7 @@
 // (The reference scans positions with 16-lane groups and FMA for both cases:
 // /root/reference/src/cuda/attention.cu:107-198.)
 #include "common.h"
+#include "qk_prep.h"
 
 TI_ERROR_API
 
@@ -213,18 +214,120 @@ __device__ __forceinline__ void walk_blocks(const PagedKV& kv, const Frag8* qf, 
   }
 }
 
+// ------------------------------------------- queries and the new key prepared in place
+// What the decode kernel needs to start from the 32-bit projections instead of prepared
+// queries: it norms and rotates its own query heads, and the workgroup whose blocks hold the
+// row's own position writes that position's key and value into the cache before it walks.
+struct QKPrep {
+  const float* qkv;          // [rows, row_width]: q heads, then (if keys are written) k heads, v heads
+  int row_width;
+  const float* q_w;          // per-head norm weights or nullptr
+  const float* k_w;
+  float eps;
+  const float* inv_freq;     // nullptr: no rotation
+  const float2* rope_table;  // (cos, sin) [table_len][hd / 2] or nullptr
+  int table_len;
+  bf16_t* pool_w;            // the cache to write the new key and value into; nullptr: nothing is written
+};
+
+// Q^T fragments of this lane's column (one q head) from the 32-bit projection: the same
+// arithmetic as qk_head_wave, in the layout of the first product.  A lane holds the dims
+// 32 s + 8 quad + j (s < HD / 32, j < 8), which are both halves of its rotation pairs; the
+// sum of squares goes up the same tree as the butterfly of a wavefront with one pair per lane.
+template <int HD>
+__device__ __forceinline__ void prepare_q(const QKPrep& pr, const float* __restrict__ src, int p, bool valid,
+                                          Frag8* qf) {
+  static_assert(HD == 64 || HD == 128, "a lane holds whole rotation pairs for these head sizes only");
+  constexpr int NS = HD / 32, NP = NS / 2, HALF = HD / 2;
+  const int lane = threadIdx.x & 63, quad = lane >> 4;
+  float x[NS][8];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const float4 a = *reinterpret_cast<const float4*>(src + s * 32 + quad * 8);
+    const float4 b = *reinterpret_cast<const float4*>(src + s * 32 + quad * 8 + 4);
+    x[s][0] = a.x; x[s][1] = a.y; x[s][2] = a.z; x[s][3] = a.w;
+    x[s][4] = b.x; x[s][5] = b.y; x[s][6] = b.z; x[s][7] = b.w;
+  }
+  float scale = 1.f;
+  if (pr.q_w) {
+    float u[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      u[j] = qk_pair_square(x[0][j], x[NP][j]);
+      if (NP == 2) u[j] += qk_pair_square(x[1][j], x[1 + NP][j]);   // pairs i and i + 32
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) u[j] += __shfl_xor(u[j], 32, 64);   // pairs i and i ^ 16
+#pragma unroll
+    for (int j = 0; j < 8; ++j) u[j] += __shfl_xor(u[j], 16, 64);   // i ^ 8
+#pragma unroll
+    for (int j = 0; j < 4; ++j) u[j] += u[j + 4];                   // i ^ 4
+    u[0] += u[2];                                                   // i ^ 2
+    u[1] += u[3];
+    scale = qk_norm_scale(u[0] + u[1], HD, pr.eps);                 // i ^ 1
+  }
+  // weights and angles of this lane's pairs: fetched in one go (the table case and the computed
+  // case are told apart once, not per element, so that the loads go out together)
+  float wl[NP][8], wh[NP][8];
+  float2 cs[NP][8];
+  const bool from_table = pr.inv_freq && pr.rope_table && p < pr.table_len;   // the same in every lane
+#pragma unroll
+  for (int sp = 0; sp < NP; ++sp) {
+    const int i0 = sp * 32 + quad * 8;
+    if (pr.q_w) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const float4 a = *reinterpret_cast<const float4*>(pr.q_w + i0 + 4 * h);
+        const float4 b = *reinterpret_cast<const float4*>(pr.q_w + i0 + HALF + 4 * h);
+        wl[sp][4 * h] = a.x; wl[sp][4 * h + 1] = a.y; wl[sp][4 * h + 2] = a.z; wl[sp][4 * h + 3] = a.w;
+        wh[sp][4 * h] = b.x; wh[sp][4 * h + 1] = b.y; wh[sp][4 * h + 2] = b.z; wh[sp][4 * h + 3] = b.w;
+      }
+    }
+    if (from_table) {
+      const float4* t = reinterpret_cast<const float4*>(pr.rope_table + (size_t)p * HALF + i0);
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        const float4 v = t[h];
+        cs[sp][2 * h] = make_float2(v.x, v.y);
+        cs[sp][2 * h + 1] = make_float2(v.z, v.w);
+      }
+    } else if (pr.inv_freq) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) cs[sp][j] = qk_cos_sin(i0 + j, HALF, p, pr.inv_freq, nullptr, 0);
+    }
+  }
+#pragma unroll
+  for (int sp = 0; sp < NP; ++sp) {
+    bf16_t* lo_h = reinterpret_cast<bf16_t*>(&qf[sp].u);
+    bf16_t* hi_h = reinterpret_cast<bf16_t*>(&qf[sp + NP].u);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float lo = x[sp][j] * scale, hi = x[sp + NP][j] * scale;
+      if (pr.q_w) {
+        lo *= wl[sp][j];
+        hi *= wh[sp][j];
+      }
+      if (pr.inv_freq) qk_rotate(lo, hi, cs[sp][j]);
+      lo_h[j] = f2bf(valid ? lo : 0.f);
+      hi_h[j] = f2bf(valid ? hi : 0.f);
+    }
+  }
+}
+
 // =================================================================== decode
 // grid (rows, n_kv * head_parts, splits), 256 threads.  Partials (splits > 1):
 //   part_o [row][head][split][hd], part_ml [row][head][split][2] = (max, sum)
-template <int HD>
+// PREP: the queries come from the 32-bit projections (see QKPrep); needs parts == 1.
+template <int HD, bool PREP>
 __global__ void __launch_bounds__(256)
 attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool, const int* __restrict__ table,
                    int table_stride, const int* __restrict__ pos, const int* __restrict__ slot,
                    const int* __restrict__ rows, bf16_t* __restrict__ out, float* __restrict__ part_o,
                    float* __restrict__ part_ml, int n_head, int n_kv, int P, float scale, int window,
-                   int n_splits) {
+                   int n_splits, QKPrep prep) {
   __shared__ float s_o[4][HD / 16][4][64];
   __shared__ float s_m[4][16], s_l[4][16];
+  __shared__ __attribute__((aligned(16))) bf16_t s_kv[PREP ? 2 * HD : 2];   // the row's own key, then its value
   const int ridx = blockIdx.x;
   const int m_row = rows ? rows[ridx] : ridx;
   const int G = n_head / n_kv;
@@ -246,11 +349,40 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
 
   PagedKV kv{pool, table + (size_t)slot[m_row] * table_stride, P, n_kv, kvh};
   Frag8 qf[HD / 32];
+  bool own_key = false;   // PREP: this workgroup takes the row's own key and value from LDS, not from the cache
+  if constexpr (PREP) {
+    const float* row = prep.qkv + (size_t)m_row * prep.row_width;
+    own_key = prep.pool_w && blk_hi >= b0 && blk_hi < b1;
+    if (own_key) {
+      // this workgroup walks the block of the row's own position.  The position's key and value
+      // are computed here (by the code that prepares whole steps) into LDS; from there they go
+      // into the cache for later steps, and into this step's attention as a block of their own,
+      // so nothing waits for the cache to hold them.
+      if (wave == 0)
+        qk_head_wave<bf16_t>(row + (size_t)(n_head + kvh) * HD, s_kv, 1, prep.k_w, prep.eps, prep.inv_freq,
+                             prep.rope_table, prep.table_len, p_q, HD);
+      if (wave == 1) v_head_wave<bf16_t>(row + (size_t)(n_head + n_kv + kvh) * HD, s_kv + HD, 1, HD);
+    }
+    prepare_q<HD>(prep, row + (size_t)(r16 < n_cols ? head : kvh * G) * HD, p_q, r16 < n_cols, qf);
+    if (own_key) {
+      __syncthreads();
+      const int page = kv.table[p_q / P];
+      if (page >= 0) {    // the host reserves pages first; never write astray
+        bf16_t* kd = kv_page_slot<bf16_t>(prep.pool_w, page, 0, kvh, p_q % P, n_kv, P, HD);
+        bf16_t* vd = kv_page_slot<bf16_t>(prep.pool_w, page, 1, kvh, p_q % P, n_kv, P, HD);
+        for (int i = threadIdx.x; i < HD; i += 256) {
+          kd[i] = s_kv[i];
+          vd[(size_t)i * P] = s_kv[HD + i];
+        }
+      }
+    }
+  } else {
 #pragma unroll
-  for (int s = 0; s < HD / 32; ++s) {
-    qf[s].u = make_uint4(0, 0, 0, 0);
-    if (r16 < n_cols)
-      qf[s].u = *reinterpret_cast<const uint4*>(q + ((size_t)m_row * n_head + head) * HD + s * 32 + quad * 8);
+    for (int s = 0; s < HD / 32; ++s) {
+      qf[s].u = make_uint4(0, 0, 0, 0);
+      if (r16 < n_cols)
+        qf[s].u = *reinterpret_cast<const uint4*>(q + ((size_t)m_row * n_head + head) * HD + s * 32 + quad * 8);
+    }
   }
   float mx = -INFINITY, l = 0.f;
   floatx4 o[HD / 16];
@@ -259,8 +391,22 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
 
   {
     const int mine = (b1 - (b0 + wave) + 3) / 4;   // blocks b0 + wave, + 4, ... below b1
-    walk_blocks<HD>(kv, qf, b0 + wave, 4, mine, lo, p_q, p_q, scale,
+    const int last = own_key ? p_q - 1 : p_q;      // what the cache holds for this workgroup
+    walk_blocks<HD>(kv, qf, b0 + wave, 4, mine, lo, last, last, scale,
                     [=](int b) { return b == blk_lo || b == blk_hi; }, mx, l, o);
+  }
+  if (PREP && own_key && wave == 0) {
+    // the row's own key and value: a block whose first key is the only one that counts
+    KVPair<HD> f;
+#pragma unroll
+    for (int s = 0; s < HD / 32; ++s) {
+      f.k[0][s].u = (r16 == 0) ? *reinterpret_cast<const uint4*>(s_kv + s * 32 + quad * 8) : make_uint4(0, 0, 0, 0);
+      f.k[1][s].u = make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int d = 0; d < HD / 16; ++d)
+      f.v[d].u = make_uint4(quad == 0 ? (unsigned)s_kv[HD + d * 16 + r16] : 0u, 0, 0, 0);
+    attend_pair<HD>(f, qf, BlockInfo{p_q, true, true}, BlockInfo{p_q, false, false}, p_q, p_q, p_q, scale, mx, l, o);
   }
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -779,13 +925,11 @@ static int check_common(const char* what, int n_head, int n_kv, int hd, int P, i
 // Decode rows.  rows: which rows of the step (nullptr: rows 0..n_rows-1).  n_splits > 1 needs
 // part_o (float [n_rows, n_head, n_splits, hd]) and part_ml (float [n_rows, n_head, n_splits, 2]).
 // Returns 3 for sizes these kernels do not serve.
-extern "C" int ti_attention_decode_bf16(const void* q, const void* pool, const int* table, int table_stride,
-                                        const int* pos, const int* slot, const int* rows, void* out,
-                                        float* part_o, float* part_ml, int n_rows, int n_head, int n_kv, int hd,
-                                        int page_size, float scale, int window, int n_splits,
-                                        hipStream_t stream) {
-  int rc = check_common("attention_decode", n_head, n_kv, hd, page_size, table_stride);
-  if (rc) return rc;
+template <bool PREP>
+static int launch_decode(const void* q, const void* pool, const int* table, int table_stride, const int* pos,
+                         const int* slot, const int* rows, void* out, float* part_o, float* part_ml, int n_rows,
+                         int n_head, int n_kv, int hd, int page_size, float scale, int window, int n_splits,
+                         QKPrep prep, hipStream_t stream) {
   TI_REQUIRE(n_splits >= 1 && n_splits <= MERGE_MAX_SPLITS, "attention_decode: bad split count %d (1..%d)", n_splits, MERGE_MAX_SPLITS);
   TI_REQUIRE(n_splits == 1 || (part_o && part_ml), "attention_decode: splits need partial buffers");
   if (n_rows == 0) return 0;
@@ -794,21 +938,73 @@ extern "C" int ti_attention_decode_bf16(const void* q, const void* pool, const i
   dim3 grid(n_rows, n_kv * parts, n_splits);
 #define TI_DEC(H)                                                                                          \
   case H:                                                                                                  \
-    attn_decode_kernel<H><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,           \
-                                                    table_stride, pos, slot, rows, (bf16_t*)out, part_o,    \
-                                                    part_ml, n_head, n_kv, page_size, scale, window,        \
-                                                    n_splits);                                              \
+    attn_decode_kernel<H, PREP><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,     \
+                                                          table_stride, pos, slot, rows, (bf16_t*)out,      \
+                                                          part_o, part_ml, n_head, n_kv, page_size, scale,  \
+                                                          window, n_splits, prep);                          \
     if (n_splits > 1)                                                                                       \
       attn_merge_kernel<H><<<dim3(n_rows, n_head), (H < 64 ? 64 : H), 0, stream>>>(part_o, part_ml, rows,   \
-                                                                                  (bf16_t*)out,            \
-                                                                   n_head, n_splits);                       \
+                                                                                  (bf16_t*)out, n_head,    \
+                                                                                  n_splits);               \
     break;
   switch (hd) {
-    TI_DEC(32) TI_DEC(64) TI_DEC(128)
+    TI_DEC(64) TI_DEC(128)
+    case 32:
+      if constexpr (!PREP) {
+        attn_decode_kernel<32, false><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,
+                                                                table_stride, pos, slot, rows, (bf16_t*)out,
+                                                                part_o, part_ml, n_head, n_kv, page_size, scale,
+                                                                window, n_splits, prep);
+        if (n_splits > 1)
+          attn_merge_kernel<32><<<dim3(n_rows, n_head), 64, 0, stream>>>(part_o, part_ml, rows, (bf16_t*)out,
+                                                                         n_head, n_splits);
+      }
+      break;
   }
 #undef TI_DEC
   TI_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int ti_attention_decode_bf16(const void* q, const void* pool, const int* table, int table_stride,
+                                        const int* pos, const int* slot, const int* rows, void* out,
+                                        float* part_o, float* part_ml, int n_rows, int n_head, int n_kv, int hd,
+                                        int page_size, float scale, int window, int n_splits,
+                                        hipStream_t stream) {
+  int rc = check_common("attention_decode", n_head, n_kv, hd, page_size, table_stride);
+  if (rc) return rc;
+  return launch_decode<false>(q, pool, table, table_stride, pos, slot, rows, out, part_o, part_ml, n_rows, n_head,
+                              n_kv, hd, page_size, scale, window, n_splits, QKPrep{}, stream);
+}
+
+// The same for rows 0..n_rows-1 of a step, starting from the 32-bit projections: qkv is float
+// [n_rows, row_width] with the q heads first and, if write_kv, the k heads and v heads after
+// them.  Per-head norm (q_w, k_w: float [hd] or nullptr), rotation (inv_freq float [hd/2] or
+// nullptr; rope_table float [table_len, hd/2, 2] or nullptr) and the write of each row's key
+// and value at its own position happen inside the attention kernel.  Returns 3 for what it
+// does not serve: head sizes other than 64 and 128, more than 16 q heads per kv head.
+extern "C" int ti_attention_decode_prepared_bf16(const float* qkv, int row_width, const float* q_w,
+                                                 const float* k_w, float eps, const float* inv_freq,
+                                                 const float* rope_table, int table_len, void* pool, int write_kv,
+                                                 const int* table, int table_stride, const int* pos,
+                                                 const int* slot, void* out, float* part_o, float* part_ml,
+                                                 int n_rows, int n_head, int n_kv, int hd, int page_size,
+                                                 float scale, int window, int n_splits, hipStream_t stream) {
+  int rc = check_common("attention_decode_prepared", n_head, n_kv, hd, page_size, table_stride);
+  if (rc) return rc;
+  if (hd == 32 || n_head / n_kv > 16 || ((uintptr_t)q_w & 15) || ((uintptr_t)rope_table & 15)) {
+    ti_set_error("attention_decode_prepared: head_dim %d with %d q heads per kv head is not served (or a norm "
+                 "weight or the sin/cos table is not 16-byte aligned)", hd, n_head / n_kv);
+    return 3;
+  }
+  TI_REQUIRE(qkv && row_width >= (n_head + (write_kv ? 2 * n_kv : 0)) * hd && row_width % 4 == 0 &&
+                 ((uintptr_t)qkv & 15) == 0,
+             "attention_decode_prepared: the projections do not fit (row_width %d)", row_width);
+  TI_REQUIRE(inv_freq || !rope_table, "attention_decode_prepared: a sin/cos table without inv_freq");
+  QKPrep prep{qkv, row_width, q_w, k_w, eps, inv_freq, (const float2*)rope_table, table_len,
+              write_kv ? (bf16_t*)pool : nullptr};
+  return launch_decode<true>(nullptr, pool, table, table_stride, pos, slot, nullptr, out, part_o, part_ml, n_rows,
+                             n_head, n_kv, hd, page_size, scale, window, n_splits, prep, stream);
 }
 
 static int g_prefill_lds = 1;

@@ -3,6 +3,7 @@
 // rotation + paged cache write.  All arithmetic is 32-bit; T is the storage
 // type of activations, weights and cache (float or bfloat16).
 #include "common.h"
+#include "qk_prep.h"
 
 TI_ERROR_API
 
@@ -176,62 +177,25 @@ qk_norm_rope_kv_write_kernel(
   const int wave = threadIdx.x / TI_WAVE, lane = threadIdx.x % TI_WAVE;
   const int u = blockIdx.y * (blockDim.x / TI_WAVE) + wave;
   if (u >= n_head + 2 * n_kv) return;
-  const int half = hd / 2;
   const int nq = n_head * hd, nk = n_kv * hd;
   const float* row = qkv + (size_t)m * (nq + 2 * nk);
   const int p = pos[m];
   const bool is_q = u < n_head;
   const bool is_v = u >= n_head + n_kv;
   const float* src = row + (size_t)u * hd;
-  T* dst;
   if (is_q) {
-    dst = q_out + (size_t)m * nq + (size_t)u * hd;
-  } else {
-    const int page = table[(size_t)slot[m] * table_stride + p / P];
-    if (page < 0) return;   // the host reserves pages first; never write astray
-    const int prow = p % P;
-    const int kvh = is_v ? u - n_head - n_kv : u - n_head;
-    dst = pool + (size_t)page * 2 * n_kv * P * hd + ((size_t)(is_v ? 1 : 0) * n_kv + kvh) * P * hd +
-          (is_v ? (size_t)prow : (size_t)prow * hd);
-  }
-  if (is_v) {
-    for (int i = lane; i < hd; i += TI_WAVE) st<T>(dst + (size_t)i * P, src[i]);
+    qk_head_wave<T>(src, q_out + (size_t)m * nq + (size_t)u * hd, 1, q_w, eps, inv_freq, rope_table, table_len, p,
+                    hd);
     return;
   }
-  const float* w = is_q ? q_w : k_w;
-  float scale = 1.f;
-  if (w) {
-    float ss = 0.f;
-    for (int i = lane; i < half; i += TI_WAVE) {
-      const float lo = src[i], hi = src[i + half];
-      ss += lo * lo + hi * hi;
-    }
-    ss = group_sum<TI_WAVE>(ss);
-    scale = 1.0f / sqrtf(ss / (float)hd + eps);
-  }
-  const float fp = (float)p;
-  for (int i = lane; i < half; i += TI_WAVE) {
-    float lo = src[i] * scale, hi = src[i + half] * scale;
-    if (w) {
-      lo *= w[i];
-      hi *= w[i + half];
-    }
-    if (inv_freq) {
-      float s, c;
-      if (rope_table && p < table_len) {
-        const float2 cs = rope_table[(size_t)p * half + i];
-        c = cs.x;
-        s = cs.y;
-      } else {
-        sincosf(fp * inv_freq[i], &s, &c);
-      }
-      const float a = lo * c - hi * s, b = lo * s + hi * c;
-      lo = a;
-      hi = b;
-    }
-    st<T>(dst + i, lo);
-    st<T>(dst + i + half, hi);
-  }
+  const int page = table[(size_t)slot[m] * table_stride + p / P];
+  if (page < 0) return;   // the host reserves pages first; never write astray
+  const int kvh = is_v ? u - n_head - n_kv : u - n_head;
+  T* dst = kv_page_slot<T>(pool, page, is_v ? 1 : 0, kvh, p % P, n_kv, P, hd);
+  if (is_v)
+    v_head_wave<T>(src, dst, (size_t)P, hd);
+  else
+    qk_head_wave<T>(src, dst, 1, k_w, eps, inv_freq, rope_table, table_len, p, hd);
 }
 
 extern "C" int ti_qk_norm_rope_kv_write(int dtype, const float* qkv, const float* q_w, const float* k_w,

@@ -27,6 +27,38 @@ def _ptr(t):
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
 
+PREPARED_HEAD_DIMS = (64, 128)   # head sizes whose queries the decode kernel prepares itself
+
+
+def run_decode_prepared(ops, ctx, view, qkv, q_w, k_w, eps, inv_freq, rope_table, pool, write_kv, out,
+                        heads, kv_heads, head_dim, scale, window) -> bool:
+    """A step of single-token rows, straight from the 32-bit projections: per-head norm,
+    rotation and the write of each row's key and value happen inside the decode kernel.
+    False if the kernel does not serve the sizes (nothing has been done then)."""
+    P = pool.shape[3]
+    if head_dim not in PREPARED_HEAD_DIMS or P % 16 != 0 or heads // kv_heads > 16 or not ctx.decode_only:
+        return False
+    lib = ops.lib("attention_bf16")
+    table = view.table
+    win = int(window or 0)
+    n = ctx.M
+    context = ctx.split_context if win == 0 else min(ctx.split_context, win + 16)
+    S = decode_splits(n, kv_heads, heads, context)
+    part_o = part_ml = None
+    if S > 1:
+        part_o = ctx.buf("attn.part_o", (n, heads, S, head_dim), torch.float32)
+        part_ml = ctx.buf("attn.part_ml", (n, heads, S, 2), torch.float32)
+    rc = lib.ti_attention_decode_prepared_bf16(
+        _ptr(qkv), qkv.shape[1], _ptr(q_w), _ptr(k_w), ctypes.c_float(eps), _ptr(inv_freq), _ptr(rope_table),
+        0 if rope_table is None else rope_table.shape[0], _ptr(pool), 1 if write_kv else 0,
+        _ptr(table), table.shape[1], _ptr(ctx.positions), _ptr(ctx.slots), _ptr(out), _ptr(part_o), _ptr(part_ml),
+        n, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, S, ops._stream())
+    if rc == 3:
+        return False
+    ops._check(lib, rc, "attention(decode, prepared)")
+    return True
+
+
 def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) -> bool:
     P = pool.shape[3]
     if head_dim not in SERVED_HEAD_DIMS or P % 16 != 0:

@@ -65,6 +65,7 @@ class Ops:
         self.use_fast_gemm = have("gemm_bf16")
         self.use_fast_attention = have("attention_bf16")
         self.use_fused_norm = True       # the norm before a product inside the product's kernel (few tokens)
+        self.use_fused_qk_decode = True  # per-head norm, rotation and cache write inside the decode attention
 
     # ------------------------------------------------------------------ loading
     def lib(self, name: str) -> ctypes.CDLL:
@@ -283,6 +284,39 @@ class Ops:
                 return
         self.attention_rows(q, pool, view.table, ctx.positions, ctx.slots, out, heads, kv_heads, head_dim,
                             scale, window)
+
+    def attention_from_projections(self, ctx, view, qkv, q_w, k_w, eps, inv_freq, rope_table, pool, write_kv,
+                                   out, heads, kv_heads, head_dim, scale, window) -> bool:
+        """`qk_norm_rope_kv_write` and `attention` in one kernel, for steps of single tokens
+        in bfloat16: qkv f32 [M, (heads + 2 kv_heads) hd] (only the q heads if not write_kv).
+        False if no kernel serves the step; then nothing has been done and the caller
+        makes the two calls."""
+        if not (self.use_fused_qk_decode and self.use_fast_attention and ctx.decode_only
+                and pool.dtype == torch.bfloat16):
+            return False
+        M = qkv.shape[0]
+        width = (heads + (2 * kv_heads if write_kv else 0)) * head_dim
+        self._dev(qkv, q_w, k_w, inv_freq, rope_table, pool, view.table, out)
+        if qkv.dim() != 2 or qkv.shape[1] < width or qkv.dtype != torch.float32 or not qkv.is_contiguous():
+            raise KernelError(f"attention_from_projections: qkv {tuple(qkv.shape)} {qkv.dtype} does not fit "
+                              f"[{M}, >= {width}] float32")
+        if out.shape != (M, heads * head_dim) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+            raise KernelError("attention_from_projections: out has the wrong shape or dtype")
+        if pool.dim() != 5 or pool.shape[1] != 2 or pool.shape[2] != kv_heads or pool.shape[4] != head_dim \
+                or not pool.is_contiguous() or not view.table.is_contiguous():
+            raise KernelError(f"attention_from_projections: pool {tuple(pool.shape)} does not fit "
+                              f"[pages,2,{kv_heads},P,{head_dim}]")
+        for wt in (q_w, k_w):
+            if wt is not None and (wt.shape != (head_dim,) or wt.dtype != torch.float32):
+                raise KernelError("attention_from_projections: norm weights must be float32 [head_dim]")
+        if inv_freq is not None and (inv_freq.shape != (head_dim // 2,) or inv_freq.dtype != torch.float32):
+            raise KernelError("attention_from_projections: inv_freq must be float32 [head_dim/2]")
+        if rope_table is not None and (rope_table.dtype != torch.float32 or not rope_table.is_contiguous()
+                                       or rope_table.shape[1:] != (head_dim // 2, 2)):
+            raise KernelError("attention_from_projections: the sin/cos table must be float32 [positions, head_dim/2, 2]")
+        from . import attention_bf16
+        return attention_bf16.run_decode_prepared(self, ctx, view, qkv, q_w, k_w, eps, inv_freq, rope_table, pool,
+                                                  write_kv, out, heads, kv_heads, head_dim, scale, window)
 
     # ------------------------------------------------------------------ sampling
     def argmax(self, logits, out):

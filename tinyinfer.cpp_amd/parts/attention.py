@@ -89,6 +89,13 @@ class Attention(Part):
         pool = ctx.kv_pool(group, layer)
         view = ctx.cache_view(group)
         rot = self.pos.fused_rotation() if self.pos is not None and hasattr(self.pos, "fused_rotation") else None
+        a = ctx.buf("attn.out", (M, self.nq), ctx.act_dtype)
+        if (self.pos is None or rot is not None) and ctx.ops.attention_from_projections(
+                ctx, view, qkv, self.q_norm_w, self.k_norm_w, self.eps,
+                None if rot is None else rot["inv_freq"], None if rot is None else rot.get("table"),
+                pool, not self.shares_kv, a, self.heads, self.kv_heads, self.head_dim, self.scale, self.window):
+            ctx.ops.linear(a, self.w_o, x, "add")        # a step of single tokens: one kernel did it all
+            return
         if self.pos is not None and rot is None:
             # a position encoding without a fused form runs on the 32-bit projections first
             qv = qkv[:, :self.nq].unflatten(1, (self.heads, self.head_dim))
@@ -100,7 +107,6 @@ class Attention(Part):
             ctx.positions, ctx.slots, view, pool, q,
             self.heads, 0 if self.shares_kv else self.kv_heads, self.head_dim,
             None if rot is None else rot.get("table"))
-        a = ctx.buf("attn.out", (M, self.nq), ctx.act_dtype)
         ctx.ops.attention(ctx, view, q, pool, a, self.heads, self.kv_heads, self.head_dim,
                           self.scale, self.window)
         ctx.ops.linear(a, self.w_o, x, "add")
