@@ -121,7 +121,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
-    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiles of decoding)")
+    ap.add_argument("--only", choices=["all", "decode", "prefill"], default="all",
+                    help="measure one phase only (for profiles): the other's fields are null")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not served (this engine runs on a single GPU)")
@@ -138,7 +139,7 @@ def main() -> int:
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     rng = np.random.default_rng(0)
-    biggest = max(args.batch, 1 if args.no_points else 64)
+    biggest = max(args.batch, 1 if (args.no_points or args.only != "all") else 64)
     say("building the model (random weights on the device) ...")
     engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", page_size=PAGE,
                                 max_tokens=biggest * (CONTEXT + 512) + PREFILL_TOKENS, max_requests=biggest + 1,
@@ -146,25 +147,26 @@ def main() -> int:
     sampler = Sampler(engine.ops, engine.device)
     nums = model_numbers(cfg)
 
-    p_s = None
-    if not args.no_prefill:
+    p_s = tps = ms = None
+    if args.only != "decode":
         say(f"prefill of {PREFILL_TOKENS} tokens ...")
         p_s = measure_prefill(engine, rng)
-    say(f"decode at batch {args.batch} ...")
-    tps, ms = measure_decode(engine, sampler, args.batch, args.steps, args.warmup, rng, "m")
+    if args.only != "prefill":
+        say(f"decode at batch {args.batch} ...")
+        tps, ms = measure_decode(engine, sampler, args.batch, args.steps, args.warmup, rng, "m")
     points = {}
-    if not args.no_points:
+    if not args.no_points and args.only == "all":
         for b, k in ((1, args.steps), (64, max(16, args.steps // 4))):
             say(f"decode at batch {b} ...")
             points[f"decode_b{b}"] = round(measure_decode(engine, sampler, b, k, max(4, args.warmup // 2), rng, f"p{b}_")[0], 1)
 
     ctx_mean = CONTEXT + args.warmup + args.steps / 2.0
     step_bytes = nums["weight_bytes"] + args.batch * ctx_mean * nums["kv_bytes_per_token"]
-    achieved = step_bytes / (ms * 1e-3)
+    achieved = step_bytes / (ms * 1e-3) if ms else None
     out = {
-        "metric": "decode tok/s @ batch 8 (Qwen3-0.6B sizes, 2,048 cached tokens per request)",
-        "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "metric": f"decode tok/s @ batch {args.batch} (Qwen3-0.6B sizes, 2,048 cached tokens per request)",
+        "value": None if tps is None else round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": None if ms is None else round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic (uniform random token ids, random weights N(0, 0.02))",
         "config": {"model": "Qwen3-0.6B sizes", "layers": cfg["num_hidden_layers"], "layers_in_config": layers_full,
                    "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
@@ -175,8 +177,9 @@ def main() -> int:
         "prefill": None if p_s is None else
         {"value": round(PREFILL_TOKENS / p_s, 1), "tokens": PREFILL_TOKENS, "ms": round(p_s * 1e3, 3),
          "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / p_s / PEAK_BF16, 4)},
-        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM, 4)},
+        "roofline": None if achieved is None else
+        {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+         "frac": round(achieved / PEAK_HBM, 4)},
         "points": points,
     }
     print(json.dumps(out), flush=True)
