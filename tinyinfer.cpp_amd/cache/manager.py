@@ -16,6 +16,7 @@ and the state live in `CacheStorage`.
 """
 from __future__ import annotations
 
+import numpy as np
 from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
@@ -73,12 +74,39 @@ class _Request:
 class PagedGroup:
     """Pages and block tables of one group of layers."""
 
-    def __init__(self, need: PagedKVNeed, n_layers: int, page_size: int, num_pages: int):
+    def __init__(self, need: PagedKVNeed, n_layers: int, page_size: int, num_pages: int, table_width: int):
         self.need = need
         self.n_layers = n_layers
         self.page_size = page_size
         self.pool = PagePool(num_pages)
         self.tables: Dict[Hashable, List[int]] = {}      # -1: given back (behind the window)
+        # the same as rows of `table_width` int32 (-1 where there is no page), ready to be
+        # copied into a step's metadata
+        self.table_width = table_width
+        self.rows: Dict[Hashable, np.ndarray] = {}
+
+    def new_table(self, req: Hashable) -> None:
+        self.tables[req] = []
+        self.rows[req] = np.full(self.table_width, -1, dtype=np.int32)
+
+    def append_page(self, req: Hashable) -> None:
+        t = self.tables[req]
+        page = self.pool.take()
+        self.rows[req][len(t)] = page
+        t.append(page)
+
+    def give_back_page(self, req: Hashable, index: int) -> None:
+        t = self.tables[req]
+        self.pool.give_back(t[index])
+        t[index] = -1
+        self.rows[req][index] = -1
+
+    def drop_table(self, req: Hashable) -> None:
+        t = self.tables.pop(req)
+        del self.rows[req]
+        for p in reversed(t):              # so the lowest page is handed out next
+            if p >= 0:
+                self.pool.give_back(p)
 
     def first_needed_page(self, next_pos: int) -> int:
         """Index of the first page that a query at `next_pos` or later still reads."""
@@ -111,12 +139,14 @@ class CacheManager:
         self.groups: List[object] = []
         for need, n_layers in groups:
             if isinstance(need, PagedKVNeed):
-                self.groups.append(PagedGroup(need, n_layers, self.page_size, num_pages))
+                self.groups.append(PagedGroup(need, n_layers, self.page_size, num_pages,
+                                              self.max_pages_per_request))
             elif isinstance(need, StateNeed):
                 self.groups.append(need)
             else:
                 raise CacheError(f"unknown cache need {need!r}")
         self.group_layers = [n for _, n in groups]
+        self._paged = [(i, g) for i, g in enumerate(self.groups) if isinstance(g, PagedGroup)]
         self._requests: Dict[Hashable, _Request] = {}
         self._free_slots: List[int] = list(range(self.max_requests - 1, -1, -1))
         # slots whose state tensors must be zeroed before their next use
@@ -124,7 +154,7 @@ class CacheManager:
 
     # ---------------------------------------------------------------- queries
     def paged_groups(self):
-        return [(i, g) for i, g in enumerate(self.groups) if isinstance(g, PagedGroup)]
+        return self._paged
 
     def state_groups(self):
         return [(i, g) for i, g in enumerate(self.groups) if isinstance(g, StateNeed)]
@@ -183,7 +213,7 @@ class CacheManager:
         slot = self._free_slots.pop()
         self._requests[req] = _Request(slot)
         for _, g in self.paged_groups():
-            g.tables[req] = []
+            g.new_table(req)
         self.slots_to_clear.append(slot)
         return slot
 
@@ -201,7 +231,7 @@ class CacheManager:
                                  f"{g.pool.num_free} are free")
         for _, g in self.paged_groups():
             for _ in range(g.pages_to_cover(req, upto)):
-                g.tables[req].append(g.pool.take())
+                g.append_page(req)
         r.reserved = upto
 
     def commit(self, req: Hashable, n_tokens: int) -> None:
@@ -213,11 +243,12 @@ class CacheManager:
         r.length += n_tokens
         for _, g in self.paged_groups():
             first = g.first_needed_page(r.length)
+            if first == 0:
+                continue
             t = g.tables[req]
             for i in range(min(first, len(t))):
                 if t[i] >= 0:
-                    g.pool.give_back(t[i])
-                    t[i] = -1
+                    g.give_back_page(req, i)
 
     def release(self, req: Hashable) -> None:
         """The request is over (finished, aborted or preempted): every page and
@@ -226,10 +257,7 @@ class CacheManager:
         if r is None:
             raise CacheError(f"request {req!r} released but not admitted")
         for _, g in self.paged_groups():
-            t = g.tables.pop(req)
-            for p in reversed(t):          # so the lowest page is handed out next
-                if p >= 0:
-                    g.pool.give_back(p)
+            g.drop_table(req)
         self._free_slots.append(r.slot)
 
     # ------------------------------------------------------------- invariants
@@ -240,6 +268,8 @@ class CacheManager:
             for req, t in g.tables.items():
                 r = self._requests[req]
                 assert len(t) * self.page_size >= r.reserved, (gi, req, "table shorter than reservation")
+                row = g.rows[req]
+                assert list(row[:len(t)]) == t and (row[len(t):] == -1).all(), (gi, req, "the table's row differs")
                 first = g.first_needed_page(r.length)
                 for i, p in enumerate(t):
                     if i >= first:

@@ -209,37 +209,40 @@ class Engine:
         if not entries:
             raise EngineError("a step needs at least one entry")
         V = self.model.vocab_size
+        cache = self.cache
         seen = set()
         M = 0
         n_want = 0
         for e in entries:
+            toks = e.tokens
+            n = len(toks)
             if e.request in seen:
                 raise EngineError(f"request {e.request!r} appears twice in one step")
             seen.add(e.request)
-            if len(e.tokens) == 0:
+            if n == 0:
                 raise EngineError(f"request {e.request!r}: an entry needs at least one token")
-            for t in e.tokens:
-                if not (0 <= int(t) < V):
-                    raise EngineError(f"request {e.request!r}: token id {t} is outside the vocabulary [0, {V})")
-            for w in e.want:
-                if not (0 <= int(w) < len(e.tokens)):
-                    raise EngineError(f"request {e.request!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
-            M += len(e.tokens)
+            if not (0 <= min(toks) and max(toks) < V):
+                bad = next(t for t in toks if not (0 <= int(t) < V))
+                raise EngineError(f"request {e.request!r}: token id {bad} is outside the vocabulary [0, {V})")
+            if e.want and not (0 <= min(e.want) and max(e.want) < n):
+                bad = next(w for w in e.want if not (0 <= int(w) < n))
+                raise EngineError(f"request {e.request!r}: wanted place {bad} is outside its {n} tokens")
+            M += n
             n_want += len(e.want)
 
-        cache = self.cache
         # all or nothing: see that every group can cover every entry before taking a page
-        new = [e.request for e in entries if not cache.has(e.request)]
-        if len(new) > cache.num_free_slots():
-            raise EngineError(f"{len(new)} new requests but only {cache.num_free_slots()} free request slots")
-        for gi, g in cache.paged_groups():
+        paged = cache.paged_groups()
+        n_new = sum(1 for e in entries if not cache.has(e.request))
+        if n_new > cache.num_free_slots():
+            raise EngineError(f"{n_new} new requests but only {cache.num_free_slots()} free request slots")
+        for gi, g in paged:
             need = 0
             for e in entries:
-                base = cache._requests[e.request].reserved if cache.has(e.request) else 0
-                if base + len(e.tokens) > cache.max_seq:
-                    raise EngineError(f"request {e.request!r}: {base + len(e.tokens)} tokens exceed "
-                                      f"max_seq = {cache.max_seq}")
-                need += g.pages_to_cover(e.request if cache.has(e.request) else None, base + len(e.tokens))
+                known = cache.has(e.request)
+                upto = (cache._requests[e.request].reserved if known else 0) + len(e.tokens)
+                if upto > cache.max_seq:
+                    raise EngineError(f"request {e.request!r}: {upto} tokens exceed max_seq = {cache.max_seq}")
+                need += g.pages_to_cover(e.request if known else None, upto)
             if need > g.pool.num_free:
                 raise OutOfPages(f"the step needs {need} new pages in cache group {gi}, {g.pool.num_free} are free")
         for e in entries:
@@ -253,26 +256,42 @@ class Engine:
         ctx = StepContext(self)
         ctx.M = M
         R = len(entries)
-        paged = cache.paged_groups()
         W = self.table_width
-        tiles: List[Tuple[int, int]] = []
+        tiles: List[int] = []             # (entry, first row) pairs, flat
         dec_rows: List[int] = []
+        tokens: List[int] = []
+        positions: List[int] = []
+        slots: List[int] = []
+        out_rows: List[int] = []
+        ent_flat: List[int] = []
         row0 = 0
         for i, e in enumerate(entries):
             n = len(e.tokens)
             start = cache.length(e.request)
-            ctx.entries.append((row0, n, start, cache.slot(e.request)))
-            ctx.max_context = max(ctx.max_context, start + n)
+            rec = (row0, n, start, cache.slot(e.request))
+            ctx.entries.append(rec)
+            ent_flat.extend(rec)
+            tokens.extend(e.tokens)
             if n > 1:
+                positions.extend(range(start, start + n))
+                slots.extend([i] * n)
                 for q0 in range(0, n, PREFILL_TILE_Q):
-                    tiles.append((i, row0 + q0))
+                    tiles.append(i)
+                    tiles.append(row0 + q0)
             else:
+                positions.append(start)
+                slots.append(i)
                 dec_rows.append(row0)
+            for w in e.want:
+                out_rows.append(row0 + int(w))
+            if start + n > ctx.max_context:
+                ctx.max_context = start + n
             row0 += n
-        ctx.decode_only = not tiles
+        n_tiles = len(tiles) // 2
+        ctx.decode_only = n_tiles == 0
         if ctx.decode_only:
             dec_rows = []
-        ctx.n_tiles = len(tiles)
+        ctx.n_tiles = n_tiles
         ctx.n_decode_rows = len(dec_rows)
         ctx.split_context = ctx.max_context
 
@@ -281,31 +300,22 @@ class Engine:
         o_out = 3 * M
         o_ent = o_out + n_want
         o_tile = o_ent + 4 * R
-        o_dec = o_tile + 2 * len(tiles)
+        o_dec = o_tile + 2 * n_tiles
         o_tab = o_dec + len(dec_rows)
         total = o_tab + len(paged) * R * W
         turn, host, dev = self._meta_buffers(total, meta_dev)
         h = host.numpy()
-        out_i = o_out
-        for i, (e, (r0, n, start, sslot)) in enumerate(zip(entries, ctx.entries)):
-            h[o_tok + r0:o_tok + r0 + n] = e.tokens
-            h[o_pos + r0:o_pos + r0 + n] = range(start, start + n)
-            h[o_slot + r0:o_slot + r0 + n] = i
-            for w in e.want:
-                h[out_i] = r0 + int(w)
-                out_i += 1
-            h[o_ent + 4 * i:o_ent + 4 * i + 4] = (r0, n, start, sslot)
-        for j, (ei, q0) in enumerate(tiles):
-            h[o_tile + 2 * j] = ei
-            h[o_tile + 2 * j + 1] = q0
-        if dec_rows:
-            h[o_dec:o_dec + len(dec_rows)] = dec_rows
+        h[o_tok:o_pos] = tokens
+        h[o_pos:o_slot] = positions
+        h[o_slot:o_out] = slots
+        h[o_out:o_tile] = out_rows + ent_flat
+        if tiles or dec_rows:
+            h[o_tile:o_tab] = tiles + dec_rows
         for k, (gi, g) in enumerate(paged):
             base = o_tab + k * R * W
-            h[base:base + R * W] = -1
+            rows = g.rows
             for i, e in enumerate(entries):
-                t = g.tables[e.request]
-                h[base + i * W:base + i * W + len(t)] = t
+                h[base + i * W:base + (i + 1) * W] = rows[e.request]
         dev[:total].copy_(host[:total], non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
@@ -316,7 +326,7 @@ class Engine:
         ctx.slots = dev[o_slot:o_slot + M]
         ctx.out_rows = dev[o_out:o_out + n_want] if n_want else None
         ctx.entry_meta = dev[o_ent:o_ent + 4 * R].view(R, 4)
-        ctx.tiles = dev[o_tile:o_tile + 2 * len(tiles)].view(-1, 2) if tiles else None
+        ctx.tiles = dev[o_tile:o_tile + 2 * n_tiles].view(-1, 2) if n_tiles else None
         ctx.decode_rows = dev[o_dec:o_dec + len(dec_rows)] if dec_rows else None
         for k, (gi, g) in enumerate(paged):
             base = o_tab + k * R * W
