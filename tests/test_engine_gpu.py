@@ -215,6 +215,27 @@ def test_prepared_decode_attention_changes_only_rounding(model_folders):
         assert not np.array_equal(results[0][r][:1], results[0][r][1:2])
 
 
+def test_prepared_qkv_product_changes_no_bit(model_folders):
+    """Steps of many tokens prepare q and write the cache in the epilogue of the q/k/v product.
+    With that switched off the same steps give the same bits (config D, head size 64)."""
+    from tinyinfer_amd.ops.kernels import get_ops
+    folder = model_folders("D", "bfloat16", True)
+    requests = {"a": random_tokens(300, CONFIGS["D"]["vocab_size"], 5), "b": random_tokens(90, CONFIGS["D"]["vocab_size"], 6)}
+    trace = [{"entries": [("a", requests["a"][:200], [0, 199]), ("b", requests["b"][:70], [69])], "end": []},
+             {"entries": [("a", requests["a"][200:], list(range(100))), ("b", requests["b"][70:71], [0])], "end": ["a", "b"]}]
+    ops = get_ops()
+    results = []
+    try:
+        for fused in (True, False):
+            ops.use_fused_qkv_prefill = fused
+            engine = build_engine(folder, "bfloat16", 512)
+            results.append(replay(engine, trace))
+    finally:
+        ops.use_fused_qkv_prefill = True
+    for r in requests:
+        assert np.array_equal(results[0][r], results[1][r]), r
+
+
 def test_step_refuses_what_it_cannot_run(model_folders):
     from tinyinfer_amd.engine import StepEntry, EngineError
     from tinyinfer_amd.cache import OutOfPages

@@ -699,6 +699,51 @@ def test_attention_bf16_decode_from_projections(ops, nh, nkv, hd, P, window, nor
     assert torch.equal(out_c.view(torch.int16), out_a.view(torch.int16))     # nothing of its own: the same walk
 
 
+@pytest.mark.parametrize("M,nh,nkv,hd,K,P,norm,rope", [
+    (300, 3, 1, 64, 192, 16, True, "table"), (257, 4, 2, 128, 128, 16, True, "table"),
+    (100, 2, 2, 128, 64, 32, False, "computed"), (513, 5, 1, 64, 256, 16, True, None), (70, 2, 0, 128, 64, 16, True, "table")])
+def test_qkv_product_with_prepared_heads(ops, M, nh, nkv, hd, K, P, norm, rope):
+    """The q/k/v product whose epilogue norms, rotates and caches, against the product followed
+    by the kernel that prepares whole steps: the same bits in q and in the cache (rows that
+    are no multiple of the tile, a last tile with a head beyond the matrix, no k/v heads)."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    g = torch.Generator().manual_seed(M + nh)
+    N = (nh + 2 * nkv) * hd
+    a = dev((torch.randn(M, K, generator=g)).to(torch.bfloat16))
+    w = dev((torch.randn(N, K, generator=g) * 0.2).to(torch.bfloat16))
+    q_w = dev(1 + 0.1 * torch.randn(hd, generator=g)) if norm else None
+    k_w = dev(1 + 0.1 * torch.randn(hd, generator=g)) if norm and nkv else None
+    inv_freq = tab = None
+    if rope:
+        inv_freq = dev((10000.0 ** (-torch.arange(hd // 2, dtype=torch.float64) * 2 / hd)).float())
+        if rope == "table":
+            tab = ops.rope_table(inv_freq, 200)          # positions beyond the table are computed
+    # two requests: rows [0, n0) continue one at position 37 (its rows straddle pages), the rest
+    # start another at 0; for some sizes that one starts on a multiple of 16 rows, so that runs of
+    # 16 tile rows are whole runs of a page (the values' fast path), for others not
+    n0 = (M // 3) // 16 * 16 if M in (300, 513) else M // 3
+    pos = torch.cat([torch.arange(37, 37 + n0), torch.arange(0, M - n0)]).to(torch.int32)
+    slot = torch.cat([torch.zeros(n0), torch.ones(M - n0)]).to(torch.int32)
+    pages_each = -(-(M + 40) // P)
+    perm = torch.randperm(2 * pages_each + 3, generator=g).to(torch.int32)
+    table = torch.stack([perm[:pages_each], perm[pages_each:2 * pages_each]]).contiguous()
+    pool0 = torch.randn(2 * pages_each + 3, 2, max(nkv, 1), P, hd, generator=g).to(torch.bfloat16)
+    view = View(dev(table))
+    pos, slot = dev(pos), dev(slot)
+    pool_a, pool_b = dev(pool0.clone()), dev(pool0.clone())
+    qkv = torch.empty(M, N, device="cuda")
+    ops.linear(a, w, qkv, "store")
+    q_a = torch.zeros(M, nh * hd, device="cuda", dtype=torch.bfloat16)
+    ops.qk_norm_rope_kv_write(qkv, q_w, k_w, 1e-5, inv_freq, pos, slot, view, pool_a, q_a, nh, nkv, hd, tab)
+    q_b = torch.zeros_like(q_a)
+    assert ops.qkv_prepared(a, w, q_w, k_w, 1e-5, inv_freq, tab, pos, slot, view, pool_b, q_b, nh, nkv, hd)
+    assert torch.equal(q_a.view(torch.int16), q_b.view(torch.int16))
+    assert torch.equal(pool_a.view(torch.int16), pool_b.view(torch.int16))
+    if nkv:
+        assert not torch.equal(pool_a.view(torch.int16), dev(pool0).view(torch.int16))
+
+
 def test_attention_bf16_far_key(ops):
     """One key far back carries the weight, for a decode row and for a row inside a portion."""
     if not ops.use_fast_attention:

@@ -19,6 +19,7 @@ typedef uint16_t bf16_t;   // bfloat16 bits; arithmetic always happens in float
 #define TI_EPI_ADD_F32 1     // out f32 [M,N] += A W^T        (residual sum in 32-bit)
 #define TI_EPI_STORE_ACT 2   // out T   [M,N] = A W^T
 #define TI_EPI_SWIGLU 3      // W = [gate; up] ([2F,K]); out T [M,F] = silu(g) * u
+#define TI_EPI_QKV_PREP 4    // W = [q; k; v] heads: per-head norm, rotation, q out and cache write (own entry point)
 
 __device__ __forceinline__ float bf2f(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 

@@ -17,6 +17,7 @@
 // /root/reference/src/cuda/gemm.cu:37-85 and 152-261; it reads the weights once
 // per row of A for M <= 32.)
 #include "common.h"
+#include "qk_prep.h"
 
 TI_ERROR_API
 
@@ -419,10 +420,30 @@ __device__ __forceinline__ void wait_vmcnt(int n) {
   }
 }
 
+// What the epilogue TI_EPI_QKV_PREP needs: the product is the fused q/k/v projection of a step's
+// rows, and instead of storing it the kernel finishes each head of each row: per-head norm and
+// rotation for q heads (to q_out, T [M, n_head hd]) and k heads (into the cache page of the row's
+// position), v heads copied into the cache transposed.  A workgroup's BN columns are whole heads.
+struct QKVEpilogue {
+  const float* q_w;          // per-head norm weights or nullptr
+  const float* k_w;
+  float eps;
+  const float* inv_freq;     // nullptr: no rotation
+  const float2* rope_table;  // (cos, sin) [table_len][hd / 2] or nullptr
+  int table_len;
+  const int* pos;            // position of each row
+  const int* slot;           // block-table row of each row
+  const int* table;
+  int table_stride;
+  bf16_t* pool;              // [pages][2][n_kv][P * hd]
+  bf16_t* q_out;
+  int n_head, n_kv, hd, P;
+};
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
 __global__ void __launch_bounds__(256)
 gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_,
-                      int M, int N, int K, long lda) {
+                      int M, int N, int K, long lda, QKVEpilogue ep = QKVEpilogue{}) {
   constexpr bool SW = (EPI == TI_EPI_SWIGLU);
   constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
   static_assert(WAVES_M * WAVES_N == 4, "four wavefronts");
@@ -552,6 +573,91 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
 
   // acc[a][b][i]: row wm*(BM/WAVES_M) + a*32 + 8*(i/4) + 4*(lane/32) + i%4, column wn*(BN/WAVES_N) + b*32 + lane%32
   const int ccol = lane & 31, crow = (lane >> 5) * 4;
+  if constexpr (EPI == TI_EPI_QKV_PREP) {
+    // The tile goes to LDS in 32-bit (the stages are free now), then every thread finishes one row:
+    // for each head of the tile, the arithmetic of the kernel that prepares whole steps.
+    static_assert(BM == 256, "a row per thread");
+    constexpr int FS = BN + 1;                              // row stride: threads of a wavefront read different rows
+    static_assert(BM * FS * 4 + 3 * BM * 4 <= PSTAGES * (BM + BN) * PBK * 2, "the 32-bit tile fits into the stages");
+    float* ft = reinterpret_cast<float*>(smem);
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+          ft[(wm * (BM / WAVES_M) + a * 32 + (i >> 2) * 8 + crow + (i & 3)) * FS + wn * (BN / WAVES_N) + b * 32 + ccol] =
+              acc[a][b][i];
+    __syncthreads();
+    // each thread's row: its position, and where its key and value go
+    int* s_page = reinterpret_cast<int*>(ft + BM * FS);     // [BM] page of the row's position, -1: none
+    int* s_prow = s_page + BM;                              // [BM] row of the position in that page
+    int* s_live = s_prow + BM;                              // [BM] block-table row (request) of the row, -1: none
+    const int m = m0 + tid;
+    const bool live = m < M;
+    const int p = live ? ep.pos[m] : 0;
+    const int hd = ep.hd, units = ep.n_head + 2 * ep.n_kv;
+    // the host reserves pages first; a row without one (-1) writes nothing
+    const int page = (live && ep.n_kv > 0) ? ep.table[(size_t)ep.slot[m] * ep.table_stride + p / ep.P] : -1;
+    s_page[tid] = page;
+    s_prow[tid] = p % ep.P;
+    s_live[tid] = live ? ep.slot[m] : -1;
+    __syncthreads();
+    for (int hh = 0; hh < BN / hd; ++hh) {
+      const int u = n0 / hd + hh;                            // the same in every thread
+      if (u >= units) break;
+      const float* src = ft + tid * FS + hh * hd;
+      const bool is_q = u < ep.n_head, is_v = u >= ep.n_head + ep.n_kv;
+      if (is_v) {
+        // values go in transposed, [dim][row of the page]: thread -> one dim, for runs of 16 rows of
+        // the tile; a run that is 16 consecutive rows of one page leaves as 32 contiguous bytes
+        const int kvh = u - ep.n_head - ep.n_kv;
+        const int d = tid % hd;
+        for (int r0 = (tid / hd) * 16; r0 < BM; r0 += (BM / hd) * 16) {
+          const int pg = s_page[r0], pr = s_prow[r0];
+          // rows of a run are consecutive positions of one request: its first and last row tell
+          bool run = (pg >= 0) & (pr % 16 == 0) & (s_page[r0 + 15] == pg) & (s_prow[r0 + 15] == pr + 15) &
+                     (s_live[r0] == s_live[r0 + 15]);
+          const float* col = ft + r0 * FS + hh * hd + d;
+          if (run) {
+            float v[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) v[j] = col[j * FS];
+            bf16_t* dst = kv_page_slot<bf16_t>(ep.pool, pg, 1, kvh, pr, ep.n_kv, ep.P, hd) + (size_t)d * ep.P;
+            *reinterpret_cast<uint4*>(dst) = make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]),
+                                                        pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
+            *reinterpret_cast<uint4*>(dst + 8) = make_uint4(pack_bf16x2(v[8], v[9]), pack_bf16x2(v[10], v[11]),
+                                                            pack_bf16x2(v[12], v[13]), pack_bf16x2(v[14], v[15]));
+          } else {
+            for (int j = 0; j < 16; ++j) {
+              const int pj = s_page[r0 + j];
+              if (pj >= 0)
+                kv_page_slot<bf16_t>(ep.pool, pj, 1, kvh, s_prow[r0 + j], ep.n_kv, ep.P, hd)[(size_t)d * ep.P] =
+                    f2bf(col[j * FS]);
+            }
+          }
+        }
+        continue;
+      }
+      if (!live) continue;
+      if (is_q) {
+        bf16_t* dst = ep.q_out + ((size_t)m * ep.n_head + u) * hd;
+        if (hd == 128)
+          qk_head_thread<128>(src, dst, ep.q_w, ep.eps, ep.inv_freq, ep.rope_table, ep.table_len, p);
+        else
+          qk_head_thread<64>(src, dst, ep.q_w, ep.eps, ep.inv_freq, ep.rope_table, ep.table_len, p);
+        continue;
+      }
+      if (page < 0) continue;
+      bf16_t* dst = kv_page_slot<bf16_t>(ep.pool, page, 0, u - ep.n_head, p % ep.P, ep.n_kv, ep.P, hd);
+      if (hd == 128)
+        qk_head_thread<128>(src, dst, ep.k_w, ep.eps, ep.inv_freq, ep.rope_table, ep.table_len, p);
+      else
+        qk_head_thread<64>(src, dst, ep.k_w, ep.eps, ep.inv_freq, ep.rope_table, ep.table_len, p);
+    }
+    return;
+  }
 #pragma unroll
   for (int a = 0; a < TM; ++a) {
 #pragma unroll
@@ -592,7 +698,46 @@ static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, 
   }
   const int bn = (EPI == TI_EPI_SWIGLU) ? BN / 2 : BN;
   dim3 grid((N + bn - 1) / bn, (M + BM - 1) / BM);
-  kernel<<<grid, 256, bytes, s>>>(A, W, out, M, N, K, lda);
+  kernel<<<grid, 256, bytes, s>>>(A, W, out, M, N, K, lda, QKVEpilogue{});
+  return 0;
+}
+
+// The fused q/k/v projection of a step's rows with the per-head work in its epilogue (see
+// QKVEpilogue): A [M, K] bf16, W [(n_head + 2 n_kv) hd, K] bf16 (n_kv = 0: q heads only, nothing is
+// written to the cache).  Returns 3 for what it does not serve: M <= 64, K not a multiple of 64,
+// head sizes other than 64 and 128.
+extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K, long lda, const float* q_w,
+                                     const float* k_w, float eps, const float* inv_freq, const float* rope_table,
+                                     int table_len, const int* pos, const int* slot, const int* table,
+                                     int table_stride, void* pool, void* q_out, int n_head, int n_kv, int hd,
+                                     int page_size, hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && K > 0 && lda >= K && n_head > 0 && n_kv >= 0 && hd > 0 && page_size > 0 && table_stride > 0,
+             "gemm_bf16_qkv_prep: bad sizes");
+  if (M <= 64 || K % 64 != 0 || lda % 8 != 0 || !(hd == 64 || hd == 128) || ((uintptr_t)A & 15) ||
+      ((uintptr_t)W & 15) || ((uintptr_t)q_out & 15) || ((uintptr_t)pool & 15) || ((uintptr_t)rope_table & 15)) {
+    ti_set_error("gemm_bf16_qkv_prep: M=%d K=%d head_dim=%d is not served (M > 64, K %% 64 == 0, head_dim 64 or 128)",
+                 M, K, hd);
+    return 3;
+  }
+  TI_REQUIRE(pos && slot && q_out && (n_kv == 0 || (table && pool)), "gemm_bf16_qkv_prep: a buffer is missing");
+  TI_REQUIRE(inv_freq || !rope_table, "gemm_bf16_qkv_prep: a sin/cos table without inv_freq");
+  QKVEpilogue ep{q_w, k_w, eps, inv_freq, (const float2*)rope_table, table_len, pos, slot, table, table_stride,
+                 (bf16_t*)pool, (bf16_t*)q_out, n_head, n_kv, hd, page_size};
+  const int N = (n_head + 2 * n_kv) * hd;
+  constexpr int BM = 256, BN = 128;
+  constexpr int bytes = PSTAGES * (BM + BN) * PBK * 2;
+  auto kernel = gemm_pipelined_kernel<BM, BN, 2, 2, TI_EPI_QKV_PREP>;
+  static bool ready = false;
+  if (!ready) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+      ti_set_error("gemm_bf16_qkv_prep: cannot reserve %d bytes of LDS", bytes);
+      return 2;
+    }
+    ready = true;
+  }
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
+  kernel<<<grid, 256, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, nullptr, M, N, K, lda, ep);
+  TI_LAUNCH_CHECK();
   return 0;
 }
 

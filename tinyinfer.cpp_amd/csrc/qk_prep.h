@@ -58,6 +58,68 @@ __device__ __forceinline__ void qk_head_wave(const float* __restrict__ src, T* _
   }
 }
 
+// One head by one thread, from hd floats at `src` (LDS or memory) to hd contiguous bfloat16 at
+// `dst` (16-byte aligned): the arithmetic of qk_head_wave with the sum of squares going up the
+// same tree as its butterfly (partners at distance 32, 16, ..., 1), so the bits are the same.
+// Eight pairs at a time: their angles come in as four 16-byte loads, their results leave as two.
+template <int HD>
+__device__ __forceinline__ void qk_head_thread(const float* src, bf16_t* dst, const float* w, float eps,
+                                               const float* inv_freq, const float2* rope_table, int table_len,
+                                               int p) {
+  constexpr int HALF = HD / 2;
+  static_assert(HALF == 32 || HALF == 64, "the tree below is that of a 64-lane butterfly with one pair a lane");
+  float scale = 1.f;
+  if (w) {
+    float t[HALF];
+#pragma unroll
+    for (int i = 0; i < HALF; ++i) t[i] = qk_pair_square(src[i], src[i + HALF]);
+#pragma unroll
+    for (int o = HALF / 2; o >= 1; o >>= 1)
+#pragma unroll
+      for (int i = 0; i < o; ++i) t[i] += t[i + o];
+    scale = qk_norm_scale(t[0], HD, eps);
+  }
+  auto run_of_eight = [&](int c, const float2* cs) {
+    float lo[8], hi[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      lo[j] = src[c + j] * scale;
+      hi[j] = src[c + j + HALF] * scale;
+      if (w) {
+        lo[j] *= w[c + j];
+        hi[j] *= w[c + j + HALF];
+      }
+      if (inv_freq) qk_rotate(lo[j], hi[j], cs[j]);
+    }
+    *reinterpret_cast<uint4*>(dst + c) = make_uint4(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]),
+                                                    pack_bf16x2(lo[4], lo[5]), pack_bf16x2(lo[6], lo[7]));
+    *reinterpret_cast<uint4*>(dst + c + HALF) = make_uint4(pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3]),
+                                                           pack_bf16x2(hi[4], hi[5]), pack_bf16x2(hi[6], hi[7]));
+  };
+  if (inv_freq && rope_table && p < table_len) {
+    // all angles of the row at once (sixteen-byte loads that do not wait for one another)
+    float2 cs[HALF];
+    const float4* tp = reinterpret_cast<const float4*>(rope_table + (size_t)p * HALF);
+#pragma unroll
+    for (int h = 0; h < HALF / 2; ++h) {
+      const float4 v = tp[h];
+      cs[2 * h] = make_float2(v.x, v.y);
+      cs[2 * h + 1] = make_float2(v.z, v.w);
+    }
+#pragma unroll
+    for (int c = 0; c < HALF; c += 8) run_of_eight(c, cs + c);
+  } else {
+    for (int c = 0; c < HALF; c += 8) {
+      float2 cs[8];
+      if (inv_freq) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) cs[j] = qk_cos_sin(c + j, HALF, p, inv_freq, nullptr, 0);
+      }
+      run_of_eight(c, cs);
+    }
+  }
+}
+
 // A value head: copied (rounded to T), element d to dst[d * dst_stride]
 template <typename T>
 __device__ __forceinline__ void v_head_wave(const float* __restrict__ src, T* __restrict__ dst, size_t dst_stride,

@@ -66,6 +66,7 @@ class Ops:
         self.use_fast_attention = have("attention_bf16")
         self.use_fused_norm = True       # the norm before a product inside the product's kernel (few tokens)
         self.use_fused_qk_decode = True  # per-head norm, rotation and cache write inside the decode attention
+        self.use_fused_qkv_prefill = True  # the same in the epilogue of the q/k/v product (steps of many tokens)
 
     # ------------------------------------------------------------------ loading
     def lib(self, name: str) -> ctypes.CDLL:
@@ -217,6 +218,48 @@ class Ops:
         rc = lib.ti_gemm_generic(code, _ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi,
                                  self._stream())
         self._check(lib, rc, "linear")
+
+    def qkv_prepared(self, a, w, q_w, k_w, eps, inv_freq, rope_table, positions, slots, view, pool, q_out,
+                     heads, kv_heads, head_dim) -> bool:
+        """`linear(a, w, qkv, "store")` and `qk_norm_rope_kv_write` in one kernel, for steps of many
+        tokens in bfloat16: w is [(heads + 2 kv_heads) hd, K] (kv_heads = 0: q heads only).  False if
+        no kernel serves the step; then nothing has been done and the caller makes the two calls."""
+        if not (self.use_fused_qkv_prefill and self.use_fast_gemm) or isinstance(a, NormedRows):
+            return False
+        if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or q_out.dtype != torch.bfloat16:
+            return False
+        M, K = a.shape
+        N = (heads + 2 * kv_heads) * head_dim
+        self._dev(a, w, q_w, k_w, inv_freq, rope_table, positions, slots, view.table, pool, q_out)
+        if w.shape != (N, K) or a.stride(1) != 1 or not w.is_contiguous():
+            raise KernelError(f"qkv_prepared: a {tuple(a.shape)} and w {tuple(w.shape)} do not fit {N} rows of heads")
+        if q_out.shape != (M, heads * head_dim) or not q_out.is_contiguous():
+            raise KernelError("qkv_prepared: q_out has the wrong shape")
+        if positions.shape[0] != M or slots.shape[0] != M or positions.dtype != torch.int32 or slots.dtype != torch.int32:
+            raise KernelError("qkv_prepared: positions and slots must be int32 [M]")
+        for wt in (q_w, k_w):
+            if wt is not None and (wt.shape != (head_dim,) or wt.dtype != torch.float32):
+                raise KernelError("qkv_prepared: norm weights must be float32 [head_dim]")
+        if inv_freq is not None and (inv_freq.shape != (head_dim // 2,) or inv_freq.dtype != torch.float32):
+            raise KernelError("qkv_prepared: inv_freq must be float32 [head_dim/2]")
+        if rope_table is not None and (rope_table.dtype != torch.float32 or not rope_table.is_contiguous()
+                                       or rope_table.shape[1:] != (head_dim // 2, 2)):
+            raise KernelError("qkv_prepared: the sin/cos table must be float32 [positions, head_dim/2, 2]")
+        if kv_heads > 0 and (pool.dim() != 5 or pool.shape[1] != 2 or pool.shape[2] != kv_heads
+                             or pool.shape[4] != head_dim or pool.dtype != torch.bfloat16
+                             or not pool.is_contiguous() or not view.table.is_contiguous()):
+            raise KernelError(f"qkv_prepared: pool {tuple(pool.shape)} {pool.dtype} does not fit "
+                              f"[pages,2,{kv_heads},P,{head_dim}] of bfloat16")
+        lib = self.lib("gemm_bf16")
+        rc = lib.ti_gemm_bf16_qkv_prep(
+            _ptr(a), _ptr(w), M, K, ctypes.c_long(a.stride(0)), _ptr(q_w), _ptr(k_w), ctypes.c_float(eps),
+            _ptr(inv_freq), _ptr(rope_table), 0 if rope_table is None else rope_table.shape[0],
+            _ptr(positions), _ptr(slots), _ptr(view.table), view.table.shape[1], _ptr(pool), _ptr(q_out),
+            heads, kv_heads, head_dim, pool.shape[3], self._stream())
+        if rc == 3:
+            return False
+        self._check(lib, rc, "qkv_prepared")
+        return True
 
     NORMED_MAX_ROWS = 16
 

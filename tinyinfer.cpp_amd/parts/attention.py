@@ -82,15 +82,25 @@ class Attention(Part):
     def forward(self, ctx, h, x):
         M = h.shape[0]
         width = self.nq + 2 * self.nk
-        qkv = ctx.buf("attn.qkv", (M, width), ctx.f32)
-        ctx.ops.linear(h, self.w_qkv, qkv, "store")
         q = ctx.buf("attn.q", (M, self.nq), ctx.act_dtype)
         group, layer = ctx.binding(self)
         pool = ctx.kv_pool(group, layer)
         view = ctx.cache_view(group)
         rot = self.pos.fused_rotation() if self.pos is not None and hasattr(self.pos, "fused_rotation") else None
         a = ctx.buf("attn.out", (M, self.nq), ctx.act_dtype)
-        if (self.pos is None or rot is not None) and ctx.ops.attention_from_projections(
+        fusable = self.pos is None or rot is not None     # a position encoding without a fused form needs qkv
+        if fusable and not ctx.decode_only and ctx.ops.qkv_prepared(
+                h, self.w_qkv, self.q_norm_w, self.k_norm_w, self.eps,
+                None if rot is None else rot["inv_freq"], None if rot is None else rot.get("table"),
+                ctx.positions, ctx.slots, view, pool, q, self.heads,
+                0 if self.shares_kv else self.kv_heads, self.head_dim):
+            # a step of many tokens: the projection's epilogue prepared q and wrote the cache
+            ctx.ops.attention(ctx, view, q, pool, a, self.heads, self.kv_heads, self.head_dim, self.scale, self.window)
+            ctx.ops.linear(a, self.w_o, x, "add")
+            return
+        qkv = ctx.buf("attn.qkv", (M, width), ctx.f32)
+        ctx.ops.linear(h, self.w_qkv, qkv, "store")
+        if fusable and ctx.ops.attention_from_projections(
                 ctx, view, qkv, self.q_norm_w, self.k_norm_w, self.eps,
                 None if rot is None else rot["inv_freq"], None if rot is None else rot.get("table"),
                 pool, not self.shares_kv, a, self.heads, self.kv_heads, self.head_dim, self.scale, self.window):
