@@ -441,16 +441,18 @@ struct QKVEpilogue {
 };
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_,
                       int M, int N, int K, long lda, QKVEpilogue ep = QKVEpilogue{}) {
   constexpr bool SW = (EPI == TI_EPI_SWIGLU);
   constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
-  static_assert(WAVES_M * WAVES_N == 4, "four wavefronts");
+  constexpr int NWV = WAVES_M * WAVES_N;                     // wavefronts: 4 or 8
+  static_assert(NWV == 4 || NWV == 8, "four or eight wavefronts");
   static_assert(!SW || TN == 2, "SwiGLU pairs two column tiles per wavefront");
   constexpr int STAGE_BYTES = (BM + BN) * PBK * 2;
   constexpr int GROUPS_A = BM / 8, GROUPS_B = BN / 8;        // 8 rows = 1 KiB = one wavefront load
-  constexpr int LOADS = (GROUPS_A + GROUPS_B) / 4;           // per wavefront and k-tile
+  static_assert((GROUPS_A + GROUPS_B) % NWV == 0, "every wavefront issues the same number of loads");
+  constexpr int LOADS = (GROUPS_A + GROUPS_B) / NWV;         // per wavefront and k-tile
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -465,7 +467,7 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
   int gpiece[LOADS];                                         // which 8-element piece of the row this lane fetches
 #pragma unroll
   for (int i = 0; i < LOADS; ++i) {
-    const int g = wave + 4 * i;                              // groups 0..GROUPS_A-1: A, then B
+    const int g = wave + NWV * i;                            // groups 0..GROUPS_A-1: A, then B
     if (g < GROUPS_A) {
       const int row = g * 8 + lr;
       const int gm = min(m0 + row, M - 1);
@@ -491,7 +493,7 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
     const int k0 = kt * PBK;
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
-      const int g = wave + 4 * i;
+      const int g = wave + NWV * i;
       unsigned char* dst = stage + g * 1024;                 // the same in every lane
       // K is a multiple of 64 here (the dispatcher sees to it): no piece lies past the end
       __builtin_amdgcn_global_load_lds(
@@ -595,15 +597,18 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
     int* s_prow = s_page + BM;                              // [BM] row of the position in that page
     int* s_live = s_prow + BM;                              // [BM] block-table row (request) of the row, -1: none
     const int m = m0 + tid;
-    const bool live = m < M;
+    const bool live = tid < BM && m < M;                    // (eight wavefronts: the upper four have no row)
     const int p = live ? ep.pos[m] : 0;
     const int hd = ep.hd, units = ep.n_head + 2 * ep.n_kv;
     // the host reserves pages first; a row without one (-1) writes nothing
     const int page = (live && ep.n_kv > 0) ? ep.table[(size_t)ep.slot[m] * ep.table_stride + p / ep.P] : -1;
-    s_page[tid] = page;
-    s_prow[tid] = p % ep.P;
-    s_live[tid] = live ? ep.slot[m] : -1;
+    if (tid < BM) {
+      s_page[tid] = page;
+      s_prow[tid] = p % ep.P;
+      s_live[tid] = live ? ep.slot[m] : -1;
+    }
     __syncthreads();
+    if (tid >= BM) return;
     for (int hh = 0; hh < BN / hd; ++hh) {
       const int u = n0 / hd + hh;                            // the same in every thread
       if (u >= units) break;
@@ -698,7 +703,7 @@ static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, 
   }
   const int bn = (EPI == TI_EPI_SWIGLU) ? BN / 2 : BN;
   dim3 grid((N + bn - 1) / bn, (M + BM - 1) / BM);
-  kernel<<<grid, 256, bytes, s>>>(A, W, out, M, N, K, lda, QKVEpilogue{});
+  kernel<<<grid, WAVES_M * WAVES_N * 64, bytes, s>>>(A, W, out, M, N, K, lda, QKVEpilogue{});
   return 0;
 }
 
@@ -726,7 +731,7 @@ extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K,
   const int N = (n_head + 2 * n_kv) * hd;
   constexpr int BM = 256, BN = 128;
   constexpr int bytes = PSTAGES * (BM + BN) * PBK * 2;
-  auto kernel = gemm_pipelined_kernel<BM, BN, 2, 2, TI_EPI_QKV_PREP>;
+  auto kernel = gemm_pipelined_kernel<BM, BN, 4, 2, TI_EPI_QKV_PREP>;
   static bool ready = false;
   if (!ready) {
     if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
@@ -736,19 +741,27 @@ extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K,
     ready = true;
   }
   dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
-  kernel<<<grid, 256, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, nullptr, M, N, K, lda, ep);
+  kernel<<<grid, 512, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, nullptr, M, N, K, lda, ep);
   TI_LAUNCH_CHECK();
   return 0;
 }
 
-// the largest tile that still gives every compute unit a workgroup
+// for measurements: 0 = choose the tile by the shape, 1 = 256 x 128 (eight wavefronts), 3 = 128 x 64 (four)
+static int g_force_tile = 0;
+extern "C" void ti_gemm_bf16_force_tile(int which) { g_force_tile = which; }
+
+// Two tiles.  256 x 128 with eight wavefronts does the most per byte it loads, one workgroup
+// to a compute unit: it is taken when its workgroups come in (nearly) whole rounds of the 256
+// units or in many rounds.  Otherwise 128 x 64 with four wavefronts, two workgroups to a unit,
+// whose small tiles fill the chip evenly for every shape.
 template <int EPI>
 static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
                              hipStream_t s) {
   const int cols = (EPI == TI_EPI_SWIGLU) ? 2 : 1;   // a SwiGLU workgroup covers BN / 2 output columns
-  auto count = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N * cols + bn - 1) / bn); };
-  if (count(256, 128) >= 256) return launch_pipelined<256, 128, 2, 2, EPI>(A, W, out, M, N, K, lda, s);
-  if (count(128, 128) >= 256) return launch_pipelined<128, 128, 2, 2, EPI>(A, W, out, M, N, K, lda, s);
+  const long big = (long)((M + 255) / 256) * ((N * cols + 127) / 128);
+  const bool whole_rounds = big >= 256 && (big % 256 == 0 || big % 256 >= 192);
+  const bool use_big = g_force_tile ? g_force_tile == 1 : (big >= 1024 || whole_rounds);
+  if (use_big) return launch_pipelined<256, 128, 4, 2, EPI>(A, W, out, M, N, K, lda, s);
   return launch_pipelined<128, 64, 4, 1, EPI>(A, W, out, M, N, K, lda, s);
 }
 
