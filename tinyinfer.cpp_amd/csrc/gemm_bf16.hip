@@ -555,6 +555,8 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
         if (TM + TN == 6) asm volatile("s_waitcnt lgkmcnt(6)" ::: "memory");
         if (TM + TN == 4) asm volatile("s_waitcnt lgkmcnt(4)" ::: "memory");
         if (TM + TN == 3) asm volatile("s_waitcnt lgkmcnt(3)" ::: "memory");
+        if (TM + TN == 2) asm volatile("s_waitcnt lgkmcnt(2)" ::: "memory");
+        static_assert(TM + TN == 6 || TM + TN == 4 || TM + TN == 3 || TM + TN == 2, "a wait for every tile shape");
       } else {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       }
@@ -746,22 +748,26 @@ extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K,
   return 0;
 }
 
-// for measurements: 0 = choose the tile by the shape, 1 = 256 x 128 (eight wavefronts), 3 = 128 x 64 (four)
+// for measurements: 0 = choose the tile by the shape, 1 = 256 x 128, 3 = 128 x 64, 6 = 64 x 64
 static int g_force_tile = 0;
 extern "C" void ti_gemm_bf16_force_tile(int which) { g_force_tile = which; }
 
-// Two tiles.  256 x 128 with eight wavefronts does the most per byte it loads, one workgroup
+// Three tiles.  256 x 128 with eight wavefronts does the most per byte it loads, one workgroup
 // to a compute unit: it is taken when its workgroups come in (nearly) whole rounds of the 256
-// units or in many rounds.  Otherwise 128 x 64 with four wavefronts, two workgroups to a unit,
-// whose small tiles fill the chip evenly for every shape.
+// units or in many rounds.  Otherwise 128 x 64 with four wavefronts, two workgroups to a unit;
+// and where even those are fewer than two to a unit, 64 x 64 (three to a unit).
 template <int EPI>
 static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
                              hipStream_t s) {
   const int cols = (EPI == TI_EPI_SWIGLU) ? 2 : 1;   // a SwiGLU workgroup covers BN / 2 output columns
   const long big = (long)((M + 255) / 256) * ((N * cols + 127) / 128);
+  const long mid = (long)((M + 127) / 128) * ((N * cols + 63) / 64);
   const bool whole_rounds = big >= 256 && (big % 256 == 0 || big % 256 >= 192);
-  const bool use_big = g_force_tile ? g_force_tile == 1 : (big >= 1024 || whole_rounds);
-  if (use_big) return launch_pipelined<256, 128, 4, 2, EPI>(A, W, out, M, N, K, lda, s);
+  int tile = (big >= 1024 || whole_rounds) ? 1 : (mid >= 512 ? 3 : 6);
+  if (g_force_tile) tile = g_force_tile;
+  if (tile == 1) return launch_pipelined<256, 128, 4, 2, EPI>(A, W, out, M, N, K, lda, s);
+  if constexpr (EPI != TI_EPI_SWIGLU)                // a SwiGLU wavefront needs two column tiles
+    if (tile == 6) return launch_pipelined<64, 64, 2, 2, EPI>(A, W, out, M, N, K, lda, s);
   return launch_pipelined<128, 64, 4, 1, EPI>(A, W, out, M, N, K, lda, s);
 }
 
