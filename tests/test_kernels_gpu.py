@@ -173,6 +173,28 @@ def test_qk_norm_rope_kv_write(ops, dtype, hd, nh, nkv, P, table_len):
 
 
 # -------------------------------------------------------------- matrix products
+def test_qk_norm_in_place(ops):
+    """The per-head norm alone, in place on 32-bit projections: the same numbers as the fused
+    kernel produces without rotation, value heads untouched, a missing weight leaves heads alone."""
+    g = torch.Generator().manual_seed(12)
+    M, nh, nkv, hd = 7, 3, 2, 48
+    qkv = torch.randn(M, (nh + 2 * nkv) * hd, generator=g) * 2
+    q_w, k_w = 1 + 0.1 * torch.randn(hd, generator=g), 1 + 0.1 * torch.randn(hd, generator=g)
+    x = dev(qkv.clone())
+    ops.qk_norm_inplace(x, dev(q_w), dev(k_w), 1e-3, nh, nkv, hd)
+    want = f64(qkv).clone()
+    for u in range(nh + nkv):
+        h = want[:, u * hd:(u + 1) * hd]
+        w = f64(q_w) if u < nh else f64(k_w)
+        want[:, u * hd:(u + 1) * hd] = h / torch.sqrt((h * h).mean(-1, keepdim=True) + 1e-3) * w
+    assert (f64(x) - want).abs().max() < 1e-5
+    assert torch.equal(x[:, (nh + nkv) * hd:].cpu(), qkv[:, (nh + nkv) * hd:])
+    y = dev(qkv.clone())
+    ops.qk_norm_inplace(y, None, dev(k_w), 1e-3, nh, nkv, hd)
+    assert torch.equal(y[:, :nh * hd].cpu(), qkv[:, :nh * hd])
+    assert torch.equal(y[:, nh * hd:], x[:, nh * hd:])
+
+
 def ref_linear(a, w):
     return f64(a) @ f64(w).T
 

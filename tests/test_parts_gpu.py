@@ -1,7 +1,7 @@
 """Each part alone against its plain function, and parts that are defined here,
-in the test: a mixer with state of its own, a block arrangement, an architecture.
-They are registered, built, loaded and stepped without a change to the
-framework's files."""
+in the test: a mixer with state of its own, a feed-forward with routing, another
+position encoding, a block arrangement, an architecture.  They are registered,
+built, loaded and stepped without a change to the framework's files."""
 import json
 import math
 import os
@@ -169,6 +169,57 @@ def register_toys():
         def forward(self, ctx, x):
             self.mixer.forward(ctx, x.to(ctx.act_dtype, copy=True), x)
 
+    class RoutedFFN(Part):
+        """A feed-forward with routing: the expert with the largest router logit takes the
+        token, out = softmax(router)[e] * W2[e] relu(W1[e] h).  Router logits in 32-bit."""
+        family = "ffn"
+
+        def __init__(self, prefix, hidden, inner, experts):
+            super().__init__(prefix)
+            self.hidden, self.inner, self.experts = hidden, inner, experts
+
+        def tensors(self):
+            H, F, E = self.hidden, self.inner, self.experts
+            return {join(self.prefix, "router"): TensorNeed((E, H), "vector", ("normal", 0.0, 0.5)),
+                    join(self.prefix, "w1"): TensorNeed((E, F, H), "matrix", ("normal", 0.0, 0.2)),
+                    join(self.prefix, "w2"): TensorNeed((E, H, F), "matrix", ("normal", 0.0, 0.2))}
+
+        def load(self, tensors):
+            self.router = tensors[join(self.prefix, "router")]
+            self.w1 = tensors[join(self.prefix, "w1")]
+            self.w2 = tensors[join(self.prefix, "w2")]
+
+        def forward(self, ctx, h, x):
+            hf = h.float()
+            prob = torch.softmax(hf @ self.router.T, dim=-1)
+            top = prob.argmax(dim=-1)
+            for e in range(self.experts):
+                rows = (top == e).nonzero().flatten()
+                if rows.numel():
+                    y = torch.relu(hf[rows] @ self.w1[e].float().T) @ self.w2[e].float().T
+                    x[rows] += prob[rows, e:e + 1] * y
+
+    class PairRotary(Part):
+        """Another position encoding: neighbours (2i, 2i + 1) rotate together.  It has no fused
+        form, so the attention part calls `apply` on its 32-bit projections."""
+        family = "pos"
+
+        def __init__(self, prefix, head_dim, theta):
+            super().__init__(prefix)
+            self.head_dim, self.theta = head_dim, theta
+
+        def apply(self, ctx, q, k):
+            half = self.head_dim // 2
+            inv = self.theta ** (-torch.arange(half, dtype=torch.float64, device=q.device) * 2 / self.head_dim)
+            ang = ctx.positions.double()[:, None] * inv[None, :]
+            cos, sin = ang.cos().float()[:, None, :], ang.sin().float()[:, None, :]
+            for t in (q, k):
+                if t is None:
+                    continue
+                a, b = t[..., 0::2].clone(), t[..., 1::2].clone()
+                t[..., 0::2] = a * cos - b * sin
+                t[..., 1::2] = a * sin + b * cos
+
     def read(d):
         return dict(d)
 
@@ -179,9 +230,19 @@ def register_toys():
                                       "window": c.get("window"),
                                       "pos": PartSpec("rope_neox", {"head_dim": c["head_dim"], "theta": c["theta"]})
                                       if c["rotate"] else None}, "attn")
+        pair_attn = PartSpec("attention", {"hidden": H, "heads": c["heads"], "kv_heads": c["kv_heads"],
+                                           "head_dim": c["head_dim"], "qk_norm": c["qk_norm"], "eps": c["eps"],
+                                           "window": c.get("window"),
+                                           "pos": PartSpec("toy_pair_rotary", {"head_dim": c["head_dim"],
+                                                                               "theta": c["theta"]})}, "attn")
         layers = []
         for i, kind in enumerate(c["layers"]):
-            if kind == "decay":
+            if kind == "routed":
+                layers.append(LayerSpec(f"l.{i}", PartSpec("pre_norm"), {
+                    "norm1": PartSpec("rmsnorm", {"dim": H, "eps": c["eps"]}, "n1"), "mixer": pair_attn,
+                    "norm2": PartSpec("rmsnorm", {"dim": H, "eps": c["eps"]}, "n2"),
+                    "ffn": PartSpec("toy_routed", {"hidden": H, "inner": c["ff"], "experts": c["experts"]}, "moe")}))
+            elif kind == "decay":
                 layers.append(LayerSpec(f"l.{i}", PartSpec("bare"), {
                     "mixer": PartSpec("toy_decay", {"hidden": H, "decay": c["decay"]}, "mix")}))
             elif kind == "bare_attention":
@@ -197,12 +258,25 @@ def register_toys():
                          schedule=c.get("schedule"))
 
     ti.register_part("mixer", "toy_decay", DecayMixer)
+    ti.register_part("ffn", "toy_routed", RoutedFFN)
+    ti.register_part("pos", "toy_pair_rotary", PairRotary)
     ti.register_part("block", "bare", BareBlock)
     ti.register_architecture("ToyLM", read, spec_of)
 
 
 TOY = dict(architectures=["ToyLM"], vocab=90, hidden=32, heads=2, kv_heads=1, head_dim=16, ff=48, eps=1e-5,
            theta=1e4, decay=0.8, qk_norm=True, rotate=True, layers=["decay", "full", "decay"])
+
+
+def pair_rotation(x, theta):
+    """x [T, heads, hd]: dims (2i, 2i + 1) of position t rotate by t * theta^(-2i/hd)."""
+    T, _, hd = x.shape
+    ang = np.arange(T)[:, None] * theta ** (-np.arange(hd // 2) * 2.0 / hd)[None, :]
+    cos, sin = np.cos(ang)[:, None, :], np.sin(ang)[:, None, :]
+    out = np.empty_like(x)
+    out[..., 0::2] = x[..., 0::2] * cos - x[..., 1::2] * sin
+    out[..., 1::2] = x[..., 0::2] * sin + x[..., 1::2] * cos
+    return out
 
 
 def toy_plain(cfg, w, toks):
@@ -222,7 +296,7 @@ def toy_plain(cfg, w, toks):
                 out[t] = s
             x = x + out
         else:
-            full = kind == "full"
+            full = kind in ("full", "routed")
             h = plain.rms_norm(x, w[p + ".n1.weight"], cfg["eps"]) if full else x
             a = p + ".attn"
             q = plain.linear(h, w[a + ".q_proj.weight"]).reshape(T, cfg["heads"], cfg["head_dim"])
@@ -231,11 +305,23 @@ def toy_plain(cfg, w, toks):
             if cfg["qk_norm"]:
                 q = plain.qk_norm(q, w[a + ".q_norm.weight"], cfg["eps"])
                 k = plain.qk_norm(k, w[a + ".k_norm.weight"], cfg["eps"])
-            if cfg["rotate"]:
+            if kind == "routed":
+                q, k = pair_rotation(q, cfg["theta"]), pair_rotation(k, cfg["theta"])
+            elif cfg["rotate"]:
                 q, k = plain.rope_neox(q, range(T), cfg["theta"]), plain.rope_neox(k, range(T), cfg["theta"])
             o = plain.attention(q, k, v, cfg.get("window")).reshape(T, -1)
             x = x + plain.linear(o, w[a + ".o_proj.weight"])
-            if full:
+            if kind == "routed":
+                h = plain.rms_norm(x, w[p + ".n2.weight"], cfg["eps"])
+                logit = h @ w[p + ".moe.router"].T
+                prob = np.exp(logit - logit.max(-1, keepdims=True))
+                prob /= prob.sum(-1, keepdims=True)
+                out = np.zeros_like(x)
+                for t in range(T):
+                    e = int(prob[t].argmax())
+                    out[t] = prob[t, e] * (w[p + ".moe.w2"][e] @ np.maximum(w[p + ".moe.w1"][e] @ h[t], 0.0))
+                x = x + out
+            elif full:
                 h = plain.rms_norm(x, w[p + ".n2.weight"], cfg["eps"])
                 x = x + plain.ffn_block(h, w, p + ".ffn", plain.no_rounding)
     return plain.linear(plain.rms_norm(x, w["norm.weight"], cfg["eps"]), w["emb.weight"])
@@ -322,3 +408,34 @@ def test_run_order_may_name_a_layer_twice(tmp_path):
     got = np.concatenate([engine.step([ti.StepEntry("r", toks[a:b], list(range(b - a)))]).cpu().numpy()
                           for a, b in ((0, 11), (11, 12), (12, 30))])
     assert np.abs(got - toy_plain(cfg, w, toks)).max() < 2e-4
+
+
+def test_toy_routed_feed_forward_and_another_position_encoding(tmp_path):
+    """A feed-forward that routes tokens to experts and a position encoding that rotates
+    neighbouring dims (no fused form: the attention part applies it to its 32-bit
+    projections), defined above in this file, beside the built-in parts: portions and single
+    tokens of two requests in one batch against the whole-sequence numpy model."""
+    import tinyinfer_amd as ti
+    cfg = dict(TOY, layers=["routed", "full", "routed"], experts=3, ff=40, heads=4, kv_heads=2)
+    engine, w = toy_engine(tmp_path, cfg)
+    assert [type(b.ffn).__name__ for b in engine.model.blocks] == ["RoutedFFN", "SwiGLU", "RoutedFFN"]
+    assert type(engine.model.blocks[0].mixer.pos).__name__ == "PairRotary"
+    reqs = {"a": random_tokens(37, 90, 21), "b": random_tokens(26, 90, 22)}
+    want = {r: toy_plain(cfg, w, t) for r, t in reqs.items()}
+    # every expert is used by some token (else the routing is not tested)
+    got = {r: [] for r in reqs}
+
+    def run(*cuts):
+        entries = [ti.StepEntry(r, reqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in cuts]
+        logits = engine.step(entries).cpu().numpy()
+        i = 0
+        for e in entries:
+            got[e.request].append(logits[i:i + len(e.tokens)])
+            i += len(e.tokens)
+
+    run(("a", 0, 18), ("b", 0, 1))
+    run(("a", 18, 19), ("b", 1, 20))
+    run(("b", 20, 21), ("a", 19, 37))
+    run(("b", 21, 26))
+    for r in reqs:
+        assert np.abs(np.concatenate(got[r]) - want[r]).max() < 2e-4, r

@@ -225,3 +225,43 @@ extern "C" int ti_qk_norm_rope_kv_write(int dtype, const float* qkv, const float
   TI_LAUNCH_CHECK();
   return 0;
 }
+
+// The per-head norm alone, in place on the 32-bit projections (rows of `row_width` floats: q heads,
+// then k heads): for a position encoding that has no fused form and must see normed heads.
+// Grid (M, ceil(units / 4)), a wavefront per (token, head); a weight that is nullptr leaves its
+// heads as they are.
+__global__ void __launch_bounds__(256)
+qk_norm_inplace_kernel(float* qkv, int row_width, const float* __restrict__ q_w,
+                       const float* __restrict__ k_w, int n_head, int n_kv, int hd, float eps) {
+  const int m = blockIdx.x;
+  const int u = blockIdx.y * (blockDim.x / TI_WAVE) + threadIdx.x / TI_WAVE;
+  if (u >= n_head + n_kv) return;
+  const float* w = u < n_head ? q_w : k_w;
+  if (!w) return;
+  float* head = qkv + (size_t)m * row_width + (size_t)u * hd;
+  // the arithmetic of qk_head_wave without a rotation; each lane reads its own elements before it
+  // writes them
+  const int lane = threadIdx.x % TI_WAVE, half = hd / 2;
+  float ss = 0.f;
+  for (int i = lane; i < half; i += TI_WAVE) ss += qk_pair_square(head[i], head[i + half]);
+  const float scale = qk_norm_scale(group_sum<TI_WAVE>(ss), hd, eps);
+  for (int i = lane; i < half; i += TI_WAVE) {
+    float lo = head[i] * scale, hi = head[i + half] * scale;
+    lo *= w[i];
+    hi *= w[i + half];
+    head[i] = lo;
+    head[i + half] = hi;
+  }
+}
+
+extern "C" int ti_qk_norm_inplace(float* qkv, int row_width, const float* q_w, const float* k_w, int M, int n_head,
+                                  int n_kv, int hd, float eps, hipStream_t stream) {
+  TI_REQUIRE(hd > 0 && hd % 2 == 0 && n_head > 0 && n_kv >= 0 && row_width >= (n_head + n_kv) * hd,
+             "qk_norm_inplace: bad sizes heads=%d kv_heads=%d head_dim=%d row_width=%d", n_head, n_kv, hd, row_width);
+  if (M == 0) return 0;
+  const int units = n_head + n_kv;
+  TI_REQUIRE((units + 3) / 4 <= 65535, "qk_norm_inplace: too many heads");
+  qk_norm_inplace_kernel<<<dim3(M, (units + 3) / 4), 256, 0, stream>>>(qkv, row_width, q_w, k_w, n_head, n_kv, hd, eps);
+  TI_LAUNCH_CHECK();
+  return 0;
+}

@@ -188,6 +188,22 @@ class Ops:
             pool.shape[3], ctypes.c_float(eps), self._stream())
         self._check(lib, rc, "qk_norm_rope_kv_write")
 
+    def qk_norm_inplace(self, qkv, q_w, k_w, eps, heads, kv_heads, head_dim):
+        """Per-head RMSNorm of the q heads (and the k heads behind them) of f32 qkv [M, width], in
+        place; a weight that is None leaves its heads alone."""
+        self._dev(qkv, q_w, k_w)
+        if qkv.dim() != 2 or qkv.dtype != torch.float32 or not qkv.is_contiguous() \
+                or qkv.shape[1] < (heads + kv_heads) * head_dim:
+            raise KernelError(f"qk_norm_inplace: qkv {tuple(qkv.shape)} {qkv.dtype} does not hold "
+                              f"{heads} + {kv_heads} heads of {head_dim}")
+        for wt in (q_w, k_w):
+            if wt is not None and (wt.shape != (head_dim,) or wt.dtype != torch.float32):
+                raise KernelError("qk_norm_inplace: norm weights must be float32 [head_dim]")
+        lib = self.lib("core")
+        rc = lib.ti_qk_norm_inplace(_ptr(qkv), qkv.shape[1], _ptr(q_w), _ptr(k_w), qkv.shape[0], heads, kv_heads,
+                                    head_dim, ctypes.c_float(eps), self._stream())
+        self._check(lib, rc, "qk_norm_inplace")
+
     # ---------------------------------------------------------- matrix products
     def linear(self, a, w, out, epilogue: str):
         """out (op)= a w^T.  a: T [M, K] (rows may be strided); w: T [N, K] contiguous.

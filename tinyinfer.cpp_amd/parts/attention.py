@@ -106,13 +106,19 @@ class Attention(Part):
                 pool, not self.shares_kv, a, self.heads, self.kv_heads, self.head_dim, self.scale, self.window):
             ctx.ops.linear(a, self.w_o, x, "add")        # a step of single tokens: one kernel did it all
             return
+        q_w, k_w = self.q_norm_w, self.k_norm_w
         if self.pos is not None and rot is None:
-            # a position encoding without a fused form runs on the 32-bit projections first
+            # a position encoding without a fused form works on the 32-bit projections, after the
+            # per-head norm (as in the fused order: norm, then position)
+            n_k = 0 if self.shares_kv else self.kv_heads
+            if q_w is not None or k_w is not None:
+                ctx.ops.qk_norm_inplace(qkv, q_w, k_w, self.eps, self.heads, n_k, self.head_dim)
+                q_w = k_w = None
             qv = qkv[:, :self.nq].unflatten(1, (self.heads, self.head_dim))
             kv = None if self.shares_kv else qkv[:, self.nq:self.nq + self.nk].unflatten(1, (self.kv_heads, self.head_dim))
             self.pos.apply(ctx, qv, kv)
         ctx.ops.qk_norm_rope_kv_write(
-            qkv, self.q_norm_w, self.k_norm_w, self.eps,
+            qkv, q_w, k_w, self.eps,
             None if rot is None else rot["inv_freq"],
             ctx.positions, ctx.slots, view, pool, q,
             self.heads, 0 if self.shares_kv else self.kv_heads, self.head_dim,
