@@ -584,14 +584,10 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
 __device__ __forceinline__ void lgkm_wait(int n) {
   switch (n) {
-    case 0: asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); break;
-    case 1: asm volatile("s_waitcnt lgkmcnt(1)" ::: "memory"); break;
-    case 2: asm volatile("s_waitcnt lgkmcnt(2)" ::: "memory"); break;
-    case 3: asm volatile("s_waitcnt lgkmcnt(3)" ::: "memory"); break;
-    case 4: asm volatile("s_waitcnt lgkmcnt(4)" ::: "memory"); break;
-    case 5: asm volatile("s_waitcnt lgkmcnt(5)" ::: "memory"); break;
-    case 6: asm volatile("s_waitcnt lgkmcnt(6)" ::: "memory"); break;
-    case 7: asm volatile("s_waitcnt lgkmcnt(7)" ::: "memory"); break;
+#define TI_LGKM(N) case N: asm volatile("s_waitcnt lgkmcnt(" #N ")" ::: "memory"); break;
+    TI_LGKM(1) TI_LGKM(2) TI_LGKM(3) TI_LGKM(4) TI_LGKM(5) TI_LGKM(6) TI_LGKM(7) TI_LGKM(8)
+    TI_LGKM(9) TI_LGKM(10) TI_LGKM(11) TI_LGKM(12) TI_LGKM(13) TI_LGKM(14) TI_LGKM(15)
+#undef TI_LGKM
     default: asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); break;
   }
 }
@@ -733,18 +729,22 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
       const int pa = __builtin_amdgcn_readlane(ids, min(2 * t, 63));
       const int pb = __builtin_amdgcn_readlane(ids, min(2 * t + 1, 63));
       const int key0 = (c0 + 2 * t) * 16;
+      // where the two blocks of the turn start, in elements from the pool's first: the same in
+      // every lane (scalar arithmetic); a lane adds the offset of its piece
+      const int prow_a = key0 % P, prow_b = (key0 + 16) % P;
+      const long k_a = (long)pa * (long)page_elems + (long)prow_a * HD, k_b = (long)pb * (long)page_elems + (long)prow_b * HD;
+      const long v_a = (long)pa * (long)page_elems + prow_a, v_b = (long)pb * (long)page_elems + prow_b;
 #pragma unroll
       for (int j = 0; j < MY_LOADS; ++j) {
-        const int blk = ld_desc[j] & 1, off = ld_desc[j] >> 1;
-        const int page = blk ? pb : pa;
-        const int prow = (key0 + 16 * blk) % P;                    // row of the block's first key in its page
+        const bool second = ld_desc[j] & 1;
+        const int off = ld_desc[j] >> 1;
         const bf16_t* src;
         unsigned dst;
         if (j < MY_K) {
-          src = kpool + (size_t)page * page_elems + (size_t)prow * HD + off;
+          src = kpool + (second ? k_b : k_a) + off;
           dst = (wave + NW * j) * 1024;
         } else {
-          src = vpool + (size_t)page * page_elems + off + prow;
+          src = vpool + (second ? v_b : v_a) + off;
           dst = K_BYTES + (wave + NW * (j - MY_K)) * 1024;
         }
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
