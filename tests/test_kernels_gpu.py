@@ -648,13 +648,20 @@ def test_attention_bf16_decode_rows(ops, nh, nkv, hd, P, window):
 @pytest.mark.parametrize("nh,nkv,hd,P,window", [
     (4, 2, 64, 16, None), (6, 2, 32, 16, None), (4, 2, 128, 16, None), (2, 1, 128, 32, None),
     (4, 4, 64, 16, 40), (2, 2, 32, 16, 7)])
-def test_attention_bf16_portions_and_mixed(ops, nh, nkv, hd, P, window):
+@pytest.mark.parametrize("groups", [1, 2])
+def test_attention_bf16_portions_and_mixed(ops, nh, nkv, hd, P, window, groups):
     """Portions of every size, starting anywhere (a page's edge, the middle of a
-    page, the start of a request), beside decode rows."""
+    page, the start of a request), beside decode rows; with one and with two groups of
+    wavefronts per workgroup (the launch would choose by its size)."""
     if not ops.use_fast_attention:
         pytest.skip("bfloat16 attention kernels are switched off")
     entries = [(2, 0), (7, 30), (1, 99), (16, 16), (17, 15), (64, 0), (65, 63), (130, 41), (1, 0), (3, 300), (200, 5)]
-    got, want = fast_attention_case(ops, entries, nh, nkv, hd, P, window, seed=nh * 10 + hd)
+    lib = ops.lib("attention_bf16")
+    lib.ti_attention_prefill_groups(groups)
+    try:
+        got, want = fast_attention_case(ops, entries, nh, nkv, hd, P, window, seed=nh * 10 + hd)
+    finally:
+        lib.ti_attention_prefill_groups(0)
     assert torch.isfinite(got).all()
     assert (got - want).abs().max() < 2e-2
 

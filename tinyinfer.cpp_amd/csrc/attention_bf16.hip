@@ -610,14 +610,20 @@ __device__ __forceinline__ void vm_wait_turns(int k) {
 #undef TI_VM
 }
 
-// CB: column blocks (of 32 tokens) per wavefront; the workgroup has 4 / CB wavefronts.
-template <int HD, int CB>
-__global__ void __launch_bounds__(256 / CB)
+// NG: groups of four wavefronts in the workgroup (1 or 2).  Every group takes all 128 rows, a
+// column block of 32 tokens per wavefront; with two groups the turns go to them alternately
+// (each group loads and walks its own turns through its own LDS stages) and their partial
+// results are merged through LDS at the end.  Two groups put two wavefronts on every SIMD
+// when a launch has only one workgroup per compute unit, so that one's loads, LDS reads and
+// vector work hide behind the other's matrix products.
+template <int HD, int NG>
+__global__ void __launch_bounds__(256 * NG)
 attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool,
                         const int* __restrict__ table, int table_stride, const int* __restrict__ tiles,
                         const int* __restrict__ entries, bf16_t* __restrict__ out, int n_head, int n_kv, int P,
                         float scale, int window) {
-  constexpr int NW = 4 / CB;                          // wavefronts
+  constexpr int CB = 1;                               // column blocks (of 32 tokens) per wavefront
+  constexpr int NW = 4;                               // wavefronts of a group
   constexpr int WROWS = 32 * CB;                      // tokens per wavefront
   constexpr int NP = HD / 8;                          // 16-byte pieces per K row
   constexpr int K_BYTES = PF_KEYS * HD * 2;
@@ -634,7 +640,7 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
   const int entry = tiles[2 * blockIdx.x], first = tiles[2 * blockIdx.x + 1];
   const int row0 = entries[4 * entry], n_tok = entries[4 * entry + 1], start = entries[4 * entry + 2];
   const int head = blockIdx.y;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int grp = (threadIdx.x >> 6) / NW, wave = (threadIdx.x >> 6) % NW, lane = threadIdx.x & 63;
   const int r32 = lane & 31, h = lane >> 5;
   const int row_end = row0 + n_tok;
   const int kv_last = start + n_tok - 1;
@@ -710,7 +716,7 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     }
   }
 
-  const unsigned lds0 = (unsigned)(size_t)smem;
+  const unsigned lds0 = (unsigned)(size_t)smem + grp * (PF_STAGES * STAGE);   // this group's stages
   // LDS addresses of this lane's fragments (without stage and k-step)
   const unsigned k_row = lds0 + r32 * (HD * 2);                     // K row r32
   const unsigned v_row = lds0 + K_BYTES + r32 * 64;                 // V^T row (dim) r32 of a 32-dim block
@@ -724,8 +730,12 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     // the page ids of this run's blocks, one per lane; blocks past the end repeat page 0
     int ids = (lane < nblk) ? tab[((c0 + lane) * 16) / P] : 0;
     if (ids < 0) ids = 0;                                           // given back: all its keys are masked
-    auto issue = [&](int t) {
-      const unsigned stage = lds0 + ((turn_count + t) % PF_STAGES) * STAGE;
+    // this group's turns are turns grp, grp + NG, ... of the run; i counts them
+    const int my_turns = (n_turns - grp + NG - 1) / NG;
+    const int n_iter = (n_turns + NG - 1) / NG;                      // the first group's count: the most
+    auto issue = [&](int i) {
+      const int t = i * NG + grp;
+      const unsigned stage = lds0 + ((turn_count + i) % PF_STAGES) * STAGE;
       const int pa = __builtin_amdgcn_readlane(ids, min(2 * t, 63));
       const int pb = __builtin_amdgcn_readlane(ids, min(2 * t + 1, 63));
       const int key0 = (c0 + 2 * t) * 16;
@@ -753,17 +763,19 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     };
     constexpr int AHEAD = PF_STAGES - 1;
 #pragma unroll
-    for (int t = 0; t < AHEAD; ++t)
-      if (t < n_turns) issue(t);
-    for (int t = 0; t < n_turns; ++t) {
-      // turn t has landed: only the turns issued after it (at most AHEAD - 1) may be outstanding
-      vm_wait_turns<MY_LOADS>(min(AHEAD - 1, n_turns - 1 - t));
+    for (int i = 0; i < AHEAD; ++i)
+      if (i < my_turns) issue(i);
+    for (int i = 0; i < n_iter; ++i) {
+      // this group's turn i has landed: only its turns issued after it (at most AHEAD - 1) may be
+      // outstanding.  Both groups pass the barrier together, also the one that has run out of turns.
+      vm_wait_turns<MY_LOADS>(max(0, min(AHEAD - 1, my_turns - 1 - i)));
       __builtin_amdgcn_s_barrier();
-      if (t + AHEAD < n_turns) issue(t + AHEAD);                   // into the stage that turn t - 1 has left
-      const int key0 = (c0 + 2 * t) * 16;
+      if (i + AHEAD < my_turns) issue(i + AHEAD);                  // into the stage that turn i - 1 has left
+      if (i >= my_turns) continue;
+      const int key0 = (c0 + 2 * (i * NG + grp)) * 16;
       // nothing of this turn is visible to this wavefront: it only helps loading
       if (w_rows == 0 || key0 > w_pos_last || key0 + PF_KEYS - 1 < w_lo) continue;
-      const unsigned st = ((turn_count + t) % PF_STAGES) * STAGE;
+      const unsigned st = ((turn_count + i) % PF_STAGES) * STAGE;
 
       // ---- the fragments of both tiles: keys now, values right behind them
       v4u kf[KS];
@@ -881,9 +893,35 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                                                                __builtin_bit_cast(bf16x8, pf[cb][tt]), o[cb][d],
                                                                0, 0, 0);
     }
-    turn_count += n_turns;
+    turn_count += n_iter;
     // every wavefront is done with this run's stages before the next run refills them
     __builtin_amdgcn_s_barrier();
+  }
+
+  if constexpr (NG == 2) {
+    // The second group hands its maxima, sums and outputs to the first through LDS (the stages are
+    // free now): lane for lane, the two hold the same columns and dims.
+    constexpr int NVAL = DB * 16 + 2;
+    float* xm = reinterpret_cast<float*>(smem) + (size_t)wave * NVAL * 64 + lane;
+    if (grp == 1) {
+#pragma unroll
+      for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) xm[(d * 16 + i) * 64] = o[0][d][i];
+      xm[(DB * 16) * 64] = mx[0];
+      xm[(DB * 16 + 1) * 64] = l[0];
+    }
+    __syncthreads();
+    if (grp == 1) return;
+    const float m1 = xm[(DB * 16) * 64], l1 = xm[(DB * 16 + 1) * 64];
+    const float m_new = fmaxf(mx[0], m1);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float a0 = __builtin_amdgcn_exp2f(mx[0] - m_safe), a1 = __builtin_amdgcn_exp2f(m1 - m_safe);
+    l[0] = l[0] * a0 + l1 * a1;
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[0][d][i] = o[0][d][i] * a0 + xm[(d * 16 + i) * 64] * a1;
   }
 
   // o[cb][d][i]: dim 32 d + 8 (i / 4) + 4 h + i % 4 of token (column) r32 of block cb
@@ -1007,6 +1045,8 @@ extern "C" int ti_attention_decode_prepared_bf16(const float* qkv, int row_width
                              n_head, n_kv, hd, page_size, scale, window, n_splits, prep, stream);
 }
 
+static int g_prefill_groups = 0;   // for measurements: 1 or 2 wavefront groups per workgroup, 0 = by the launch
+extern "C" void ti_attention_prefill_groups(int groups) { g_prefill_groups = groups; }
 static int g_prefill_lds = 1;
 // 1: head sizes 64 and 128 take the kernel that shares keys and values through LDS
 // (default); 0: every head size takes the kernel that reads them per wavefront
@@ -1024,28 +1064,34 @@ extern "C" int ti_attention_prefill_bf16(const void* q, const void* pool, const 
   if (n_tiles == 0) return 0;
   dim3 grid(n_tiles, n_head);
   if (g_prefill_lds && (hd == 64 || hd == 128)) {
-    const int lds = PF_STAGES * 2 * PF_KEYS * hd * 2;
+    // two groups of wavefronts per workgroup when the launch would else leave a SIMD with one wavefront
+    const int groups = g_prefill_groups ? g_prefill_groups : ((long)n_tiles * n_head < 512 ? 2 : 1);
+    const int lds = groups * PF_STAGES * 2 * PF_KEYS * hd * 2;
     static bool ready = false;          // allow more than 64 KiB of dynamic LDS, once
     if (!ready) {
+      const int most = 2 * PF_STAGES * 2 * PF_KEYS * 128 * 2;
       if (hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<128, 1>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              PF_STAGES * 2 * PF_KEYS * 128 * 2) != hipSuccess ||
+                              hipFuncAttributeMaxDynamicSharedMemorySize, most / 2) != hipSuccess ||
+          hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<128, 2>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess ||
           hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<64, 1>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              PF_STAGES * 2 * PF_KEYS * 64 * 2) != hipSuccess) {
-        ti_set_error("attention_prefill: cannot reserve %d bytes of LDS", lds);
+                              hipFuncAttributeMaxDynamicSharedMemorySize, most / 4) != hipSuccess ||
+          hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<64, 2>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, most / 2) != hipSuccess) {
+        ti_set_error("attention_prefill: cannot reserve %d bytes of LDS", most);
         return 2;
       }
       ready = true;
     }
-    if (hd == 128)
-      attn_prefill_lds_kernel<128, 1><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,
-                                                                  table_stride, tiles, entries, (bf16_t*)out,
-                                                                  n_head, n_kv, page_size, scale, window);
-    else
-      attn_prefill_lds_kernel<64, 1><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,
-                                                                 table_stride, tiles, entries, (bf16_t*)out,
-                                                                 n_head, n_kv, page_size, scale, window);
+#define TI_PLDS(H, G)                                                                                          \
+  attn_prefill_lds_kernel<H, G><<<grid, 256 * G, lds, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,   \
+                                                                table_stride, tiles, entries, (bf16_t*)out,     \
+                                                                n_head, n_kv, page_size, scale, window)
+    if (hd == 128 && groups == 2) TI_PLDS(128, 2);
+    else if (hd == 128) TI_PLDS(128, 1);
+    else if (groups == 2) TI_PLDS(64, 2);
+    else TI_PLDS(64, 1);
+#undef TI_PLDS
     TI_LAUNCH_CHECK();
     return 0;
   }
