@@ -23,6 +23,7 @@
 // (The reference scans positions with 16-lane groups and FMA for both cases:
 // /root/reference/src/cuda/attention.cu:107-198.)
 #include "common.h"
+#include "tinyinfer_kernels.h"
 #include "qk_prep.h"
 
 TI_ERROR_API

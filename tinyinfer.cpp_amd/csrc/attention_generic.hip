@@ -9,6 +9,7 @@
 // results are merged in LDS with the usual rescaling.  Scores, softmax statistics
 // and the output accumulate in 32-bit.
 #include "common.h"
+#include "tinyinfer_kernels.h"
 
 TI_ERROR_API
 

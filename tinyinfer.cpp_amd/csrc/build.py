@@ -27,7 +27,7 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-shared",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]
-HEADERS = ["common.h", "qk_prep.h"]
+HEADERS = ["common.h", "qk_prep.h", "tinyinfer_kernels.h"]
 # flags of single libraries.  The attention kernels rescale their MFMA accumulators with
 # vector instructions; kept in the accumulation registers they would be copied out and back
 # on every turn of the loop, so their MFMAs are told to work on ordinary vector registers.

@@ -3,6 +3,7 @@
 // rotation + paged cache write.  All arithmetic is 32-bit; T is the storage
 // type of activations, weights and cache (float or bfloat16).
 #include "common.h"
+#include "tinyinfer_kernels.h"
 #include "qk_prep.h"
 
 TI_ERROR_API

@@ -17,6 +17,7 @@
 // /root/reference/src/cuda/gemm.cu:37-85 and 152-261; it reads the weights once
 // per row of A for M <= 32.)
 #include "common.h"
+#include "tinyinfer_kernels.h"
 #include "qk_prep.h"
 
 TI_ERROR_API

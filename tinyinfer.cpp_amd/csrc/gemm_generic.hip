@@ -6,6 +6,7 @@
 // Every output element sums its K products in ascending k, whatever M is, so a
 // token's result does not depend on what else is in the batch.
 #include "common.h"
+#include "tinyinfer_kernels.h"
 
 TI_ERROR_API
 

@@ -11,6 +11,7 @@
 // bisection over the order-preserving integer image of the floats; every sum is
 // reduced in a fixed order, so the result is reproducible.
 #include "common.h"
+#include "tinyinfer_kernels.h"
 
 TI_ERROR_API
 

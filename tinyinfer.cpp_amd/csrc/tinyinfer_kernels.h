@@ -1,0 +1,100 @@
+// The C interface of the kernel libraries: what `ops/kernels.py` binds through ctypes, and what a
+// C or C++ program may link against.  One shared library per source file (libti_<name>.<hash>.so,
+// built by build.py); each also exports `const char* ti_last_error()`.
+//
+// Conventions.  Every pointer is device memory of the GPU that `stream` belongs to.  Every function
+// returns 0 on success, 3 for sizes its kernels do not serve (nothing was launched; use the more
+// general function) and another non-zero value for an error; `ti_last_error()` of the same library
+// then holds the message.  Nothing here allocates: scratch comes in through arguments.
+// dtype codes: 0 = float32, 1 = bfloat16.  Epilogue codes `epi`: 0 store f32, 1 add into f32,
+// 2 store in the operand dtype, 3 SwiGLU over stacked [gate; up] rows.
+//
+// Shapes: M tokens (rows) of a step; H residual width; a cache pool of one layer is
+// [pages][2][n_kv][P][hd] with keys as [row][hd] and values transposed as [hd][row]; `table` is
+// int32 [requests][table_stride] of page ids (-1: none), `slot[m]` the table row of token m, `pos[m]`
+// its position.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+// ---- libti_core: embedding, norms, rotation, cache write (templated on the storage dtype)
+int ti_embed(int dtype, const void* table, const int* tok, float* x, int M, int H, int V, hipStream_t stream);
+// out[r] = rmsnorm(x[rows ? rows[r] : r]) * w, in `out_dtype`
+int ti_rmsnorm(int out_dtype, const float* x, const float* w, const int* rows, void* out, int n_rows, int H, float eps,
+               hipStream_t stream);
+// half-split rotation in place on f32 [M, heads, hd] (rows `row_stride` floats apart)
+int ti_rope_neox(float* x, const int* pos, const float* inv_freq, int M, int heads, int hd, long row_stride,
+                 hipStream_t stream);
+// table[p][k] = (cos, sin)(p * inv_freq[k]) for p < n_pos
+int ti_rope_table(float* table, const float* inv_freq, int half, int n_pos, hipStream_t stream);
+// qkv f32 [M, (n_head + 2 n_kv) hd]: per-head norm (weights may be null), rotation (inv_freq may be
+// null; rope_table [table_len][hd/2][2] may be null), q to q_out, k and v into the cache pages
+int ti_qk_norm_rope_kv_write(int dtype, const float* qkv, const float* q_w, const float* k_w, const float* inv_freq,
+                             const float* rope_table, int table_len, const int* pos, const int* slot, const int* table,
+                             int table_stride, void* pool, void* q_out, int M, int n_head, int n_kv, int hd,
+                             int page_size, float eps, hipStream_t stream);
+// the per-head norm alone, in place
+int ti_qk_norm_inplace(float* qkv, int row_width, const float* q_w, const float* k_w, int M, int n_head, int n_kv, int hd,
+                       float eps, hipStream_t stream);
+
+// ---- libti_gemm_generic: out (op)= A W^T for any sizes, float32 or bfloat16, fixed summation order
+int ti_gemm_generic(int dtype, const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
+                    hipStream_t stream);
+
+// ---- libti_gemm_bf16: the same on the matrix cores (K a multiple of 8)
+int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi, hipStream_t stream);
+// out (op)= rmsnorm(x; nw, eps) W^T for M <= 16, K a multiple of 64
+int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, const void* W, void* out, int M, int N, int K, int epi,
+                        hipStream_t stream);
+// the q/k/v product of a step (M > 64) that finishes its heads itself: see ti_qk_norm_rope_kv_write
+int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K, long lda, const float* q_w, const float* k_w,
+                          float eps, const float* inv_freq, const float* rope_table, int table_len, const int* pos,
+                          const int* slot, const int* table, int table_stride, void* pool, void* q_out, int n_head,
+                          int n_kv, int hd, int page_size, hipStream_t stream);
+// switches for measurements and tests (0 restores the choice by shape)
+void ti_gemm_bf16_force_tile(int which);      // 1: 256 x 128, 3: 128 x 64, 6: 64 x 64
+void ti_gemm_bf16_skinny_waves(int waves);    // 4 or 8 wavefronts in the kernel for M <= 64
+void ti_gemm_bf16_use_pipelined(int on);      // 0: the plain tiled kernel for every K
+
+// ---- libti_attention_generic: paged causal attention of every row, any head size in steps of 16
+int ti_attention_rows(int dtype, const void* q, const void* pool, const int* table, int table_stride, const int* pos,
+                      const int* slot, void* out, int M, int n_head, int n_kv, int hd, int page_size, float scale,
+                      int window, hipStream_t stream);
+
+// ---- libti_attention_bf16: the same on the matrix cores (head sizes 32, 64, 128; pages of 16 n rows)
+// rows of single tokens; n_splits > 1 needs part_o f32 [n_rows, n_head, n_splits, hd] and part_ml f32
+// [n_rows, n_head, n_splits, 2]
+int ti_attention_decode_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* pos,
+                             const int* slot, const int* rows, void* out, float* part_o, float* part_ml, int n_rows,
+                             int n_head, int n_kv, int hd, int page_size, float scale, int window, int n_splits,
+                             hipStream_t stream);
+// the same from the 32-bit projections: norm, rotation and the cache write of the row's own key and
+// value happen inside (head sizes 64 and 128, at most 16 q heads per kv head)
+int ti_attention_decode_prepared_bf16(const float* qkv, int row_width, const float* q_w, const float* k_w, float eps,
+                                      const float* inv_freq, const float* rope_table, int table_len, void* pool,
+                                      int write_kv, const int* table, int table_stride, const int* pos,
+                                      const int* slot, void* out, float* part_o, float* part_ml, int n_rows,
+                                      int n_head, int n_kv, int hd, int page_size, float scale, int window,
+                                      int n_splits, hipStream_t stream);
+// portions of prompts: tiles int32 [n_tiles][2] = (entry, first row) of 128 rows each, entries int32
+// [n_entries][4] = (row0, n_tokens, start_pos, -)
+int ti_attention_prefill_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* tiles,
+                              const int* entries, void* out, int n_tiles, int n_head, int n_kv, int hd, int page_size,
+                              float scale, int window, hipStream_t stream);
+void ti_attention_prefill_groups(int groups);  // 1 or 2 groups of wavefronts per workgroup, 0: by the launch
+void ti_attention_prefill_use_lds(int on);     // 0: the kernel without LDS for every head size
+
+// ---- libti_sampling
+// out[r] = lowest index of the largest logit; scratch: 2 * 64 * n_rows four-byte words (two stages:
+// 64 workgroups per row, then one) or null (one workgroup reads a whole row)
+int ti_argmax(const float* logits, int* out, void* scratch, int n_rows, int V, hipStream_t stream);
+// temperature, top-k (0: all), top-p and one uniform number per row
+int ti_sample(const float* logits, const float* temp, const int* top_k, const float* top_p, const float* uni, int* out,
+              int n_rows, int V, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
