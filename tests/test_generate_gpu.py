@@ -157,3 +157,13 @@ def test_smoke_entry():
     sys.path.insert(0, ROOT)
     import __graft_entry__
     __graft_entry__.smoke()
+
+
+def test_operator_selftest_of_the_command_line():
+    """TINY_SELFTEST=1 runs every kernel against a CPU computation; the exit code counts failures."""
+    env = dict(os.environ, TINY_SELFTEST="1")
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "tinyinfer")], capture_output=True, text=True,
+                         timeout=300, env=env)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "[selftest] all cases passed" in run.stdout
+    assert run.stdout.count(" ok") >= 20 and "FAIL" not in run.stdout

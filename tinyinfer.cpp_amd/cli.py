@@ -48,6 +48,11 @@ def _as_ids(text: str) -> Optional[List[int]]:
 def main(argv: Optional[List[str]] = None) -> int:
     argv = list(sys.argv if argv is None else argv)
     prog, args = argv[0], argv[1:]
+    if os.environ.get("TINY_SELFTEST") == "1":
+        # every kernel against a CPU computation; the exit code counts the failures
+        # (the reference's QWEN_SELFTEST=1: /root/reference/src/main.cpp:123-125)
+        from .selftest import run_selftest
+        return run_selftest()
     model = None
     prompts: List[str] = []
     n_predict, temp, top_k, top_p, seed, max_seq = 128, 0.0, 0, 1.0, 42, 2048
