@@ -17,6 +17,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..cache import CacheManager, CacheStorage, OutOfPages, PagedGroup
@@ -257,60 +258,63 @@ class Engine:
         ctx.M = M
         R = len(entries)
         W = self.table_width
-        tiles: List[int] = []             # (entry, first row) pairs, flat
-        dec_rows: List[int] = []
-        tokens: List[int] = []
-        positions: List[int] = []
-        slots: List[int] = []
-        out_rows: List[int] = []
-        ent_flat: List[int] = []
-        row0 = 0
-        for i, e in enumerate(entries):
-            n = len(e.tokens)
-            start = cache.length(e.request)
-            rec = (row0, n, start, cache.slot(e.request))
-            ctx.entries.append(rec)
-            ent_flat.extend(rec)
-            tokens.extend(e.tokens)
-            if n > 1:
-                positions.extend(range(start, start + n))
-                slots.extend([i] * n)
-                for q0 in range(0, n, PREFILL_TILE_Q):
-                    tiles.append(i)
-                    tiles.append(row0 + q0)
-            else:
-                positions.append(start)
-                slots.append(i)
-                dec_rows.append(row0)
-            for w in e.want:
-                out_rows.append(row0 + int(w))
-            if start + n > ctx.max_context:
-                ctx.max_context = start + n
-            row0 += n
-        n_tiles = len(tiles) // 2
-        ctx.decode_only = n_tiles == 0
-        if ctx.decode_only:
-            dec_rows = []
-        ctx.n_tiles = n_tiles
-        ctx.n_decode_rows = len(dec_rows)
-        ctx.split_context = ctx.max_context
-
         # layout: tokens | positions | slots | out_rows | entries [R,4] | tiles [n_tiles,2] | decode rows | tables
+        n_tiles = sum(-(-len(e.tokens) // PREFILL_TILE_Q) for e in entries if len(e.tokens) > 1)
+        ctx.decode_only = n_tiles == 0
+        n_dec = 0 if ctx.decode_only else sum(1 for e in entries if len(e.tokens) == 1)
+        ctx.n_tiles, ctx.n_decode_rows = n_tiles, n_dec
         o_tok, o_pos, o_slot = 0, M, 2 * M
         o_out = 3 * M
         o_ent = o_out + n_want
         o_tile = o_ent + 4 * R
         o_dec = o_tile + 2 * n_tiles
-        o_tab = o_dec + len(dec_rows)
+        o_tab = o_dec + n_dec
         total = o_tab + len(paged) * R * W
         turn, host, dev = self._meta_buffers(total, meta_dev)
         h = host.numpy()
-        h[o_tok:o_pos] = tokens
-        h[o_pos:o_slot] = positions
-        h[o_slot:o_out] = slots
-        h[o_out:o_tile] = out_rows + ent_flat
-        if tiles or dec_rows:
+        out_rows: List[int] = []
+        ent_flat: List[int] = []
+        if ctx.decode_only:
+            # single tokens only: three short lists, one assignment each
+            starts = [cache.length(e.request) for e in entries]
+            h[o_tok:o_pos] = [e.tokens[0] for e in entries]
+            h[o_pos:o_slot] = starts
+            h[o_slot:o_out] = range(R)
+            for i, (e, start) in enumerate(zip(entries, starts)):
+                rec = (i, 1, start, cache.slot(e.request))
+                ctx.entries.append(rec)
+                ent_flat.extend(rec)
+                for _ in e.want:
+                    out_rows.append(i)
+            ctx.max_context = max(starts) + 1
+        else:
+            tiles: List[int] = []         # (entry, first row) pairs, flat
+            dec_rows: List[int] = []
+            row0 = 0
+            for i, e in enumerate(entries):
+                n = len(e.tokens)
+                start = cache.length(e.request)
+                rec = (row0, n, start, cache.slot(e.request))
+                ctx.entries.append(rec)
+                ent_flat.extend(rec)
+                h[o_tok + row0:o_tok + row0 + n] = e.tokens
+                h[o_slot + row0:o_slot + row0 + n] = i
+                if n > 1:
+                    h[o_pos + row0:o_pos + row0 + n] = np.arange(start, start + n, dtype=np.int32)
+                    for q0 in range(0, n, PREFILL_TILE_Q):
+                        tiles.append(i)
+                        tiles.append(row0 + q0)
+                else:
+                    h[o_pos + row0] = start
+                    dec_rows.append(row0)
+                for w in e.want:
+                    out_rows.append(row0 + int(w))
+                if start + n > ctx.max_context:
+                    ctx.max_context = start + n
+                row0 += n
             h[o_tile:o_tab] = tiles + dec_rows
+        ctx.split_context = ctx.max_context
+        h[o_out:o_tile] = out_rows + ent_flat
         for k, (gi, g) in enumerate(paged):
             base = o_tab + k * R * W
             rows = g.rows
@@ -327,7 +331,7 @@ class Engine:
         ctx.out_rows = dev[o_out:o_out + n_want] if n_want else None
         ctx.entry_meta = dev[o_ent:o_ent + 4 * R].view(R, 4)
         ctx.tiles = dev[o_tile:o_tile + 2 * n_tiles].view(-1, 2) if n_tiles else None
-        ctx.decode_rows = dev[o_dec:o_dec + len(dec_rows)] if dec_rows else None
+        ctx.decode_rows = dev[o_dec:o_dec + n_dec] if n_dec else None
         for k, (gi, g) in enumerate(paged):
             base = o_tab + k * R * W
             ctx._views[gi] = CacheView(dev[base:base + R * W].view(R, W), self.page_size)
