@@ -459,6 +459,41 @@ def test_linear_bf16_matrix_cores(ops, M, N, K):
         assert (f64(out) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
 
 
+@pytest.mark.parametrize("tile", [1, 3, 6])
+@pytest.mark.parametrize("M,N,K", [(300, 520, 128), (257, 384, 192), (130, 200, 64), (700, 96, 320)])
+def test_linear_bf16_every_tile(ops, tile, M, N, K):
+    """Each tile of the pipelined kernel (256 x 128 with eight wavefronts, 128 x 64, 64 x 64), whatever
+    the dispatch would have chosen for the shape, with every epilogue, against float64."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    lib = ops.lib("gemm_bf16")
+    g = torch.Generator().manual_seed(M + N + tile)
+    a = (torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16)
+    w = (torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16)
+    ref = ref_linear(a, w)
+    tol = 2e-5 * K
+    lib.ti_gemm_bf16_force_tile(tile)
+    try:
+        out = torch.empty(M, N, device="cuda")
+        ops.linear(dev(a), dev(w), out, "store")
+        assert (f64(out) - ref).abs().max() < tol
+        base = torch.randn(M, N, generator=g)
+        out = dev(base.clone())
+        ops.linear(dev(a), dev(w), out, "add")
+        assert (f64(out) - (ref + f64(base))).abs().max() < tol
+        out = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+        ops.linear(dev(a), dev(w), out, "store_act")
+        assert (f64(out) - ref).abs().max() < 0.005 * ref.abs().max() + tol
+        F = N // 2
+        out = torch.empty(M, F, device="cuda", dtype=torch.bfloat16)
+        ops.linear(dev(a), dev(w), out, "swiglu")
+        gte, up = ref[:, :F], ref[:, F:]
+        want = gte / (1 + torch.exp(-gte)) * up
+        assert (f64(out) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
+    finally:
+        lib.ti_gemm_bf16_force_tile(0)
+
+
 def test_linear_bf16_rows_do_not_depend_on_the_batch(ops):
     """Within one kernel a row's bits do not depend on the other rows."""
     if not ops.use_fast_gemm:
