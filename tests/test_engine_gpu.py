@@ -100,7 +100,7 @@ def make_trace(mode, requests):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,sharp,page_size", [("A", False, 16), ("B", False, 4), ("B", True, 16), ("C", True, 16), ("D", True, 16)])
+@pytest.mark.parametrize("name,sharp,page_size", [("A", False, 16), ("B", False, 4), ("B", True, 16), ("C", True, 16), ("D", True, 16), ("D", True, 32)])
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_engine_matches_plain(model_folders, name, sharp, page_size, dtype, mode):
     folder = model_folders(name, "bfloat16", sharp)
