@@ -33,6 +33,14 @@ CONFIGS = {
               vocab_size=333, rope_theta=200000.0, rms_norm_eps=2e-6, tie_word_embeddings=True,
               attention_bias=False, hidden_act="silu", max_position_embeddings=4096,
               layer_types=["full_attention", "sliding_attention", "sliding_attention"], sliding_window=37),
+    # not tiny in its widths: the layer sizes of Qwen3-0.6B (width 1024, 16 heads in 8 groups, head 128,
+    # feed-forward 3072), 2 layers, a small vocabulary.  The kernels chosen for these widths (the tiles
+    # of the products, the projection that finishes its heads, two-group prefill attention, the norm
+    # inside a product, decode attention that prepares its query) differ from the tiny models' ones.
+    "E": dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2, hidden_size=1024,
+              num_attention_heads=16, num_key_value_heads=8, head_dim=128, intermediate_size=3072,
+              vocab_size=1500, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+              attention_bias=False, hidden_act="silu", max_position_embeddings=4096),
 }
 
 
