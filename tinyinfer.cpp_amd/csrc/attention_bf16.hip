@@ -32,6 +32,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short short4v;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
+#define TI_LOG2E 1.4426950408889634f
+
 union Frag8 {
   uint4 u;
   bf16x8 v;
@@ -69,24 +71,26 @@ __device__ __forceinline__ void load_pair(const PagedKV& kv, int pageA, int keyA
                                           KVPair<HD>& f) {
   const int lane = threadIdx.x & 63;
   const int r16 = lane & 15, quad = lane >> 4;
+  // where a block's keys and values start is the same in every lane (scalar registers); a lane
+  // adds one offset of its own, and the steps are constants in the load instructions
   const size_t page_elems = (size_t)2 * kv.n_kv * kv.P * HD;
-  const size_t k_off = (size_t)kv.kvh * kv.P * HD, v_off = (size_t)(kv.n_kv + kv.kvh) * kv.P * HD;
-  const bf16_t* pa = kv.pool + (size_t)pageA * page_elems;
-  const bf16_t* pb = kv.pool + (size_t)pageB * page_elems;
   const int rowA = keyA % kv.P, rowB = keyB % kv.P;
-  const bf16_t* ka = pa + k_off + (size_t)(rowA + r16) * HD + quad * 8;
-  const bf16_t* kb = pb + k_off + (size_t)(rowB + r16) * HD + quad * 8;
-  const bf16_t* va = pa + v_off + (size_t)r16 * kv.P + rowA + quad * 4;
-  const bf16_t* vb = pb + v_off + (size_t)r16 * kv.P + rowB + quad * 4;
+  const bf16_t* ka = kv.pool + (size_t)pageA * page_elems + (size_t)kv.kvh * kv.P * HD + (size_t)rowA * HD;
+  const bf16_t* kb = kv.pool + (size_t)pageB * page_elems + (size_t)kv.kvh * kv.P * HD + (size_t)rowB * HD;
+  const bf16_t* va = kv.pool + (size_t)pageA * page_elems + (size_t)(kv.n_kv + kv.kvh) * kv.P * HD + rowA;
+  const bf16_t* vb = kv.pool + (size_t)pageB * page_elems + (size_t)(kv.n_kv + kv.kvh) * kv.P * HD + rowB;
+  const unsigned k_lane = (unsigned)(r16 * HD + quad * 8);          // elements
+  const unsigned v_lane = (unsigned)(r16 * kv.P + quad * 4);
 #pragma unroll
   for (int s = 0; s < HD / 32; ++s) {
-    f.k[0][s].u = *reinterpret_cast<const uint4*>(ka + s * 32);
-    f.k[1][s].u = *reinterpret_cast<const uint4*>(kb + s * 32);
+    f.k[0][s].u = *reinterpret_cast<const uint4*>(ka + k_lane + s * 32);
+    f.k[1][s].u = *reinterpret_cast<const uint4*>(kb + k_lane + s * 32);
   }
+  const unsigned v_step = 16u * kv.P;                                // elements between blocks of 16 dims
 #pragma unroll
   for (int d = 0; d < HD / 16; ++d) {
-    const uint2 a = *reinterpret_cast<const uint2*>(va + (size_t)d * 16 * kv.P);
-    const uint2 b = *reinterpret_cast<const uint2*>(vb + (size_t)d * 16 * kv.P);
+    const uint2 a = *reinterpret_cast<const uint2*>(va + v_lane + d * v_step);
+    const uint2 b = *reinterpret_cast<const uint2*>(vb + v_lane + d * v_step);
     f.v[d].u = make_uint4(a.x, a.y, b.x, b.y);
   }
 }
@@ -101,6 +105,8 @@ struct BlockInfo {
 
 // One pair of blocks for this wavefront's 16 columns.
 //   qf       Q^T fragments: column lane % 16, dims 32 * step + 8 * (lane / 16) .. + 7
+//   scale    softmax scale times log2(e): scores, maxima and partial maxima are in units of log 2,
+//            so that the weights are bare exp2
 //   lo, hi   the keys this lane's column may see: lo <= key <= hi
 //   kv_last  last position of the request that has been written (rows after it hold rubbish)
 template <int HD>
@@ -152,17 +158,17 @@ __device__ __forceinline__ void attend_pair(KVPair<HD>& f, const Frag8* qf, Bloc
   const float m_new = fmaxf(m, bm);
   const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
   Frag8 pf;
-  bf16_t* ph = reinterpret_cast<bf16_t*>(&pf.u);
-  float ps = 0.f;
+  float pv[8], ps = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const float p = __expf(sv[i] - m_safe);
-    ps += p;
-    ph[i] = f2bf(p);
+    pv[i] = __builtin_amdgcn_exp2f(sv[i] - m_safe);      // scores are in units of log 2
+    ps += pv[i];
   }
+  pf.u = make_uint4(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]), pack_bf16x2(pv[4], pv[5]),
+                    pack_bf16x2(pv[6], pv[7]));
   // the running maximum settles after a few blocks; then nothing needs rescaling
   if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
-    const float alpha = __expf(m - m_safe);
+    const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
     l *= alpha;
 #pragma unroll
     for (int d = 0; d < HD / 16; ++d)
@@ -393,7 +399,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
   {
     const int mine = (b1 - (b0 + wave) + 3) / 4;   // blocks b0 + wave, + 4, ... below b1
     const int last = own_key ? p_q - 1 : p_q;      // what the cache holds for this workgroup
-    walk_blocks<HD>(kv, qf, b0 + wave, 4, mine, lo, last, last, scale,
+    walk_blocks<HD>(kv, qf, b0 + wave, 4, mine, lo, last, last, scale * TI_LOG2E,
                     [=](int b) { return b == blk_lo || b == blk_hi; }, mx, l, o);
   }
   if (PREP && own_key && wave == 0) {
@@ -407,7 +413,8 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
 #pragma unroll
     for (int d = 0; d < HD / 16; ++d)
       f.v[d].u = make_uint4(quad == 0 ? (unsigned)s_kv[HD + d * 16 + r16] : 0u, 0, 0, 0);
-    attend_pair<HD>(f, qf, BlockInfo{p_q, true, true}, BlockInfo{p_q, false, false}, p_q, p_q, p_q, scale, mx, l, o);
+    attend_pair<HD>(f, qf, BlockInfo{p_q, true, true}, BlockInfo{p_q, false, false}, p_q, p_q, p_q, scale * TI_LOG2E,
+                    mx, l, o);
   }
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -428,7 +435,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
   float wgt[4], lt = 0.f;
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
-    wgt[w] = (s_m[w][r16] == -INFINITY) ? 0.f : __expf(s_m[w][r16] - mm);
+    wgt[w] = (s_m[w][r16] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s_m[w][r16] - mm);
     lt += s_l[w][r16] * wgt[w];
   }
   if (r16 >= n_cols) return;
@@ -480,7 +487,7 @@ attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ pa
     const float ms = (d < n_splits) ? pm[2 * d] : -INFINITY;
     const float ls = (d < n_splits) ? pm[2 * d + 1] : 0.f;
     const float mm = group_max<64>(ms);
-    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - mm);
+    const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - mm);
     const float lt = group_sum<64>(ls * w);
     s_w[d] = w;
     if (d == 0) s_inv = 1.0f / lt;
@@ -542,7 +549,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ poo
   // a block is free of checks if every column sees all of it: it ends at or before the
   // tile's first position and (with a window) starts inside the last column's window
   const int hi_col = col_ok ? my_pos : -1;          // columns beyond the portion see nothing
-  walk_blocks<HD>(kv, qf, blk_lo, 1, blk_hi - blk_lo + 1, my_lo, hi_col, kv_last, scale,
+  walk_blocks<HD>(kv, qf, blk_lo, 1, blk_hi - blk_lo + 1, my_lo, hi_col, kv_last, scale * TI_LOG2E,
                   [=](int b) {
                     const int key0 = b * 16;
                     const bool inside = (key0 + 15 <= pos_first) && (w_rows == 16) &&

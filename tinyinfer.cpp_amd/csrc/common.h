@@ -23,14 +23,6 @@ typedef uint16_t bf16_t;   // bfloat16 bits; arithmetic always happens in float
 
 __device__ __forceinline__ float bf2f(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
-// round to nearest, ties to even; NaN stays NaN
-__device__ __forceinline__ bf16_t f2bf(float f) {
-  const uint32_t u = __float_as_uint(f);
-  const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-  const uint32_t quiet = (u >> 16) | 0x40u;
-  return (bf16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? quiet : rounded);   // a select, not a branch
-}
-
 // two floats -> two bfloat16 in one word (first in the low half), round to nearest even:
 // gfx950 has an instruction for it (v_cvt_pk_bf16_f32)
 typedef float ti_float2v __attribute__((ext_vector_type(2)));
@@ -39,6 +31,8 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   const ti_float2v v = {a, b};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, ti_bf16x2));
 }
+// one float -> bfloat16, round to nearest even, NaN stays NaN (the same instruction)
+__device__ __forceinline__ bf16_t f2bf(float f) { return (bf16_t)(pack_bf16x2(f, 0.f) & 0xffffu); }
 
 template <typename T> __device__ __forceinline__ float ld(const T* p);
 template <> __device__ __forceinline__ float ld<float>(const float* p) { return *p; }
