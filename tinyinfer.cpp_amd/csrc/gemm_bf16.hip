@@ -39,7 +39,10 @@ __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f +
 // ============================================================== skinny kernel
 // grid.x = ceil(N / 16) (SwiGLU: ceil(F / 8): 8 gate rows and their 8 up rows).
 // NW wavefronts split K between them.
-template <int MT, int EPI, int NW = 4>
+// UN: 64-element chunks of K a wavefront has in flight at a time.  All loads of a pass are
+// issued before the first product: out-of-range pieces read a valid address (piece 0 of the
+// row) and get a zeroed weight instead of a branch, so that nothing waits in between.
+template <int MT, int EPI, int NW = 4, int UN = 4>
 __global__ void __launch_bounds__(NW * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_,
                    int M, int N, int K, long lda) {
@@ -47,7 +50,6 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, v
   __shared__ float red[NW][MT][16][17];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, j = lane >> 4;   // MFMA row / column, and k group
-  const int rows_total = SW ? 2 * N : N;
   // the weight row this lane feeds
   int wrow;
   if (SW) {
@@ -57,15 +59,22 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, v
     const int n = blockIdx.x * 16 + r;
     wrow = n < N ? n : N - 1;
   }
-  (void)rows_total;
-  const bf16_t* wp = W + (size_t)wrow * K + j * 16;
+  const bf16_t* wp = W + (size_t)wrow * K;
   const bf16_t* ap[MT];
-  bool aok[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + r;
-    aok[t] = m < M;
-    ap[t] = A + (size_t)(aok[t] ? m : 0) * lda + j * 16;
+    ap[t] = A + (size_t)(m < M ? m : 0) * lda;   // columns beyond M are computed from row 0 and never stored
+  }
+  // the residual this thread will add to, asked for before the product
+  const int tok = threadIdx.x >> 4, row = threadIdx.x & 15;
+  float prev[MT];
+  if (EPI == TI_EPI_ADD_F32 && threadIdx.x < 256) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = t * 16 + tok, n = blockIdx.x * 16 + row;
+      prev[t] = (m < M && n < N) ? ((const float*)out_)[(size_t)m * N + n] : 0.f;
+    }
   }
   floatx4 acc[MT];
 #pragma unroll
@@ -74,27 +83,35 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, v
   const uint4 zero = make_uint4(0, 0, 0, 0);
   // chunk c covers k in [64 c, 64 c + 64); lane group j takes [64 c + 16 j, +16)
   const int chunks = (K + 63) / 64;
-  constexpr int UN = 4;
   for (int c0 = wave; c0 < chunks; c0 += NW * UN) {
-    Frag w0[UN], w1[UN];
+    Frag w0[UN], w1[UN], a0[UN][MT], a1[UN][MT];
+    bool ok0[UN], ok1[UN];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int k = (c0 + NW * u) * 64 + j * 16;
-      const bool mine = c0 + NW * u < chunks;
-      w0[u].u = (mine && k + 8 <= K) ? ld16(wp + (size_t)(c0 + NW * u) * 64) : zero;
-      w1[u].u = (mine && k + 16 <= K) ? ld16(wp + (size_t)(c0 + NW * u) * 64 + 8) : zero;
+      ok0[u] = k + 8 <= K;    // false too for chunks beyond the last
+      ok1[u] = k + 16 <= K;
+      w0[u].u = ld16(wp + (ok0[u] ? k : 0));
+      w1[u].u = ld16(wp + (ok1[u] ? k + 8 : 0));
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int k = (c0 + NW * u) * 64 + j * 16;
-      const bool mine = c0 + NW * u < chunks;
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        Frag a0, a1;
-        a0.u = (mine && aok[t] && k + 8 <= K) ? ld16(ap[t] + (size_t)(c0 + NW * u) * 64) : zero;
-        a1.u = (mine && aok[t] && k + 16 <= K) ? ld16(ap[t] + (size_t)(c0 + NW * u) * 64 + 8) : zero;
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u].v, a0.v, acc[t], 0, 0, 0);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, a1.v, acc[t], 0, 0, 0);
+        a0[u][t].u = ld16(ap[t] + (ok0[u] ? k : 0));
+        a1[u][t].u = ld16(ap[t] + (ok1[u] ? k + 8 : 0));
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);   // every load above is issued before the first product waits
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      if (!ok0[u]) w0[u].u = zero;
+      if (!ok1[u]) w1[u].u = zero;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u].v, a0[u][t].v, acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, a1[u][t].v, acc[t], 0, 0, 0);
       }
     }
   }
@@ -106,7 +123,6 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, v
   __syncthreads();
   // thread -> (token = tid / 16, row = tid % 16): consecutive threads, consecutive columns
   if (NW > 4 && threadIdx.x >= 256) return;
-  const int tok = threadIdx.x >> 4, row = threadIdx.x & 15;
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + tok;
@@ -130,7 +146,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, v
       for (int w = 0; w < NW; ++w) s += red[w][t][tok][row];
       const size_t o = (size_t)m * N + n;
       if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = s;
-      if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] += s;
+      if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] = prev[t] + s;
       if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(s);
     }
   }
@@ -168,45 +184,56 @@ gemm_skinny_normed_kernel(const float* __restrict__ X, const float* __restrict__
   const int chunks = K / 64;
   constexpr int UN = 4;
 
-  // the first weights of this wavefront: on their way while the norm is computed
+  // the first weights of this wavefront: on their way while the norm is computed.  A chunk
+  // beyond the last reads chunk 0 and is zeroed afterwards: no branch between the loads.
   Frag w0[UN], w1[UN];
 #pragma unroll
   for (int u = 0; u < UN; ++u) {
-    const bool mine = wave + NW * u < chunks;
-    w0[u].u = mine ? ld16(wp + (size_t)(wave + NW * u) * 64) : zero;
-    w1[u].u = mine ? ld16(wp + (size_t)(wave + NW * u) * 64 + 8) : zero;
+    const int c = wave + NW * u < chunks ? wave + NW * u : 0;
+    w0[u].u = ld16(wp + (size_t)c * 64);
+    w1[u].u = ld16(wp + (size_t)c * 64 + 8);
   }
 
-  // ---- the norm: wavefront w takes rows w, w + NW, ...; a lane holds KC float4 of a row
+  // ---- the norm: wavefront w takes rows w, w + NW, ...; a lane holds KC float4 of a row.
+  // Two rows' loads are issued together where the registers allow; a lane's pieces beyond
+  // K read piece 0 and are left out of the sum and the store.
   float4 g[KC];
 #pragma unroll
   for (int c = 0; c < KC; ++c) {
     const int k = lane * 4 + 256 * c;
-    g[c] = k < K ? *reinterpret_cast<const float4*>(Gw + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+    g[c] = *reinterpret_cast<const float4*>(Gw + (k < K ? k : 0));
   }
+  constexpr int RB = KC <= 8 ? 2 : 1;
+  for (int r0 = wave; r0 < M; r0 += NW * RB) {
+    float4 v[RB][KC];
 #pragma unroll
-  for (int rr = 0; rr < 16 / NW; ++rr) {
-    const int m = wave + NW * rr;
-    if (m >= M) break;
-    const float* xr = X + (size_t)m * K;
-    float4 v[KC];
-    float ss = 0.f;
+    for (int b = 0; b < RB; ++b) {
+      const int m = r0 + NW * b < M ? r0 + NW * b : r0;
+      const float* xr = X + (size_t)m * K;
 #pragma unroll
-    for (int c = 0; c < KC; ++c) {
-      const int k = lane * 4 + 256 * c;
-      v[c] = k < K ? *reinterpret_cast<const float4*>(xr + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int c = 0; c < KC; ++c) {
+        const int k = lane * 4 + 256 * c;
+        v[b][c] = *reinterpret_cast<const float4*>(xr + (k < K ? k : 0));
+      }
     }
 #pragma unroll
-    for (int c = 0; c < KC; ++c)
-      if (lane * 4 + 256 * c < K) ss = rms_accumulate(ss, v[c]);
-    const float scale = rms_scale(ss, K, eps);
+    for (int b = 0; b < RB; ++b) {
+      const int m = r0 + NW * b;
+      float ss = 0.f;
 #pragma unroll
-    for (int c = 0; c < KC; ++c) {
-      const int k = lane * 4 + 256 * c;
-      if (k < K) {
-        const uint2 hb = make_uint2(pack_bf16x2(v[c].x * scale * g[c].x, v[c].y * scale * g[c].y),
-                                    pack_bf16x2(v[c].z * scale * g[c].z, v[c].w * scale * g[c].w));
-        *reinterpret_cast<uint2*>(sA + (size_t)m * lda + k) = hb;
+      for (int c = 0; c < KC; ++c)
+        if (lane * 4 + 256 * c < K) ss = rms_accumulate(ss, v[b][c]);
+      const float scale = rms_scale(ss, K, eps);
+      if (m < M) {
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+          const int k = lane * 4 + 256 * c;
+          if (k < K) {
+            const uint2 hb = make_uint2(pack_bf16x2(v[b][c].x * scale * g[c].x, v[b][c].y * scale * g[c].y),
+                                        pack_bf16x2(v[b][c].z * scale * g[c].z, v[b][c].w * scale * g[c].w));
+            *reinterpret_cast<uint2*>(sA + (size_t)m * lda + k) = hb;
+          }
+        }
       }
     }
   }
@@ -220,19 +247,24 @@ gemm_skinny_normed_kernel(const float* __restrict__ X, const float* __restrict__
     if (c0 != wave) {
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
-        const bool mine = c0 + NW * u < chunks;
-        w0[u].u = mine ? ld16(wp + (size_t)(c0 + NW * u) * 64) : zero;
-        w1[u].u = mine ? ld16(wp + (size_t)(c0 + NW * u) * 64 + 8) : zero;
+        const int c = c0 + NW * u < chunks ? c0 + NW * u : 0;
+        w0[u].u = ld16(wp + (size_t)c * 64);
+        w1[u].u = ld16(wp + (size_t)c * 64 + 8);
       }
     }
+    Frag a0[UN], a1[UN];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const bool mine = aok && (c0 + NW * u < chunks);
-      Frag a0, a1;
-      a0.u = mine ? ld16(ap + (size_t)(c0 + NW * u) * 64) : zero;
-      a1.u = mine ? ld16(ap + (size_t)(c0 + NW * u) * 64 + 8) : zero;
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u].v, a0.v, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, a1.v, acc, 0, 0, 0);
+      const int c = c0 + NW * u < chunks ? c0 + NW * u : 0;
+      a0[u].u = ld16(ap + (size_t)c * 64);
+      a1[u].u = ld16(ap + (size_t)c * 64 + 8);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      if (c0 + NW * u >= chunks) w0[u].u = w1[u].u = zero;
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u].v, a0[u].v, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, a1[u].v, acc, 0, 0, 0);
     }
   }
 #pragma unroll
@@ -793,6 +825,15 @@ static void launch_skinny(const bf16_t* A, const bf16_t* W, void* out, int M, in
       gemm_skinny_kernel<MTV, EPI, 8><<<grid, 512, 0, s>>>(A, W, out, M, N, K, lda); \
     else                                                                             \
       gemm_skinny_kernel<MTV, EPI, 4><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda); \
+  }
+  // up to 16 tokens: a wavefront whose share of K is more than four chunks takes eight at a
+  // time, so that one round trip to memory serves K up to 512 per wavefront
+  if (mt == 1 && (K + 63) / 64 > 4 * waves) {
+    if (waves == 8)
+      gemm_skinny_kernel<1, EPI, 8, 8><<<grid, 512, 0, s>>>(A, W, out, M, N, K, lda);
+    else
+      gemm_skinny_kernel<1, EPI, 4, 8><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
+    return;
   }
   TI_SKINNY(1)
   TI_SKINNY(2)
