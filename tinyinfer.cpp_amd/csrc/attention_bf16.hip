@@ -467,44 +467,47 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
   }
 }
 
-// grid (rows, n_head), max(HD, 64) threads: out = sum_s w_s o_s / sum_s w_s l_s, w_s = exp(m_s - max m).
-// The statistics of all splits are fetched at once into LDS and the partial outputs
-// in batches of eight independent loads: the kernel waits for memory a few times,
-// not once per split.
+// grid (rows, n_head), max(HD, 64) threads: out = sum_s w_s o_s / sum_s w_s l_s, w_s = 2^(m_s - max m).
+// The partial outputs are fetched in batches of eight independent loads: the kernel waits for
+// memory a few times, not once per split.
 #define MERGE_MAX_SPLITS 64
 template <int HD>
 __global__ void __launch_bounds__(HD < 64 ? 64 : HD)
 attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                   const int* __restrict__ rows, bf16_t* __restrict__ out, int n_head, int n_splits) {
-  __shared__ float s_w[MERGE_MAX_SPLITS];
-  __shared__ float s_inv;
   const int ridx = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
-  const int m_row = rows ? rows[ridx] : ridx;
-  const float* pm = part_ml + ((size_t)ridx * n_head + head) * n_splits * 2;
-  const float* po = part_o + ((size_t)ridx * n_head + head) * n_splits * HD;
-  // one wavefront fetches (max, sum) of every split and turns them into weights
-  if (d < 64) {
-    const float ms = (d < n_splits) ? pm[2 * d] : -INFINITY;
-    const float ls = (d < n_splits) ? pm[2 * d + 1] : 0.f;
-    const float mm = group_max<64>(ms);
-    const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - mm);
-    const float lt = group_sum<64>(ls * w);
-    s_w[d] = w;
-    if (d == 0) s_inv = 1.0f / lt;
-  }
-  __syncthreads();
   if (d >= HD) return;
-  float acc = 0.f;
+  const int m_row = rows ? rows[ridx] : ridx;
+  const float2* pm = reinterpret_cast<const float2*>(part_ml) + ((size_t)ridx * n_head + head) * n_splits;
+  const float* po = part_o + ((size_t)ridx * n_head + head) * n_splits * HD + d;
+  // every thread works the weights of the splits out for itself: they are few, and no thread waits
+  // for another
+  float mm = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, pm[s].x);
+  float acc = 0.f, lt = 0.f;
   int s = 0;
   for (; s + 8 <= n_splits; s += 8) {
     float v[8];
+    float2 ml[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = po[(size_t)(s + j) * HD + d];
+    for (int j = 0; j < 8; ++j) {
+      v[j] = po[(size_t)(s + j) * HD];
+      ml[j] = pm[s + j];
+    }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc += v[j] * s_w[s + j];
+    for (int j = 0; j < 8; ++j) {
+      const float w = split_weight(ml[j].x, mm);
+      lt = fmaf(ml[j].y, w, lt);
+      acc = split_accumulate(acc, v[j], w);
+    }
   }
-  for (; s < n_splits; ++s) acc += po[(size_t)s * HD + d] * s_w[s];
-  out[((size_t)m_row * n_head + head) * HD + d] = f2bf(acc * s_inv);
+  for (; s < n_splits; ++s) {
+    const float2 ml = pm[s];
+    const float w = split_weight(ml.x, mm);
+    lt = fmaf(ml.y, w, lt);
+    acc = split_accumulate(acc, po[(size_t)s * HD], w);
+  }
+  out[((size_t)m_row * n_head + head) * HD + d] = f2bf(acc * (1.0f / lt));
 }
 
 // ================================================================== prefill

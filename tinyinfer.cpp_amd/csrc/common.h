@@ -67,6 +67,19 @@ __device__ __forceinline__ float rms_scale(float lane_acc, int width, float eps)
   return 1.0f / sqrtf(group_sum<TI_WAVE>(lane_acc) / (float)width + eps);
 }
 
+// The merge of an attention that was split over the context.  Split s of a (row, head) left
+// (m_s, l_s): its maximum in the exp2 domain and the sum of its weights, and o_s, its
+// weighted values.  With mm = max_s m_s and w_s = 2^(m_s - mm), the merged row is
+// (sum_s o_s w_s) / (sum_s l_s w_s), both sums taken in ascending order of s with fused
+// multiply-adds.  Every kernel that merges goes through these functions: same bits.
+__device__ __forceinline__ float split_weight(float m_s, float mm) {
+  return (m_s == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_s - mm);
+}
+__device__ __forceinline__ float split_accumulate(float acc, float o_s, float w) { return fmaf(o_s, w, acc); }
+__device__ __forceinline__ float4 split_accumulate(float4 acc, float4 o_s, float w) {
+  return make_float4(fmaf(o_s.x, w, acc.x), fmaf(o_s.y, w, acc.y), fmaf(o_s.z, w, acc.z), fmaf(o_s.w, w, acc.w));
+}
+
 // sum over a workgroup of NT threads (NT multiple of 64, <= 1024); `red` holds
 // NT/64 floats of LDS.  Every thread gets the total.  Fixed order: deterministic.
 template <int NT> __device__ __forceinline__ float block_sum(float v, float* red) {

@@ -69,11 +69,11 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, v
   // the residual this thread will add to, asked for before the product
   const int tok = threadIdx.x >> 4, row = threadIdx.x & 15;
   float prev[MT];
-  if (EPI == TI_EPI_ADD_F32 && threadIdx.x < 256) {
+  if (EPI == TI_EPI_ADD_F32) {   // threads without an output element read a valid one: no branch
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      const int m = t * 16 + tok, n = blockIdx.x * 16 + row;
-      prev[t] = (m < M && n < N) ? ((const float*)out_)[(size_t)m * N + n] : 0.f;
+      const int m = t * 16 + (tok & 15), n = blockIdx.x * 16 + row;
+      prev[t] = ((const float*)out_)[(size_t)(m < M ? m : 0) * N + (n < N ? n : N - 1)];
     }
   }
   floatx4 acc[MT];
@@ -152,18 +152,84 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, v
   }
 }
 
-// ============================================= skinny kernel with an RMSNorm in front
-// out = rmsnorm(x; nw, eps) W^T for M <= 16 tokens.  The norm that stands before a
-// projection is computed by every workgroup for itself: the rows are few and lie in the
-// cache, the first weight loads are already under way while it runs, and it costs no
-// launch of its own.  x: float [M, K]; nw: norm weight [K].  The normed rows go to LDS as
-// bfloat16 (the rounding every product operand gets, so the result equals that of the
-// norm kernel followed by the plain product) and the main loop reads its token fragments
-// from there.  KC: float4 pieces of a row each lane holds (K <= 256 KC).
-template <int EPI, int KC, int NW>
+// ================================== skinny kernel whose token rows are made in the kernel
+// out = rows W^T for M <= 16 tokens, where the rows do not exist in memory yet: a producer
+// makes them, as bfloat16 in LDS, in every workgroup for itself.  The rows are few and what
+// they are made from lies in the cache; the first weight loads are already under way while
+// the producer runs; and it costs no launch of its own.  The rounding to bfloat16 is the
+// one every product operand gets, so the result equals that of the producer's own kernel
+// followed by the plain product.
+//
+// A producer has `template <int NW> __device__ void fill(bf16_t* sA, int lda, int M, int K)`,
+// called by all NW * 64 threads, writing sA[m * lda + k]; the kernel synchronizes after it.
+
+// RMSNorm of float rows X [M, K] with weight Gw [K].  KC: float4 pieces of a row each lane
+// holds (K <= 256 KC).  Wavefront w takes rows w, w + NW, ...; two rows' loads are issued
+// together where the registers allow; a lane's pieces beyond K read piece 0 and are left
+// out of the sum and the store.
+template <int KC>
+struct NormProducer {
+  const float* X;
+  const float* Gw;
+  float eps;
+  template <int NW, class IssueWeights>
+  __device__ __forceinline__ void fill(bf16_t* sA, int lda, int M, int K, IssueWeights issue_weights) const {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    constexpr int RB = KC <= 8 ? 2 : 1;
+    float4 g[KC], v[RB][KC];
+    auto load_rows = [&](int r0) {
+#pragma unroll
+      for (int b = 0; b < RB; ++b) {
+        const int m = r0 + NW * b < M ? r0 + NW * b : (r0 < M ? r0 : 0);
+        const float* xr = X + (size_t)m * K;
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+          const int k = lane * 4 + 256 * c;
+          v[b][c] = *reinterpret_cast<const float4*>(xr + (k < K ? k : 0));
+        }
+      }
+    };
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int k = lane * 4 + 256 * c;
+      g[c] = *reinterpret_cast<const float4*>(Gw + (k < K ? k : 0));
+    }
+    load_rows(wave);
+    // loads come back in the order they were issued: the rows (from the cache) before the
+    // weights (from memory), so the norm does not wait for the weights
+    __builtin_amdgcn_sched_barrier(0);
+    issue_weights();
+    __builtin_amdgcn_sched_barrier(0);
+    for (int r0 = wave; r0 < M; r0 += NW * RB) {
+      if (r0 != wave) load_rows(r0);
+#pragma unroll
+      for (int b = 0; b < RB; ++b) {
+        const int m = r0 + NW * b;
+        float ss = 0.f;
+#pragma unroll
+        for (int c = 0; c < KC; ++c)
+          if (lane * 4 + 256 * c < K) ss = rms_accumulate(ss, v[b][c]);
+        const float scale = rms_scale(ss, K, eps);
+        if (m < M) {
+#pragma unroll
+          for (int c = 0; c < KC; ++c) {
+            const int k = lane * 4 + 256 * c;
+            if (k < K) {
+              const uint2 hb = make_uint2(pack_bf16x2(v[b][c].x * scale * g[c].x, v[b][c].y * scale * g[c].y),
+                                          pack_bf16x2(v[b][c].z * scale * g[c].z, v[b][c].w * scale * g[c].w));
+              *reinterpret_cast<uint2*>(sA + (size_t)m * lda + k) = hb;
+            }
+          }
+        }
+      }
+    }
+  }
+};
+
+template <class Producer, int EPI, int NW>
 __global__ void __launch_bounds__(NW * 64)
-gemm_skinny_normed_kernel(const float* __restrict__ X, const float* __restrict__ Gw, float eps,
-                          const bf16_t* __restrict__ W, void* __restrict__ out_, int M, int N, int K) {
+gemm_skinny_staged_kernel(Producer producer, const bf16_t* __restrict__ W, void* __restrict__ out_, int M, int N,
+                          int K) {
   constexpr bool SW = (EPI == TI_EPI_SWIGLU);
   extern __shared__ __attribute__((aligned(16))) unsigned char dyn_smem[];
   bf16_t* sA = reinterpret_cast<bf16_t*>(dyn_smem);          // [M][K + 8]
@@ -184,64 +250,31 @@ gemm_skinny_normed_kernel(const float* __restrict__ X, const float* __restrict__
   const int chunks = K / 64;
   constexpr int UN = 4;
 
-  // the first weights of this wavefront: on their way while the norm is computed.  A chunk
-  // beyond the last reads chunk 0 and is zeroed afterwards: no branch between the loads.
-  Frag w0[UN], w1[UN];
-#pragma unroll
-  for (int u = 0; u < UN; ++u) {
-    const int c = wave + NW * u < chunks ? wave + NW * u : 0;
-    w0[u].u = ld16(wp + (size_t)c * 64);
-    w1[u].u = ld16(wp + (size_t)c * 64 + 8);
+  // the residual this thread will add to
+  const int tok = threadIdx.x >> 4, row = threadIdx.x & 15;   // tok >= 16 for the wavefronts beyond four
+  float prev = 0.f;
+  if (EPI == TI_EPI_ADD_F32) {   // threads without an output element read a valid one: no branch
+    const int n = blockIdx.x * 16 + row;
+    prev = ((const float*)out_)[(size_t)(tok < M ? tok : 0) * N + (n < N ? n : N - 1)];
   }
 
-  // ---- the norm: wavefront w takes rows w, w + NW, ...; a lane holds KC float4 of a row.
-  // Two rows' loads are issued together where the registers allow; a lane's pieces beyond
-  // K read piece 0 and are left out of the sum and the store.
-  float4 g[KC];
+  // the first weights of this wavefront: the producer asks for them right after its own first
+  // loads, so that they are on their way while the rows are made.  A chunk beyond the last
+  // reads chunk 0 and is zeroed afterwards: no branch between the loads.
+  Frag w0[UN], w1[UN];
+  auto issue_weights = [&]() {
 #pragma unroll
-  for (int c = 0; c < KC; ++c) {
-    const int k = lane * 4 + 256 * c;
-    g[c] = *reinterpret_cast<const float4*>(Gw + (k < K ? k : 0));
-  }
-  constexpr int RB = KC <= 8 ? 2 : 1;
-  for (int r0 = wave; r0 < M; r0 += NW * RB) {
-    float4 v[RB][KC];
-#pragma unroll
-    for (int b = 0; b < RB; ++b) {
-      const int m = r0 + NW * b < M ? r0 + NW * b : r0;
-      const float* xr = X + (size_t)m * K;
-#pragma unroll
-      for (int c = 0; c < KC; ++c) {
-        const int k = lane * 4 + 256 * c;
-        v[b][c] = *reinterpret_cast<const float4*>(xr + (k < K ? k : 0));
-      }
+    for (int u = 0; u < UN; ++u) {
+      const int c = wave + NW * u < chunks ? wave + NW * u : 0;
+      w0[u].u = ld16(wp + (size_t)c * 64);
+      w1[u].u = ld16(wp + (size_t)c * 64 + 8);
     }
-#pragma unroll
-    for (int b = 0; b < RB; ++b) {
-      const int m = r0 + NW * b;
-      float ss = 0.f;
-#pragma unroll
-      for (int c = 0; c < KC; ++c)
-        if (lane * 4 + 256 * c < K) ss = rms_accumulate(ss, v[b][c]);
-      const float scale = rms_scale(ss, K, eps);
-      if (m < M) {
-#pragma unroll
-        for (int c = 0; c < KC; ++c) {
-          const int k = lane * 4 + 256 * c;
-          if (k < K) {
-            const uint2 hb = make_uint2(pack_bf16x2(v[b][c].x * scale * g[c].x, v[b][c].y * scale * g[c].y),
-                                        pack_bf16x2(v[b][c].z * scale * g[c].z, v[b][c].w * scale * g[c].w));
-            *reinterpret_cast<uint2*>(sA + (size_t)m * lda + k) = hb;
-          }
-        }
-      }
-    }
-  }
+  };
+  producer.template fill<NW>(sA, lda, M, K, issue_weights);
   __syncthreads();
 
   // ---- the product, as in the plain skinny kernel with the token fragments from LDS
-  const bool aok = r < M;
-  const bf16_t* ap = sA + (size_t)(aok ? r : 0) * lda + j * 16;
+  const bf16_t* ap = sA + (size_t)(r < M ? r : 0) * lda + j * 16;
   floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
   for (int c0 = wave; c0 < chunks; c0 += NW * UN) {
     if (c0 != wave) {
@@ -270,7 +303,6 @@ gemm_skinny_normed_kernel(const float* __restrict__ X, const float* __restrict__
 #pragma unroll
   for (int i = 0; i < 4; ++i) red[wave][r][4 * j + i] = acc[i];
   __syncthreads();
-  const int tok = threadIdx.x >> 4, row = threadIdx.x & 15;   // tok >= 16 for the wavefronts beyond four
   if (tok >= M) return;
   if (SW) {
     if (row >= 8) return;
@@ -291,7 +323,7 @@ gemm_skinny_normed_kernel(const float* __restrict__ X, const float* __restrict__
     for (int w = 0; w < NW; ++w) sum += red[w][tok][row];
     const size_t o = (size_t)tok * N + n;
     if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = sum;
-    if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] += sum;
+    if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] = prev + sum;
     if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(sum);
   }
 }
@@ -810,6 +842,9 @@ static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M,
 // more loads in flight.  0 = choose by the shape.
 static int g_skinny_waves = 0;
 extern "C" void ti_gemm_bf16_skinny_waves(int waves) { g_skinny_waves = waves; }
+// 1 (default): eight chunks of K in flight per wavefront where its share of K is more than four
+static int g_skinny_deep = 1;
+extern "C" void ti_gemm_bf16_skinny_deep(int on) { g_skinny_deep = on; }
 
 template <int EPI>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
@@ -828,7 +863,7 @@ static void launch_skinny(const bf16_t* A, const bf16_t* W, void* out, int M, in
   }
   // up to 16 tokens: a wavefront whose share of K is more than four chunks takes eight at a
   // time, so that one round trip to memory serves K up to 512 per wavefront
-  if (mt == 1 && (K + 63) / 64 > 4 * waves) {
+  if (mt == 1 && (K + 63) / 64 > 4 * waves && g_skinny_deep) {
     if (waves == 8)
       gemm_skinny_kernel<1, EPI, 8, 8><<<grid, 512, 0, s>>>(A, W, out, M, N, K, lda);
     else
@@ -850,7 +885,29 @@ static void launch_tiled(const bf16_t* A, const bf16_t* W, void* out, int M, int
   gemm_tiled_kernel<EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
 }
 
-// out = rmsnorm(x; nw, eps) W^T for M <= 16 (see gemm_skinny_normed_kernel).  Returns 3 for
+template <class Producer, int EPI, int NW>
+static int launch_staged(const char* what, Producer producer, const bf16_t* w, void* out, int M, int N, int K,
+                         int grid, hipStream_t stream) {
+  const size_t lds = (size_t)M * (K + 8) * 2;
+  auto kern = gemm_skinny_staged_kernel<Producer, EPI, NW>;
+  static size_t allowed = 48 * 1024;   // per instantiation: the largest size asked for so far
+  if (lds > allowed) {
+    TI_REQUIRE(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) ==
+                   hipSuccess, "%s: LDS size refused", what);
+    allowed = lds;
+  }
+  kern<<<grid, NW * 64, lds, stream>>>(producer, w, out, M, N, K);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// The number of wavefronts the plain skinny kernel takes for this weight: the kernels that
+// make their rows themselves take the same, so that they give the same bits.
+static int skinny_waves_for(int grid, int K) {
+  return g_skinny_waves ? g_skinny_waves : ((grid <= 128 && K >= 1024) ? 8 : 4);
+}
+
+// out = rmsnorm(x; nw, eps) W^T for M <= 16 (see gemm_skinny_staged_kernel).  Returns 3 for
 // sizes it does not serve (M > 16, K not a multiple of 64 or above 4096).
 extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, const void* W, void* out,
                                    int M, int N, int K, int epi, hipStream_t stream) {
@@ -860,32 +917,21 @@ extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, c
     return 3;
   }
   if (M == 0) return 0;
-  const size_t lds = (size_t)M * (K + 8) * 2;
   const bf16_t* w = (const bf16_t*)W;
   const int grid = (epi == TI_EPI_SWIGLU) ? (N + 7) / 8 : (N + 15) / 16;
   const int kc = (K + 255) / 256;
-  // the same number of wavefronts as the plain skinny kernel takes for this weight: same bits
-  int waves = g_skinny_waves;
-  if (waves == 0) waves = (grid <= 128 && K >= 1024) ? 8 : 4;
-#define TI_GNW(E, KCV, NWV)                                                                                 \
-  {                                                                                                         \
-    auto kern = gemm_skinny_normed_kernel<E, KCV, NWV>;                                                     \
-    if (lds > 48 * 1024)                                                                                    \
-      TI_REQUIRE(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,         \
-                                     (int)lds) == hipSuccess, "gemm_bf16_normed: LDS size refused");        \
-    kern<<<grid, NWV * 64, lds, stream>>>(x, nw, eps, w, out, M, N, K);                                     \
-  }
-#define TI_GNK(E, KCV)                \
-  {                                   \
-    if (waves == 8) TI_GNW(E, KCV, 8) \
-    else TI_GNW(E, KCV, 4)            \
-  }
+  const int waves = skinny_waves_for(grid, K);
+#define TI_GNK(E, KCV)                                                                                          \
+  return waves == 8                                                                                             \
+             ? launch_staged<NormProducer<KCV>, E, 8>("gemm_bf16_normed", NormProducer<KCV>{x, nw, eps}, w, out, \
+                                                      M, N, K, grid, stream)                                    \
+             : launch_staged<NormProducer<KCV>, E, 4>("gemm_bf16_normed", NormProducer<KCV>{x, nw, eps}, w, out, \
+                                                      M, N, K, grid, stream);
 #define TI_GN(E)                        \
   case E:                               \
     if (kc <= 4) TI_GNK(E, 4)           \
     else if (kc <= 8) TI_GNK(E, 8)      \
-    else TI_GNK(E, 16)                  \
-    break;
+    else TI_GNK(E, 16)
   switch (epi) {
     TI_GN(TI_EPI_STORE_F32)
     TI_GN(TI_EPI_ADD_F32)
@@ -896,8 +942,6 @@ extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, c
   }
 #undef TI_GN
 #undef TI_GNK
-#undef TI_GNW
-  TI_LAUNCH_CHECK();
   return 0;
 }
 
