@@ -16,7 +16,6 @@ and the state live in `CacheStorage`.
 """
 from __future__ import annotations
 
-import random
 
 import numpy as np
 from dataclasses import dataclass
@@ -34,20 +33,13 @@ class OutOfPages(CacheError):
 
 
 class PagePool:
-    """Page ids 0..num_pages-1 with a LIFO free list.
+    """Page ids 0..num_pages-1 with a LIFO free list."""
 
-    `scatter`: the pages are first handed out in a fixed pseudo-random order instead of 0, 1, 2, ...
-    Requests that are filled one after the other then do not lie at equal distances in memory;
-    at equal distances (a few MiB) the attention kernels, which walk all requests in step, keep
-    hitting the same memory channels (measured on MI355X: 4.7 against 5.6 TB/s at batch 64)."""
-
-    def __init__(self, num_pages: int, scatter: bool = False):
+    def __init__(self, num_pages: int):
         if num_pages <= 0:
             raise CacheError(f"a page pool needs at least one page, got {num_pages}")
         self.num_pages = int(num_pages)
         self._free: List[int] = list(range(self.num_pages - 1, -1, -1))   # pop() gives page 0 first
-        if scatter:
-            random.Random(self.num_pages).shuffle(self._free)
         self._held = [False] * self.num_pages
         self.high_water = 0
         self.taken_total = 0          # pages handed out so far, counting a page again each time
@@ -83,12 +75,11 @@ class _Request:
 class PagedGroup:
     """Pages and block tables of one group of layers."""
 
-    def __init__(self, need: PagedKVNeed, n_layers: int, page_size: int, num_pages: int, table_width: int,
-                 scatter: bool = False):
+    def __init__(self, need: PagedKVNeed, n_layers: int, page_size: int, num_pages: int, table_width: int):
         self.need = need
         self.n_layers = n_layers
         self.page_size = page_size
-        self.pool = PagePool(num_pages, scatter)
+        self.pool = PagePool(num_pages)
         self.tables: Dict[Hashable, List[int]] = {}      # -1: given back (behind the window)
         # the same as rows of `table_width` int32 (-1 where there is no page), ready to be
         # copied into a step's metadata
@@ -139,7 +130,7 @@ class CacheManager:
     """
 
     def __init__(self, groups: Sequence[Tuple[object, int]], page_size: int, num_pages: int,
-                 max_requests: int, max_seq: int, scatter_pages: bool = False):
+                 max_requests: int, max_seq: int):
         if page_size <= 0:
             raise CacheError("page_size must be positive")
         self.page_size = int(page_size)
@@ -150,7 +141,7 @@ class CacheManager:
         for need, n_layers in groups:
             if isinstance(need, PagedKVNeed):
                 self.groups.append(PagedGroup(need, n_layers, self.page_size, num_pages,
-                                              self.max_pages_per_request, scatter_pages))
+                                              self.max_pages_per_request))
             elif isinstance(need, StateNeed):
                 self.groups.append(need)
             else:

@@ -117,8 +117,7 @@ class Engine:
             if model.spec.max_position_embeddings:
                 max_seq = min(max_seq, model.spec.max_position_embeddings)
         self.max_seq = int(max_seq)
-        self.cache = CacheManager(model.cache_groups, self.page_size, self.num_pages, max_requests, self.max_seq,
-                                  scatter_pages=True)
+        self.cache = CacheManager(model.cache_groups, self.page_size, self.num_pages, max_requests, self.max_seq)
         self.storage = CacheStorage(self.cache, self.act_dtype, self.device)
         self.table_width = self.cache.max_pages_per_request
         for part in model.parts():
