@@ -590,6 +590,9 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
 #pragma unroll
   for (int ks = 0; ks < PBK / 16; ++ks) xo[ks] = ((ks * 2 + fh) ^ ((fr >> 1) & 7)) << 4;
 
+  // the residual an adding epilogue adds to: asked for while the last k-tile is multiplied
+  // (elements outside the matrix read a valid one and are not stored)
+  float prev[EPI == TI_EPI_ADD_F32 ? TM : 1][EPI == TI_EPI_ADD_F32 ? TN : 1][16];
   const int n_k = K / PBK;
   issue(0);
   if (n_k > 1) issue(1);
@@ -599,6 +602,20 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
     if (kt + 1 < n_k) wait_vmcnt(LOADS); else wait_vmcnt(0);
     __builtin_amdgcn_s_barrier();
     if (kt + 2 < n_k) issue(kt + 2);
+    if constexpr (EPI == TI_EPI_ADD_F32) {
+      if (kt == n_k - 1) {
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+          for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int m = m0 + wm * (BM / WAVES_M) + a * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+              const int n = n0 + wn * (BN / WAVES_N) + b * 32 + (lane & 31);
+              prev[a][b][i] = ((const float*)out_)[(size_t)min(m, M - 1) * N + min(n, N - 1)];
+            }
+      }
+    }
     const unsigned st = (kt % PSTAGES) * STAGE_BYTES;
     v4u fa[2][TM], fb[2][TN];
     auto read_step = [&](int ks, int set) {
@@ -747,7 +764,7 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
           const size_t o = (size_t)m * N + n;
           const float v = acc[a][b][i];
           if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = v;
-          if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] += v;
+          if constexpr (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] = prev[a][b][i] + v;
           if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(v);
         }
       }
