@@ -598,7 +598,7 @@ class FakeCtx:
     def __init__(self, entries, decode_rows_only=False):
         # entries: [(n_tokens, start_pos)], rows laid out in order
         self.entries = entries
-        pos, slot, tiles, dec, meta = [], [], [], [], []
+        pos, slot, tiles, dec, meta, small = [], [], [], [], [], []
         row0 = 0
         for e, (n, start) in enumerate(entries):
             meta.append([row0, n, start, 0])
@@ -606,9 +606,13 @@ class FakeCtx:
             slot += [e] * n
             if n > 1:
                 tiles += [[e, row0 + q0] for q0 in range(0, n, 128)]
+                small += [(start + min(q0 + 64, n) - 1, e, row0 + q0) for q0 in range(0, n, 64)]
             else:
                 dec.append(row0)
             row0 += n
+        small.sort(key=lambda t: -t[0])             # from the tile that sees the most keys to the fewest
+        self.tiles_small = dev(torch.tensor([t[1:] for t in small], dtype=torch.int32)) if small else None
+        self.n_tiles_small = len(small)
         self.M = row0
         self.decode_only = not tiles
         self.positions = dev(torch.tensor(pos, dtype=torch.int32))
@@ -683,22 +687,44 @@ def test_attention_bf16_decode_rows(ops, nh, nkv, hd, P, window):
 @pytest.mark.parametrize("nh,nkv,hd,P,window", [
     (4, 2, 64, 16, None), (6, 2, 32, 16, None), (4, 2, 128, 16, None), (2, 1, 128, 32, None),
     (4, 4, 64, 16, 40), (2, 2, 32, 16, 7)])
-@pytest.mark.parametrize("groups", [1, 2])
-def test_attention_bf16_portions_and_mixed(ops, nh, nkv, hd, P, window, groups):
+@pytest.mark.parametrize("variant", ["one group", "two groups", "paired"])
+def test_attention_bf16_portions_and_mixed(ops, nh, nkv, hd, P, window, variant):
     """Portions of every size, starting anywhere (a page's edge, the middle of a
     page, the start of a request), beside decode rows; with one and with two groups of
-    wavefronts per workgroup (the launch would choose by its size)."""
+    wavefronts per workgroup, and with the kernel that gives a workgroup two tiles of
+    64 rows (the launch would choose by its size)."""
     if not ops.use_fast_attention:
         pytest.skip("bfloat16 attention kernels are switched off")
-    entries = [(2, 0), (7, 30), (1, 99), (16, 16), (17, 15), (64, 0), (65, 63), (130, 41), (1, 0), (3, 300), (200, 5)]
+    entries = [(2, 0), (7, 30), (1, 99), (16, 16), (17, 15), (64, 0), (65, 63), (130, 41), (1, 0), (3, 300), (200, 5),
+               (333, 700)]
     lib = ops.lib("attention_bf16")
-    lib.ti_attention_prefill_groups(groups)
+    lib.ti_attention_prefill_groups({"one group": 1, "two groups": 2, "paired": 0}[variant])
+    ops.use_paired_prefill = variant == "paired"
     try:
         got, want = fast_attention_case(ops, entries, nh, nkv, hd, P, window, seed=nh * 10 + hd)
     finally:
         lib.ti_attention_prefill_groups(0)
+        ops.use_paired_prefill = True
     assert torch.isfinite(got).all()
     assert (got - want).abs().max() < 2e-2
+
+
+def test_attention_bf16_paired_tiles_of_one_long_prompt(ops):
+    """A prompt of 1,100 tokens in one step (an odd number of 64-row tiles, the last one short):
+    the kernel that pairs the tile of the most keys with the one of the fewest, against the
+    kernel that takes one tile of 128 rows per workgroup and against the softmax in float64."""
+    if not ops.use_fast_attention:
+        pytest.skip("bfloat16 attention kernels are switched off")
+    outs = []
+    try:
+        for paired in (True, False):
+            ops.use_paired_prefill = paired
+            got, want = fast_attention_case(ops, [(1100, 0), (1, 40)], 4, 2, 128, 16, None, seed=5)
+            assert (got - want).abs().max() < 2e-2
+            outs.append(got)
+    finally:
+        ops.use_paired_prefill = True
+    assert (outs[0] - outs[1]).abs().max() < 2e-2
 
 
 @pytest.mark.parametrize("nh,nkv,hd,P,window,norm,rope", [

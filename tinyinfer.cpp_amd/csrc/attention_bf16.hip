@@ -604,10 +604,10 @@ __device__ __forceinline__ void lgkm_wait(int n) {
 }
 // wait until at most k * LOADS vector-memory operations are outstanding
 // (s_waitcnt with only vmcnt set: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
-template <int LOADS>
+template <int LOADS, int STAGES>
 __device__ __forceinline__ void vm_wait_turns(int k) {
 #define TI_VM(N) __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | ((((N) >> 4) & 3) << 14))
-  static_assert(LOADS * (PF_STAGES - 2) <= 63, "vmcnt has six bits");
+  static_assert(LOADS * (STAGES - 2) <= 63, "vmcnt has six bits");
   switch (k) {
     case 0: TI_VM(0); break;
     case 1: TI_VM(LOADS); break;
@@ -621,21 +621,25 @@ __device__ __forceinline__ void vm_wait_turns(int k) {
 #undef TI_VM
 }
 
-// NG: groups of four wavefronts in the workgroup (1 or 2).  Every group takes all 128 rows, a
-// column block of 32 tokens per wavefront; with two groups the turns go to them alternately
-// (each group loads and walks its own turns through its own LDS stages) and their partial
-// results are merged through LDS at the end.  Two groups put two wavefronts on every SIMD
-// when a launch has only one workgroup per compute unit, so that one's loads, LDS reads and
-// vector work hide behind the other's matrix products.
-template <int HD, int NG>
-__global__ void __launch_bounds__(256 * NG)
+// NG groups of NW wavefronts in the workgroup.  A tile is 32 NW rows: a column block of 32
+// tokens per wavefront of a group, and every group takes all of the tile's rows.  With more
+// than one group the turns (32 keys) go to the groups in rotation (each group loads and walks
+// its own turns through its own ST LDS stages) and their partial results are merged through
+// LDS at the end.  More groups put two wavefronts on every SIMD when a launch has only one
+// workgroup per compute unit, so that one's loads, LDS reads and vector work hide behind the
+// other's matrix products.
+// PAIRED: a workgroup takes two tiles, one after the other: tiles[blockIdx.x] and
+// tiles[n_tiles - 1 - blockIdx.x] of a list ordered from the most keys to the fewest, so that
+// under a causal mask every workgroup of a launch has about the same work.
+template <int HD, int NG, int NW = 4, int ST = PF_STAGES, bool PAIRED = false>
+__global__ void __launch_bounds__(64 * NW * NG)
 attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool,
                         const int* __restrict__ table, int table_stride, const int* __restrict__ tiles,
-                        const int* __restrict__ entries, bf16_t* __restrict__ out, int n_head, int n_kv, int P,
-                        float scale, int window) {
+                        int n_tiles, const int* __restrict__ entries, bf16_t* __restrict__ out, int n_head,
+                        int n_kv, int P, float scale, int window) {
   constexpr int CB = 1;                               // column blocks (of 32 tokens) per wavefront
-  constexpr int NW = 4;                               // wavefronts of a group
   constexpr int WROWS = 32 * CB;                      // tokens per wavefront
+  constexpr int TROWS = NW * WROWS;                   // tokens per tile
   constexpr int NP = HD / 8;                          // 16-byte pieces per K row
   constexpr int K_BYTES = PF_KEYS * HD * 2;
   constexpr int STAGE = 2 * K_BYTES;                  // K tile + V^T tile
@@ -648,17 +652,66 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
   constexpr int DB = HD / 32;                         // 32-dim blocks of the output
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
-  const int entry = tiles[2 * blockIdx.x], first = tiles[2 * blockIdx.x + 1];
-  const int row0 = entries[4 * entry], n_tok = entries[4 * entry + 1], start = entries[4 * entry + 2];
-  const int head = blockIdx.y;
+  // Which (tile, head) this workgroup takes.  Workgroups go to the eight XCDs in turn (linear id
+  // mod 8) and each XCD has an L2 of its own: with a multiple of eight kv heads, an XCD is given
+  // whole kv heads, so that the keys and values of a head are read into one L2 only.
+  int head = blockIdx.y, bx = blockIdx.x;
+  if (n_kv % 8 == 0) {
+    const int id = blockIdx.y * gridDim.x + blockIdx.x;
+    const int xcd = id & 7, local = id >> 3;
+    const int per_kv = (n_head / n_kv) * gridDim.x;       // workgroups of one kv head
+    const int rest = local % per_kv;
+    head = (xcd + 8 * (local / per_kv)) * (n_head / n_kv) + rest / gridDim.x;
+    bx = rest % gridDim.x;
+  }
   const int grp = (threadIdx.x >> 6) / NW, wave = (threadIdx.x >> 6) % NW, lane = threadIdx.x & 63;
   const int r32 = lane & 31, h = lane >> 5;
-  const int row_end = row0 + n_tok;
-  const int kv_last = start + n_tok - 1;
   const int kvh = head / (n_head / n_kv);
   const size_t page_elems = (size_t)2 * n_kv * P * HD;
   const bf16_t* kpool = pool + (size_t)kvh * P * HD;
   const bf16_t* vpool = pool + (size_t)(n_kv + kvh) * P * HD;
+
+  // scores are kept in units of log 2: softmax weights are then bare exp2
+  const float scale2 = scale * 1.4426950408889634f;
+
+  // what this lane fetches in each of its loads of a turn
+  //  K load g: LDS rows K_ROWS g .. + K_ROWS - 1; lane i -> row r = K_ROWS g + i / NP, slot c = i % NP,
+  //            holds piece c ^ (r & (NP - 1)) of key 16 (r / 16) + swap23(r % 16)
+  //  V load g: dims 16 g .. 16 g + 15, 64 bytes each; lane i -> dim d = 16 g + i / 4, slot c = i % 4,
+  //            holds piece c ^ ((d >> 2) & 3): keys 16 (piece / 2) + 8 (piece % 2) .. + 7
+  // packed per load: (element offset inside the page, without the row of the block's first
+  // key) * 2 + (which 16-key block of the turn).  Loads j < MY_K are K loads.
+  int ld_desc[MY_LOADS];
+#pragma unroll
+  for (int j = 0; j < MY_LOADS; ++j) {
+    if (j < MY_K) {
+      const int g = wave + NW * j;
+      const int r = K_ROWS * g + lane / NP, c = lane % NP;
+      const int r16 = r & 15;
+      const int key16 = ((r16 & 4) << 1) | ((r16 & 8) >> 1) | (r16 & 3);
+      ld_desc[j] = (key16 * HD + (c ^ (r & (NP - 1))) * 8) * 2 + (r >> 4);
+    } else {
+      const int gv = wave + NW * (j - MY_K);
+      const int d = 16 * gv + (lane >> 2), c = lane & 3;
+      const int piece = c ^ ((d >> 2) & 3);
+      ld_desc[j] = (d * P + (piece & 1) * 8) * 2 + (piece >> 1);
+    }
+  }
+
+  const unsigned lds0 = (unsigned)(size_t)smem + grp * (ST * STAGE);   // this group's stages
+  // LDS addresses of this lane's fragments (without stage and k-step)
+  const unsigned k_row = lds0 + r32 * (HD * 2);                     // K row r32
+  const unsigned v_row = lds0 + K_BYTES + r32 * 64;                 // V^T row (dim) r32 of a 32-dim block
+
+  int turn_count = 0;                                               // turns so far: picks the stage
+  for (int slot = 0; slot < (PAIRED ? 2 : 1); ++slot) {
+  // ---- this slot's tile
+  const int tile = (slot == 0) ? bx : n_tiles - 1 - bx;
+  if (PAIRED && slot == 1 && tile <= bx) break;                     // an odd count: the middle tile came first
+  const int entry = tiles[2 * tile], first = tiles[2 * tile + 1];
+  const int row0 = entries[4 * entry], n_tok = entries[4 * entry + 1], start = entries[4 * entry + 2];
+  const int row_end = row0 + n_tok;
+  const int kv_last = start + n_tok - 1;
   const int* tab = table + (size_t)entry * table_stride;
 
   // this wavefront: rows w_first .. w_first + WROWS - 1, in column blocks of 32
@@ -666,13 +719,10 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
   const int w_rows = max(0, min(WROWS, row_end - w_first));
   const int w_pos_first = start + (w_first - row0), w_pos_last = w_pos_first + w_rows - 1;
   const int w_lo = (window > 0 && w_pos_first - window + 1 > 0) ? w_pos_first - window + 1 : 0;
-  // the workgroup: rows first .. first + 127
-  const int g_rows = min(PF_ROWS, row_end - first);
+  // the workgroup: rows first .. first + TROWS - 1
+  const int g_rows = min(TROWS, row_end - first);
   const int g_pos_first = start + (first - row0), g_pos_last = g_pos_first + g_rows - 1;
   const int g_lo = (window > 0 && g_pos_first - window + 1 > 0) ? g_pos_first - window + 1 : 0;
-
-  // scores are kept in units of log 2: softmax weights are then bare exp2
-  const float scale2 = scale * 1.4426950408889634f;
 
   v4u qf[CB][KS];
   int my_pos[CB];
@@ -703,38 +753,8 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
       for (int i = 0; i < 16; ++i) o[cb][d][i] = 0.f;
   }
 
-  // what this lane fetches in each of its loads of a turn
-  //  K load g: LDS rows K_ROWS g .. + K_ROWS - 1; lane i -> row r = K_ROWS g + i / NP, slot c = i % NP,
-  //            holds piece c ^ (r & (NP - 1)) of key 16 (r / 16) + swap23(r % 16)
-  //  V load g: dims 16 g .. 16 g + 15, 64 bytes each; lane i -> dim d = 16 g + i / 4, slot c = i % 4,
-  //            holds piece c ^ ((d >> 2) & 3): keys 16 (piece / 2) + 8 (piece % 2) .. + 7
-  // packed per load: (element offset inside the page, without the row of the block's first
-  // key) * 2 + (which 16-key block of the turn).  Loads j < MY_K are K loads.
-  int ld_desc[MY_LOADS];
-#pragma unroll
-  for (int j = 0; j < MY_LOADS; ++j) {
-    if (j < MY_K) {
-      const int g = wave + NW * j;
-      const int r = K_ROWS * g + lane / NP, c = lane % NP;
-      const int r16 = r & 15;
-      const int key16 = ((r16 & 4) << 1) | ((r16 & 8) >> 1) | (r16 & 3);
-      ld_desc[j] = (key16 * HD + (c ^ (r & (NP - 1))) * 8) * 2 + (r >> 4);
-    } else {
-      const int gv = wave + NW * (j - MY_K);
-      const int d = 16 * gv + (lane >> 2), c = lane & 3;
-      const int piece = c ^ ((d >> 2) & 3);
-      ld_desc[j] = (d * P + (piece & 1) * 8) * 2 + (piece >> 1);
-    }
-  }
-
-  const unsigned lds0 = (unsigned)(size_t)smem + grp * (PF_STAGES * STAGE);   // this group's stages
-  // LDS addresses of this lane's fragments (without stage and k-step)
-  const unsigned k_row = lds0 + r32 * (HD * 2);                     // K row r32
-  const unsigned v_row = lds0 + K_BYTES + r32 * 64;                 // V^T row (dim) r32 of a 32-dim block
-
   const int blk_lo = (g_lo / PF_KEYS) * 2, blk_hi = g_pos_last / 16;   // 16-key blocks, starting on a turn
   const int v_limit = min(kv_last, blk_hi * 16 + 15);               // last key whose value row is real
-  int turn_count = 0;                                               // turns so far: picks the stage
   for (int c0 = blk_lo; c0 <= blk_hi; c0 += 64) {
     const int nblk = min(64, blk_hi + 1 - c0);
     const int n_turns = (nblk + 1) / 2;
@@ -746,7 +766,7 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     const int n_iter = (n_turns + NG - 1) / NG;                      // the first group's count: the most
     auto issue = [&](int i) {
       const int t = i * NG + grp;
-      const unsigned stage = lds0 + ((turn_count + i) % PF_STAGES) * STAGE;
+      const unsigned stage = lds0 + ((turn_count + i) % ST) * STAGE;
       const int pa = __builtin_amdgcn_readlane(ids, min(2 * t, 63));
       const int pb = __builtin_amdgcn_readlane(ids, min(2 * t + 1, 63));
       const int key0 = (c0 + 2 * t) * 16;
@@ -772,21 +792,21 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                                          (__attribute__((address_space(3))) void*)(size_t)(stage + dst), 16, 0, 0);
       }
     };
-    constexpr int AHEAD = PF_STAGES - 1;
+    constexpr int AHEAD = ST - 1;
 #pragma unroll
     for (int i = 0; i < AHEAD; ++i)
       if (i < my_turns) issue(i);
     for (int i = 0; i < n_iter; ++i) {
       // this group's turn i has landed: only its turns issued after it (at most AHEAD - 1) may be
       // outstanding.  Both groups pass the barrier together, also the one that has run out of turns.
-      vm_wait_turns<MY_LOADS>(max(0, min(AHEAD - 1, my_turns - 1 - i)));
+      vm_wait_turns<MY_LOADS, ST>(max(0, min(AHEAD - 1, my_turns - 1 - i)));
       __builtin_amdgcn_s_barrier();
       if (i + AHEAD < my_turns) issue(i + AHEAD);                  // into the stage that turn i - 1 has left
       if (i >= my_turns) continue;
       const int key0 = (c0 + 2 * (i * NG + grp)) * 16;
       // nothing of this turn is visible to this wavefront: it only helps loading
       if (w_rows == 0 || key0 > w_pos_last || key0 + PF_KEYS - 1 < w_lo) continue;
-      const unsigned st = ((turn_count + i) % PF_STAGES) * STAGE;
+      const unsigned st = ((turn_count + i) % ST) * STAGE;
 
       // ---- the fragments of both tiles: keys now, values right behind them
       v4u kf[KS];
@@ -909,12 +929,13 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     __builtin_amdgcn_s_barrier();
   }
 
-  if constexpr (NG == 2) {
-    // The second group hands its maxima, sums and outputs to the first through LDS (the stages are
-    // free now): lane for lane, the two hold the same columns and dims.
+  if constexpr (NG > 1) {
+    // The other groups hand their maxima, sums and outputs to the first through LDS (the stages
+    // are free now): lane for lane, all hold the same columns and dims.
     constexpr int NVAL = DB * 16 + 2;
-    float* xm = reinterpret_cast<float*>(smem) + (size_t)wave * NVAL * 64 + lane;
-    if (grp == 1) {
+    static_assert((NG - 1) * NW * NVAL * 64 * 4 <= NG * ST * STAGE, "the partial results fit into the stages");
+    if (grp > 0) {
+      float* xm = reinterpret_cast<float*>(smem) + (size_t)((grp - 1) * NW + wave) * NVAL * 64 + lane;
 #pragma unroll
       for (int d = 0; d < DB; ++d)
 #pragma unroll
@@ -923,35 +944,46 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
       xm[(DB * 16 + 1) * 64] = l[0];
     }
     __syncthreads();
-    if (grp == 1) return;
-    const float m1 = xm[(DB * 16) * 64], l1 = xm[(DB * 16 + 1) * 64];
-    const float m_new = fmaxf(mx[0], m1);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    const float a0 = __builtin_amdgcn_exp2f(mx[0] - m_safe), a1 = __builtin_amdgcn_exp2f(m1 - m_safe);
-    l[0] = l[0] * a0 + l1 * a1;
+    if (grp == 0) {
 #pragma unroll
-    for (int d = 0; d < DB; ++d)
+      for (int g = 1; g < NG; ++g) {
+        const float* xm = reinterpret_cast<const float*>(smem) + (size_t)((g - 1) * NW + wave) * NVAL * 64 + lane;
+        const float m1 = xm[(DB * 16) * 64], l1 = xm[(DB * 16 + 1) * 64];
+        const float m_new = fmaxf(mx[0], m1);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float a0 = __builtin_amdgcn_exp2f(mx[0] - m_safe), a1 = __builtin_amdgcn_exp2f(m1 - m_safe);
+        l[0] = l[0] * a0 + l1 * a1;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) o[0][d][i] = o[0][d][i] * a0 + xm[(d * 16 + i) * 64] * a1;
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[0][d][i] = o[0][d][i] * a0 + xm[(d * 16 + i) * 64] * a1;
+        mx[0] = m_new;
+      }
+    }
   }
 
   // o[cb][d][i]: dim 32 d + 8 (i / 4) + 4 h + i % 4 of token (column) r32 of block cb
+  if (grp == 0) {
 #pragma unroll
-  for (int cb = 0; cb < CB; ++cb) {
-    const float lt = l[cb] + __shfl_xor(l[cb], 32, 64);
-    if (!col_ok[cb]) continue;
-    const float inv = 1.0f / lt;
-    const int row = w_first + cb * 32 + r32;
-    bf16_t* dst = out + ((size_t)row * n_head + head) * HD;
+    for (int cb = 0; cb < CB; ++cb) {
+      const float lt = l[cb] + __shfl_xor(l[cb], 32, 64);
+      if (!col_ok[cb]) continue;
+      const float inv = 1.0f / lt;
+      const int row = w_first + cb * 32 + r32;
+      bf16_t* dst = out + ((size_t)row * n_head + head) * HD;
 #pragma unroll
-    for (int d = 0; d < DB; ++d)
+      for (int d = 0; d < DB; ++d)
 #pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const uint2 r = make_uint2(pack_bf16x2(o[cb][d][4 * g4] * inv, o[cb][d][4 * g4 + 1] * inv),
-                                   pack_bf16x2(o[cb][d][4 * g4 + 2] * inv, o[cb][d][4 * g4 + 3] * inv));
-        *reinterpret_cast<uint2*>(dst + 32 * d + 8 * g4 + 4 * h) = r;
-      }
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const uint2 r = make_uint2(pack_bf16x2(o[cb][d][4 * g4] * inv, o[cb][d][4 * g4 + 1] * inv),
+                                     pack_bf16x2(o[cb][d][4 * g4 + 2] * inv, o[cb][d][4 * g4 + 3] * inv));
+          *reinterpret_cast<uint2*>(dst + 32 * d + 8 * g4 + 4 * h) = r;
+        }
+    }
   }
+  // the next tile's loads go into the LDS that the merge has just read
+  if (PAIRED && NG > 1) __syncthreads();
+  }   // slot
 }
 
 // ------------------------------------------------------------------ dispatch
@@ -1096,8 +1128,9 @@ extern "C" int ti_attention_prefill_bf16(const void* q, const void* pool, const 
     }
 #define TI_PLDS(H, G)                                                                                          \
   attn_prefill_lds_kernel<H, G><<<grid, 256 * G, lds, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,   \
-                                                                table_stride, tiles, entries, (bf16_t*)out,     \
-                                                                n_head, n_kv, page_size, scale, window)
+                                                                table_stride, tiles, n_tiles, entries,          \
+                                                                (bf16_t*)out, n_head, n_kv, page_size, scale,   \
+                                                                window)
     if (hd == 128 && groups == 2) TI_PLDS(128, 2);
     else if (hd == 128) TI_PLDS(128, 1);
     else if (groups == 2) TI_PLDS(64, 2);
@@ -1116,6 +1149,49 @@ extern "C" int ti_attention_prefill_bf16(const void* q, const void* pool, const 
     TI_PRE(32) TI_PRE(64) TI_PRE(128)
   }
 #undef TI_PRE
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// The same for launches of few tiles, with the work evened out under a causal mask.  tiles: int
+// [n_tiles, 2] = (entry, first row) of tiles of 64 rows, ordered from the tile that sees the most
+// keys to the one that sees the fewest; a workgroup takes tile b and tile n_tiles - 1 - b, one
+// after the other, with four groups of two wavefronts taking the turns of keys in rotation.
+// Returns 3 for head sizes other than 64 and 128.
+extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool, const int* table, int table_stride,
+                                                const int* tiles, const int* entries, void* out, int n_tiles,
+                                                int n_head, int n_kv, int hd, int page_size, float scale,
+                                                int window, hipStream_t stream) {
+  int rc = check_common("attention_prefill_paired", n_head, n_kv, hd, page_size, table_stride);
+  if (rc) return rc;
+  if (hd == 32) {
+    ti_set_error("attention_prefill_paired: head_dim 32 is not served (64, 128)");
+    return 3;
+  }
+  TI_REQUIRE(n_head <= 65535, "attention_prefill_paired: too many heads");
+  if (n_tiles == 0) return 0;
+  constexpr int NG = 4, NW = 2, ST = 2;
+  const int lds = NG * ST * 2 * PF_KEYS * hd * 2;
+  static bool ready = false;          // allow more than 64 KiB of dynamic LDS, once
+  if (!ready) {
+    if (hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<128, NG, NW, ST, true>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, NG * ST * 2 * PF_KEYS * 128 * 2) != hipSuccess ||
+        hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<64, NG, NW, ST, true>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, NG * ST * 2 * PF_KEYS * 64 * 2) != hipSuccess) {
+      ti_set_error("attention_prefill_paired: cannot reserve the LDS");
+      return 2;
+    }
+    ready = true;
+  }
+  dim3 grid((n_tiles + 1) / 2, n_head);
+  if (hd == 128)
+    attn_prefill_lds_kernel<128, NG, NW, ST, true><<<grid, 64 * NW * NG, lds, stream>>>(
+        (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, n_tiles, entries, (bf16_t*)out, n_head,
+        n_kv, page_size, scale, window);
+  else
+    attn_prefill_lds_kernel<64, NG, NW, ST, true><<<grid, 64 * NW * NG, lds, stream>>>(
+        (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, n_tiles, entries, (bf16_t*)out, n_head,
+        n_kv, page_size, scale, window);
   TI_LAUNCH_CHECK();
   return 0;
 }

@@ -85,6 +85,11 @@ int ti_attention_decode_prepared_bf16(const float* qkv, int row_width, const flo
 int ti_attention_prefill_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* tiles,
                               const int* entries, void* out, int n_tiles, int n_head, int n_kv, int hd, int page_size,
                               float scale, int window, hipStream_t stream);
+// the same for launches of few tiles (head sizes 64, 128): tiles of 64 rows ordered from the most visible
+// keys to the fewest; a workgroup takes tile b and tile n_tiles - 1 - b, so that all have about the same work
+int ti_attention_prefill_paired_bf16(const void* q, const void* pool, const int* table, int table_stride,
+                                     const int* tiles, const int* entries, void* out, int n_tiles, int n_head,
+                                     int n_kv, int hd, int page_size, float scale, int window, hipStream_t stream);
 void ti_attention_prefill_groups(int groups);  // 1 or 2 groups of wavefronts per workgroup, 0: by the launch
 void ti_attention_prefill_use_lds(int on);     // 0: the kernel without LDS for every head size
 

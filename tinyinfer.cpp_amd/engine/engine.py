@@ -26,6 +26,7 @@ from ..ops.kernels import get_ops
 from ..weights.loader import DTYPES
 
 PREFILL_TILE_Q = 128    # query rows per work item of the tiled attention kernels
+PREFILL_TILE_SMALL = 64  # and of the kernel that pairs a tile of many keys with one of few
 
 
 class EngineError(RuntimeError):
@@ -68,6 +69,8 @@ class StepContext:
         self.entry_meta = None
         self.tiles = None                 # int32 [n_tiles, 2]: (entry, first row) of each query tile
         self.n_tiles = 0
+        self.tiles_small = None           # the same in tiles of PREFILL_TILE_SMALL rows, from the tile whose
+        self.n_tiles_small = 0            # last row sees the most keys to the one that sees the fewest
         self.decode_only = False
         self.decode_rows = None           # int32: rows of single-token entries (None if decode_only)
         self.n_decode_rows = 0
@@ -258,16 +261,19 @@ class Engine:
         ctx.M = M
         R = len(entries)
         W = self.table_width
-        # layout: tokens | positions | slots | out_rows | entries [R,4] | tiles [n_tiles,2] | decode rows | tables
+        # layout: tokens | positions | slots | out_rows | entries [R,4] | tiles [n_tiles,2] |
+        #         small tiles [n_small,2] | decode rows | tables
         n_tiles = sum(-(-len(e.tokens) // PREFILL_TILE_Q) for e in entries if len(e.tokens) > 1)
+        n_small = sum(-(-len(e.tokens) // PREFILL_TILE_SMALL) for e in entries if len(e.tokens) > 1)
         ctx.decode_only = n_tiles == 0
         n_dec = 0 if ctx.decode_only else sum(1 for e in entries if len(e.tokens) == 1)
-        ctx.n_tiles, ctx.n_decode_rows = n_tiles, n_dec
+        ctx.n_tiles, ctx.n_tiles_small, ctx.n_decode_rows = n_tiles, n_small, n_dec
         o_tok, o_pos, o_slot = 0, M, 2 * M
         o_out = 3 * M
         o_ent = o_out + n_want
         o_tile = o_ent + 4 * R
-        o_dec = o_tile + 2 * n_tiles
+        o_small = o_tile + 2 * n_tiles
+        o_dec = o_small + 2 * n_small
         o_tab = o_dec + n_dec
         total = o_tab + len(paged) * R * W
         turn, host, dev = self._meta_buffers(total, meta_dev)
@@ -289,6 +295,7 @@ class Engine:
             ctx.max_context = max(starts) + 1
         else:
             tiles: List[int] = []         # (entry, first row) pairs, flat
+            small: List[Tuple[int, int, int]] = []   # (last position, entry, first row)
             dec_rows: List[int] = []
             row0 = 0
             for i, e in enumerate(entries):
@@ -304,6 +311,8 @@ class Engine:
                     for q0 in range(0, n, PREFILL_TILE_Q):
                         tiles.append(i)
                         tiles.append(row0 + q0)
+                    for q0 in range(0, n, PREFILL_TILE_SMALL):
+                        small.append((start + min(q0 + PREFILL_TILE_SMALL, n) - 1, i, row0 + q0))
                 else:
                     h[o_pos + row0] = start
                     dec_rows.append(row0)
@@ -312,7 +321,8 @@ class Engine:
                 if start + n > ctx.max_context:
                     ctx.max_context = start + n
                 row0 += n
-            h[o_tile:o_tab] = tiles + dec_rows
+            small.sort(key=lambda t: -t[0])
+            h[o_tile:o_tab] = tiles + [v for t in small for v in t[1:]] + dec_rows
         ctx.split_context = ctx.max_context
         h[o_out:o_tile] = out_rows + ent_flat
         for k, (gi, g) in enumerate(paged):
@@ -331,6 +341,7 @@ class Engine:
         ctx.out_rows = dev[o_out:o_out + n_want] if n_want else None
         ctx.entry_meta = dev[o_ent:o_ent + 4 * R].view(R, 4)
         ctx.tiles = dev[o_tile:o_tile + 2 * n_tiles].view(-1, 2) if n_tiles else None
+        ctx.tiles_small = dev[o_small:o_small + 2 * n_small].view(-1, 2) if n_small else None
         ctx.decode_rows = dev[o_dec:o_dec + n_dec] if n_dec else None
         for k, (gi, g) in enumerate(paged):
             base = o_tab + k * R * W

@@ -28,6 +28,8 @@ def _ptr(t):
 
 
 PREPARED_HEAD_DIMS = (64, 128)   # head sizes whose queries the decode kernel prepares itself
+PAIRED_HEAD_DIMS = (64, 128)     # head sizes of the prefill kernel that pairs tiles
+PAIRED_BELOW = 512               # (tiles of 128 rows) x heads below which a launch takes that kernel
 
 
 def run_decode_prepared(ops, ctx, view, qkv, q_w, k_w, eps, inv_freq, rope_table, pool, write_kv, out,
@@ -83,7 +85,17 @@ def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) 
         if rc == 3:
             return False
         ops._check(lib, rc, "attention(decode)")
-    if ctx.n_tiles:
+    if ctx.n_tiles and head_dim in PAIRED_HEAD_DIMS and ctx.n_tiles * heads < PAIRED_BELOW \
+            and getattr(ctx, "tiles_small", None) is not None and ops.use_paired_prefill:
+        # few tiles: under a causal mask they differ much in work, and a launch lasts as long as its
+        # heaviest workgroup; the paired kernel gives every workgroup a heavy and a light tile
+        rc = lib.ti_attention_prefill_paired_bf16(
+            _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.tiles_small), _ptr(ctx.entry_meta), _ptr(out),
+            ctx.n_tiles_small, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, stream)
+        if rc == 3:
+            return False
+        ops._check(lib, rc, "attention(prefill, paired)")
+    elif ctx.n_tiles:
         rc = lib.ti_attention_prefill_bf16(
             _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.tiles), _ptr(ctx.entry_meta), _ptr(out),
             ctx.n_tiles, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, stream)

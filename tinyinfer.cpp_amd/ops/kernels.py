@@ -67,6 +67,7 @@ class Ops:
         self.use_fused_norm = True       # the norm before a product inside the product's kernel (few tokens)
         self.use_fused_qk_decode = True  # per-head norm, rotation and cache write inside the decode attention
         self.use_fused_qkv_prefill = True  # the same in the epilogue of the q/k/v product (steps of many tokens)
+        self.use_paired_prefill = True   # small prefill launches: a heavy and a light tile per workgroup
 
     # ------------------------------------------------------------------ loading
     def lib(self, name: str) -> ctypes.CDLL:

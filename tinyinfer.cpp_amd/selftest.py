@@ -58,6 +58,9 @@ class _Ctx:
         self.decode_rows, self.n_decode_rows = None, 0
         self.n_tiles = -(-M // 128) if one_portion else 0
         self.tiles = _dev(np.array([[0, 128 * i] for i in range(self.n_tiles)], dtype=np.int32)) if one_portion else None
+        self.n_tiles_small = -(-M // 64) if one_portion else 0     # from the most keys to the fewest
+        self.tiles_small = _dev(np.array([[0, 64 * i] for i in reversed(range(self.n_tiles_small))],
+                                         dtype=np.int32)) if one_portion else None
         self.entry_meta = _dev(np.array([[0, M, positions[0], 0]], dtype=np.int32))
         self.max_context = self.split_context = int(max(positions)) + 1
 
