@@ -32,6 +32,32 @@ def test_pages_are_taken_in_order_and_reused_lifo():
     m.check()
 
 
+def test_pages_scattered_within_windows_are_a_permutation():
+    """With a scatter window every page is still handed out exactly once, each from the window
+    that is due, in an order that is not 0, 1, 2, ...; released pages come back LIFO as before."""
+    from tinyinfer_amd.cache.manager import PagePool
+    pool = PagePool(70, scatter_window=16)
+    taken = [pool.take() for _ in range(70)]
+    assert sorted(taken) == list(range(70))
+    for i in range(0, 70, 16):
+        assert sorted(taken[i:i + 16]) == list(range(i, min(i + 16, 70)))
+    assert taken != list(range(70))
+    assert PagePool(70, scatter_window=16)._free == PagePool(70, scatter_window=16)._free   # a fixed order
+    with pytest.raises(OutOfPages):
+        pool.take()
+    pool.give_back(taken[3])
+    pool.give_back(taken[40])
+    assert pool.take() == taken[40] and pool.take() == taken[3]
+    m = CacheManager([(FULL, 1)], page_size=4, num_pages=64, max_requests=2, max_seq=128, scatter_window=8)
+    m.admit("a")
+    m.reserve("a", 100)
+    m.commit("a", 100)
+    m.check()
+    m.release("a")
+    m.check()
+    assert m.num_free_pages() == 64
+
+
 def test_reserve_is_all_or_nothing():
     m = manager(pages=3)
     m.admit("a")

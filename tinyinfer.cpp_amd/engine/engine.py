@@ -27,6 +27,7 @@ from ..weights.loader import DTYPES
 
 PREFILL_TILE_Q = 128    # query rows per work item of the tiled attention kernels
 PREFILL_TILE_SMALL = 64  # and of the kernel that pairs a tile of many keys with one of few
+PAGE_SCATTER_WINDOW = 512  # free pages are first handed out shuffled within windows of this many (see PagePool)
 
 
 class EngineError(RuntimeError):
@@ -120,7 +121,8 @@ class Engine:
             if model.spec.max_position_embeddings:
                 max_seq = min(max_seq, model.spec.max_position_embeddings)
         self.max_seq = int(max_seq)
-        self.cache = CacheManager(model.cache_groups, self.page_size, self.num_pages, max_requests, self.max_seq)
+        self.cache = CacheManager(model.cache_groups, self.page_size, self.num_pages, max_requests, self.max_seq,
+                                  scatter_window=PAGE_SCATTER_WINDOW)
         self.storage = CacheStorage(self.cache, self.act_dtype, self.device)
         self.table_width = self.cache.max_pages_per_request
         for part in model.parts():
