@@ -495,7 +495,9 @@ def test_linear_bf16_every_tile(ops, tile, M, N, K):
 
 
 def test_linear_bf16_rows_do_not_depend_on_the_batch(ops):
-    """Within one kernel a row's bits do not depend on the other rows."""
+    """Within one family of kernels a row's bits do not depend on the other rows: the tiled
+    kernels (more than 64 rows), the kernels whose workgroups own 16 weight rows (9 to 64 rows
+    here), and the kernel with a weight row per wavefront (up to 8 rows, a weight of few rows)."""
     if not ops.use_fast_gemm:
         pytest.skip("bfloat16 MFMA kernels are switched off")
     g = torch.Generator().manual_seed(4)
@@ -507,17 +509,25 @@ def test_linear_bf16_rows_do_not_depend_on_the_batch(ops):
     ops.linear(dev(a[100:170].contiguous()), dev(w), part, "store")     # tiled, other rows
     assert torch.equal(part, full[100:170])
     small = torch.empty(40, 150, device="cuda")
-    ops.linear(dev(a[:40].contiguous()), dev(w), small, "store")        # skinny
-    one = torch.empty(1, 150, device="cuda")
-    for m in (0, 17, 39):
-        ops.linear(dev(a[m:m + 1].contiguous()), dev(w), one, "store")  # skinny, alone
-        assert torch.equal(one[0], small[m])
+    ops.linear(dev(a[:40].contiguous()), dev(w), small, "store")        # 16 weight rows a workgroup, 3 token tiles
+    for lo, hi in ((0, 9), (17, 33), (24, 40)):
+        some = torch.empty(hi - lo, 150, device="cuda")
+        ops.linear(dev(a[lo:hi].contiguous()), dev(w), some, "store")   # the same family, fewer rows
+        assert torch.equal(some, small[lo:hi])
+    few = torch.empty(8, 150, device="cuda")
+    ops.linear(dev(a[:8].contiguous()), dev(w), few, "store")           # a weight row per wavefront
+    for lo, hi in ((0, 1), (3, 4), (2, 4), (4, 8), (7, 8)):
+        some = torch.empty(hi - lo, 150, device="cuda")
+        ops.linear(dev(a[lo:hi].contiguous()), dev(w), some, "store")
+        assert torch.equal(some, few[lo:hi])
+    assert (f64(few) - f64(small[:8])).abs().max() < 2e-5 * 264         # the families agree up to rounding
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 48, 1024), (7, 1000, 1096), (40, 130, 2048), (64, 2048, 1032)])
 def test_linear_bf16_few_columns_many_wavefronts(ops, M, N, K):
-    """Few output columns and a long K: the skinny kernel runs with eight wavefronts
-    that split K.  Same result as float64, and a row alone has the bits it has in a batch."""
+    """Few output columns and a long K: up to 8 rows take the kernel with a weight row per
+    wavefront, more rows the kernel with eight wavefronts that split K.  Same result as float64,
+    and a row has the bits it has in a larger batch of the same family."""
     if not ops.use_fast_gemm:
         pytest.skip("bfloat16 MFMA kernels are switched off")
     g = torch.Generator().manual_seed(M + N)
@@ -530,17 +540,19 @@ def test_linear_bf16_few_columns_many_wavefronts(ops, M, N, K):
     assert (f64(out) - (ref + f64(base))).abs().max() < 2e-5 * K
     full = torch.empty(M, N, device="cuda")
     ops.linear(dev(a), dev(w), full, "store")
-    one = torch.empty(1, N, device="cuda")
-    m = M - 1
-    ops.linear(dev(a[m:m + 1].contiguous()), dev(w), one, "store")
-    assert torch.equal(one[0], full[m])
+    k = 1 if M <= 8 else 9                       # fewer rows of the same family of kernels
+    some = torch.empty(k, N, device="cuda")
+    ops.linear(dev(a[M - k:].contiguous()), dev(w), some, "store")
+    assert torch.equal(some, full[M - k:])
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 48, 64), (5, 261, 1024), (16, 40, 192), (3, 130, 1280), (8, 64, 2304),
-                                   (2, 18, 4096)])
+@pytest.mark.parametrize("M,N,K", [(1, 4100, 64), (5, 4096, 1024), (16, 40, 192), (9, 130, 1280), (12, 64, 2304),
+                                   (2, 4112, 4096), (8, 6144, 1024)])
 def test_linear_with_the_norm_inside(ops, M, N, K):
     """rmsnorm and product in one kernel (few tokens) give the bits of the norm kernel
-    followed by the product kernel, for every epilogue; and both agree with float64."""
+    followed by the product kernel, for every epilogue; and both agree with float64.  (Up to 8
+    tokens and a weight of fewer than 4,096 rows are left to the kernel with a weight row per
+    wavefront, except for SwiGLU: see the next test.)"""
     from tinyinfer_amd.ops.kernels import NormedRows
     if not ops.use_fast_gemm:
         pytest.skip("bfloat16 MFMA kernels are switched off")
@@ -572,13 +584,14 @@ def test_linear_with_the_norm_inside(ops, M, N, K):
 
 
 def test_linear_with_the_norm_inside_refuses_what_it_does_not_serve(ops):
-    """More rows than the kernel holds, or a K that is no multiple of 64: `linear` computes
-    the norm first and the result is still right."""
+    """More rows than the kernel holds, a K that is no multiple of 64, or few tokens with a weight
+    of few rows (which another kernel takes): `linear` computes the norm first and the result
+    is that of the norm kernel followed by the product."""
     from tinyinfer_amd.ops.kernels import NormedRows
     if not ops.use_fast_gemm:
         pytest.skip("bfloat16 MFMA kernels are switched off")
     g = torch.Generator().manual_seed(9)
-    for M, N, K in ((17, 32, 128), (4, 32, 72)):
+    for M, N, K in ((17, 32, 128), (4, 32, 72), (4, 32, 128), (8, 1024, 2048)):
         x = dev(torch.randn(M, K, generator=g))
         nw = dev(1 + 0.1 * torch.randn(K, generator=g))
         w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))

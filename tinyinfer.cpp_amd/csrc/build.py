@@ -24,8 +24,11 @@ from typing import Dict, Iterable, List
 HERE = os.path.dirname(os.path.abspath(__file__))
 ARCH = "gfx950"
 # packed 32-bit float instructions are switched off for every kernel
+# and the first kernel arguments arrive in scalar registers with the wavefront (the command
+# processor preloads them) instead of being fetched by the kernel's first instructions
 FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-shared",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-mllvm", "-amdgpu-kernarg-preload-count=16",
          "-Wno-unused-command-line-argument"]
 HEADERS = ["common.h", "qk_prep.h", "tinyinfer_kernels.h"]
 # flags of single libraries.  The attention kernels rescale their MFMA accumulators with

@@ -226,7 +226,46 @@ struct NormProducer {
   }
 };
 
-template <class Producer, int EPI, int NW>
+// Rows that do exist in memory (bfloat16 [M, K], row stride lda): copied into LDS once per
+// workgroup, 16 bytes per thread and load, instead of every wavefront fetching its token
+// fragments from memory with one load instruction per fragment (for one token fifteen of
+// sixteen lanes of such a load repeat a row): a compute unit takes a load instruction of 64
+// lanes every 16 cycles or so, and the kernel for few tokens is bound by that.
+struct CopyProducer {
+  const bf16_t* A;
+  long lda;
+  template <int NW, class IssueWeights>
+  __device__ __forceinline__ void fill(bf16_t* sA, int lds_stride, int M, int K, IssueWeights issue_weights) const {
+    constexpr int NT = NW * 64, PB = 8;
+    const int kp = K >> 3, pieces = M * kp;
+    bool first = true;
+    for (int p0 = threadIdx.x; first || p0 < pieces; p0 += NT * PB) {
+      uint4 v[PB];
+      int dst[PB];
+      bool ok[PB];
+#pragma unroll
+      for (int b = 0; b < PB; ++b) {
+        const int p = p0 + NT * b;
+        ok[b] = p < pieces;
+        const int pc = ok[b] ? p : 0;
+        const int m = pc / kp, k8 = pc - m * kp;
+        v[b] = ld16(A + (size_t)m * lda + k8 * 8);
+        dst[b] = m * lds_stride + k8 * 8;
+      }
+      if (first) {
+        __builtin_amdgcn_sched_barrier(0);
+        issue_weights();
+        __builtin_amdgcn_sched_barrier(0);
+        first = false;
+      }
+#pragma unroll
+      for (int b = 0; b < PB; ++b)
+        if (ok[b]) *reinterpret_cast<uint4*>(sA + dst[b]) = v[b];
+    }
+  }
+};
+
+template <class Producer, int EPI, int NW, int UN = 4>
 __global__ void __launch_bounds__(NW * 64)
 gemm_skinny_staged_kernel(Producer producer, const bf16_t* __restrict__ W, void* __restrict__ out_, int M, int N,
                           int K) {
@@ -248,7 +287,6 @@ gemm_skinny_staged_kernel(Producer producer, const bf16_t* __restrict__ W, void*
   const bf16_t* wp = W + (size_t)wrow * K + j * 16;
   const uint4 zero = make_uint4(0, 0, 0, 0);
   const int chunks = K / 64;
-  constexpr int UN = 4;
 
   // the residual this thread will add to
   const int tok = threadIdx.x >> 4, row = threadIdx.x & 15;   // tok >= 16 for the wavefronts beyond four
@@ -325,6 +363,104 @@ gemm_skinny_staged_kernel(Producer producer, const bf16_t* __restrict__ W, void*
     if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = sum;
     if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] = prev + sum;
     if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(sum);
+  }
+}
+
+// ================================== few tokens, a weight of few rows: a row per wavefront
+// out (op)= A W^T for M <= MMAX tokens and a weight with so few rows that the kernels above,
+// whose workgroups own 16 rows each, would leave most compute units idle (N = 1024: 64
+// workgroups), while each busy unit would have hundreds of load instructions to get through
+// (a unit takes one 64-lane load every ~25 cycles: measured 2.7 us to issue 256 of them).
+// Here a wavefront owns one weight row: lane l holds the 8-element pieces l, l + 64, ... of
+// it (every load instruction fetches 1 KiB that nobody else fetches), the token rows are
+// copied into LDS once per workgroup, the products are v_dot2c_f32_bf16 (two multiply-adds
+// on packed bfloat16, accumulated in 32-bit), and the lanes' partial sums meet in a
+// butterfly.  N / 4 workgroups of four wavefronts.  A row's bits do not depend on the rows
+// beside it.  K a multiple of 8, up to 512 NL (NL: pieces of the weight row per lane); MMAX: the
+// most tokens.  Both are template parameters so that every load is unconditional and counted.
+#define GR_LOADS 8
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float dot2_bf16(unsigned a, unsigned b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+
+template <int EPI, int MMAX, int NL>
+__global__ void __launch_bounds__(256)
+gemv_rows_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_, int M, int N,
+                 int K, long lda) {
+  static_assert(EPI != TI_EPI_SWIGLU, "no SwiGLU here");
+  extern __shared__ __attribute__((aligned(16))) unsigned char dyn_smem[];
+  bf16_t* sA = reinterpret_cast<bf16_t*>(dyn_smem);          // [M][K]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + wave;
+  const bf16_t* wp = W + (size_t)(n < N ? n : N - 1) * K;
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+
+  // the residual lane m will add to (row m of the tokens): asked for first
+  float prev = 0.f;
+  if (EPI == TI_EPI_ADD_F32) prev = ((const float*)out_)[(size_t)(lane < M ? lane : 0) * N + (n < N ? n : N - 1)];
+  // the token rows (from the cache), 16 bytes per thread and load, all in flight at once; then
+  // this wavefront's weight row (from memory).  Loads come back in the order they were issued.
+  constexpr int PB = (MMAX * NL + 3) / 4;                     // pieces per thread: all of [MMAX][512 NL]
+  const int kp = K >> 3, pieces = M * kp;
+  uint4 av[PB];
+#pragma unroll
+  for (int b = 0; b < PB; ++b) {
+    const int p = threadIdx.x + 256 * b;
+    const int pc = p < pieces ? p : 0;
+    const int m = pc / kp, k8 = pc - m * kp;
+    av[b] = ld16(A + (size_t)m * lda + k8 * 8);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  uint4 wv[NL];
+#pragma unroll
+  for (int i = 0; i < NL; ++i) {
+    const int kk = (i * 64 + lane) * 8;
+    wv[i] = ld16(wp + (kk < K ? kk : 0));
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int b = 0; b < PB; ++b) {
+    const int p = threadIdx.x + 256 * b;
+    if (p < pieces) {
+      const int m = p / kp, k8 = p - m * kp;
+      *reinterpret_cast<uint4*>(sA + (size_t)m * K + k8 * 8) = av[b];
+    }
+  }
+  __syncthreads();
+
+  // rows beyond M repeat row 0 and are dropped: all LDS reads of a piece go out together
+  float acc[MMAX];
+#pragma unroll
+  for (int m = 0; m < MMAX; ++m) acc[m] = 0.f;
+#pragma unroll
+  for (int i = 0; i < NL; ++i) {
+    const int kk = (i * 64 + lane) * 8;
+    const bool ok = kk < K;
+    const uint4 w = ok ? wv[i] : zero;
+    const bf16_t* ap = sA + (ok ? kk : 0);
+    uint4 a[MMAX];
+#pragma unroll
+    for (int m = 0; m < MMAX; ++m) a[m] = *reinterpret_cast<const uint4*>(ap + (size_t)(m < M ? m : 0) * K);
+#pragma unroll
+    for (int m = 0; m < MMAX; ++m) {
+      acc[m] = dot2_bf16(w.x, a[m].x, acc[m]);
+      acc[m] = dot2_bf16(w.y, a[m].y, acc[m]);
+      acc[m] = dot2_bf16(w.z, a[m].z, acc[m]);
+      acc[m] = dot2_bf16(w.w, a[m].w, acc[m]);
+    }
+  }
+  float mine = 0.f;
+#pragma unroll
+  for (int m = 0; m < MMAX; ++m) {
+    const float t = group_sum<TI_WAVE>(acc[m]);
+    if (lane == m) mine = t;
+  }
+  if (lane < M && n < N) {
+    const size_t o = (size_t)lane * N + n;
+    if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = mine;
+    if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] = prev + mine;
+    if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(mine);
   }
 }
 
@@ -902,11 +1038,52 @@ static void launch_tiled(const bf16_t* A, const bf16_t* W, void* out, int M, int
   gemm_tiled_kernel<EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
 }
 
-template <class Producer, int EPI, int NW>
+// 1 (default): up to GR_MMAX tokens and a weight of fewer than GR_ROWS_BELOW rows take the kernel
+// with a weight row per wavefront; 0: they take the kernels whose workgroups own 16 rows
+#define GR_MMAX 8
+#define GR_ROWS_BELOW 4096
+static int g_row_per_wave = 1;
+extern "C" void ti_gemm_bf16_row_per_wave(int on) { g_row_per_wave = on; }
+static bool row_per_wave_serves(int M, int N, int K, int epi) {
+  return g_row_per_wave && M <= GR_MMAX && N < GR_ROWS_BELOW && K % 8 == 0 && K <= 64 * 8 * GR_LOADS &&
+         (epi == TI_EPI_STORE_F32 || epi == TI_EPI_ADD_F32);
+}
+
+template <int EPI, int MMAX, int NL>
+static int launch_rows_mk(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda, hipStream_t s) {
+  const size_t lds = (size_t)M * K * 2;
+  auto kern = gemv_rows_kernel<EPI, MMAX, NL>;
+  static size_t allowed = 48 * 1024;
+  if (lds > allowed) {
+    TI_REQUIRE(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) ==
+                   hipSuccess, "gemm_bf16: LDS size refused");
+    allowed = lds;
+  }
+  kern<<<(N + 3) / 4, 256, lds, s>>>(A, W, out, M, N, K, lda);
+  return 0;
+}
+template <int EPI, int MMAX>
+static int launch_rows_m(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda, hipStream_t s) {
+  if (K <= 1024) return launch_rows_mk<EPI, MMAX, 2>(A, W, out, M, N, K, lda, s);
+  if (K <= 2048) return launch_rows_mk<EPI, MMAX, 4>(A, W, out, M, N, K, lda, s);
+  if (K <= 3072) return launch_rows_mk<EPI, MMAX, 6>(A, W, out, M, N, K, lda, s);
+  return launch_rows_mk<EPI, MMAX, GR_LOADS>(A, W, out, M, N, K, lda, s);
+}
+// the kernel is compiled for 1, 2, 4 and GR_MMAX tokens and four lengths of K; a row's bits are
+// the same in all of them
+template <int EPI>
+static int launch_rows(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda, hipStream_t s) {
+  if (M <= 1) return launch_rows_m<EPI, 1>(A, W, out, M, N, K, lda, s);
+  if (M <= 2) return launch_rows_m<EPI, 2>(A, W, out, M, N, K, lda, s);
+  if (M <= 4) return launch_rows_m<EPI, 4>(A, W, out, M, N, K, lda, s);
+  return launch_rows_m<EPI, GR_MMAX>(A, W, out, M, N, K, lda, s);
+}
+
+template <class Producer, int EPI, int NW, int UN = 4>
 static int launch_staged(const char* what, Producer producer, const bf16_t* w, void* out, int M, int N, int K,
                          int grid, hipStream_t stream) {
   const size_t lds = (size_t)M * (K + 8) * 2;
-  auto kern = gemm_skinny_staged_kernel<Producer, EPI, NW>;
+  auto kern = gemm_skinny_staged_kernel<Producer, EPI, NW, UN>;
   static size_t allowed = 48 * 1024;   // per instantiation: the largest size asked for so far
   if (lds > allowed) {
     TI_REQUIRE(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) ==
@@ -931,6 +1108,12 @@ extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, c
   TI_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16_normed: bad sizes M=%d N=%d K=%d", M, N, K);
   if (M > 16 || K % 64 != 0 || K > 4096 || ((uintptr_t)W & 15) || ((uintptr_t)x & 15) || ((uintptr_t)nw & 15)) {
     ti_set_error("gemm_bf16_normed: M=%d K=%d is not served (M <= 16, K %% 64 == 0, K <= 4096)", M, K);
+    return 3;
+  }
+  if (row_per_wave_serves(M, N, K, epi)) {
+    // the plain product of these sizes takes another kernel, with another order of summation: the
+    // caller norms first and takes that one too, so that the norm in front changes no bit
+    ti_set_error("gemm_bf16_normed: M=%d N=%d is left to the kernel with a weight row per wavefront", M, N);
     return 3;
   }
   if (M == 0) return 0;
@@ -962,6 +1145,26 @@ extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, c
   return 0;
 }
 
+// 1 (default): up to 16 tokens with K a multiple of 64 up to 4096, the token rows are copied into
+// LDS once per workgroup (see CopyProducer); 0: every wavefront fetches its fragments from memory
+static int g_skinny_copy = 1;
+extern "C" void ti_gemm_bf16_skinny_copy(int on) { g_skinny_copy = on; }
+
+template <int EPI>
+static int launch_skinny_copied(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
+                                hipStream_t s) {
+  const int grid = (EPI == TI_EPI_SWIGLU) ? (N + 7) / 8 : (N + 15) / 16;
+  int waves = g_skinny_waves;
+  if (waves == 0) waves = (grid <= 128 && K >= 1024) ? 8 : 4;         // as the plain kernel: same bits
+  const bool deep = K / 64 > 4 * waves && g_skinny_deep;
+  CopyProducer pr{A, lda};
+  if (waves == 8)
+    return deep ? launch_staged<CopyProducer, EPI, 8, 8>("gemm_bf16", pr, W, out, M, N, K, grid, s)
+                : launch_staged<CopyProducer, EPI, 8, 4>("gemm_bf16", pr, W, out, M, N, K, grid, s);
+  return deep ? launch_staged<CopyProducer, EPI, 4, 8>("gemm_bf16", pr, W, out, M, N, K, grid, s)
+              : launch_staged<CopyProducer, EPI, 4, 4>("gemm_bf16", pr, W, out, M, N, K, grid, s);
+}
+
 static int g_use_pipelined = 1;
 // 1: the pipelined tiled kernel for M > 64 (default); 0: the plain tiled kernel (for comparison)
 extern "C" void ti_gemm_bf16_use_pipelined(int on) { g_use_pipelined = on; }
@@ -983,9 +1186,21 @@ extern "C" int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int 
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
   const bool skinny = M <= 64;
+  const bool copied = g_skinny_copy && M <= 16 && K % 64 == 0 && K <= 4096;
+  if (row_per_wave_serves(M, N, K, epi)) {
+    int rc_ = 0;
+    if (epi == TI_EPI_STORE_F32) rc_ = launch_rows<TI_EPI_STORE_F32>(a, w, out, M, N, K, lda, stream);
+    else rc_ = launch_rows<TI_EPI_ADD_F32>(a, w, out, M, N, K, lda, stream);
+    if (rc_) return rc_;
+    TI_LAUNCH_CHECK();
+    return 0;
+  }
 #define TI_GO(E)                                                  \
   case E:                                                         \
-    if (skinny)                                                   \
+    if (copied) {                                                 \
+      int rc_ = launch_skinny_copied<E>(a, w, out, M, N, K, lda, stream); \
+      if (rc_) return rc_;                                        \
+    } else if (skinny)                                            \
       launch_skinny<E>(a, w, out, M, N, K, lda, stream);          \
     else if (g_use_pipelined && K % PBK == 0) {                   \
       int rc_ = launch_tiled_best<E>(a, w, out, M, N, K, lda, stream); \

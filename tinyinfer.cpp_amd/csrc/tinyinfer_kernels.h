@@ -58,6 +58,8 @@ int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K, long lda, 
 void ti_gemm_bf16_force_tile(int which);      // 1: 256 x 128, 3: 128 x 64, 6: 64 x 64
 void ti_gemm_bf16_skinny_waves(int waves);    // 4 or 8 wavefronts in the kernel for M <= 64
 void ti_gemm_bf16_use_pipelined(int on);      // 0: the plain tiled kernel for every K
+void ti_gemm_bf16_row_per_wave(int on);        // 0: few tokens and a weight of few rows take the 16-row kernels too
+void ti_gemm_bf16_skinny_copy(int on);        // 0: up to 16 tokens, fragments of the token rows straight from memory
 void ti_gemm_bf16_skinny_deep(int on);        // 0: four chunks of K in flight per wavefront also for a long K
 
 // ---- libti_attention_generic: paged causal attention of every row, any head size in steps of 16
