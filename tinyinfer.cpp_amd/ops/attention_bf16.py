@@ -12,7 +12,7 @@ import torch
 SERVED_HEAD_DIMS = (32, 64, 128)
 TARGET_WORKGROUPS = 256       # one per compute unit: a unit streams about as fast with 4 wavefronts as with 8
 MAX_SPLITS = 64               # the merge kernel's limit
-MIN_BLOCKS_PER_SPLIT = 8      # two 16-key blocks per wavefront at least
+MIN_BLOCKS_PER_SPLIT = 16     # four 16-key blocks per wavefront at least (fewer, and the merge costs more than the split gains)
 
 
 def decode_splits(n_rows: int, kv_heads: int, heads: int, context: int) -> int:
