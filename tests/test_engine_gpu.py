@@ -238,21 +238,22 @@ def test_prepared_qkv_product_changes_no_bit(model_folders):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_layers_of_real_width_match_plain(model_folders, dtype):
-    """Two layers with the widths of Qwen3-0.6B: a prompt of 300 tokens in portions (one of them
-    beside another request's decoded token), then 24 tokens one by one, against the plain model.
-    These widths take other kernels than the tiny configurations do."""
+    """Two layers with the widths of Qwen3-0.6B: a prompt of 540 tokens in portions (one of them
+    beside another request's decoded token), then 24 tokens one by one (a context long enough for
+    the decode attention to split it over workgroups), against the plain model.  These widths take
+    other kernels than the tiny configurations do."""
     folder = model_folders("E", "bfloat16", True)
     V = CONFIGS["E"]["vocab_size"]
-    requests = {"a": random_tokens(324, V, 31), "b": random_tokens(40, V, 32)}
+    requests = {"a": random_tokens(564, V, 31), "b": random_tokens(40, V, 32)}
     want, tol = plain_logits(folder, requests, dtype)
     a, b = requests["a"], requests["b"]
     trace = [{"entries": [("a", a[:200], [0, 100, 199]), ("b", b[:39], [38])], "end": []},
-             {"entries": [("b", b[39:40], [0]), ("a", a[200:300], list(range(0, 100, 9)))], "end": ["b"]}]
-    trace += [{"entries": [("a", a[i:i + 1], [0])], "end": []} for i in range(300, 324)]
+             {"entries": [("b", b[39:40], [0]), ("a", a[200:540], list(range(0, 340, 31)))], "end": ["b"]}]
+    trace += [{"entries": [("a", a[i:i + 1], [0])], "end": []} for i in range(540, 564)]
     trace[-1]["end"] = ["a"]
-    engine = build_engine(folder, dtype, 512)
+    engine = build_engine(folder, dtype, 704)
     got = replay(engine, trace)
-    rows = {"a": [0, 100, 199] + [200 + i for i in range(0, 100, 9)] + list(range(300, 324)), "b": [38, 39]}
+    rows = {"a": [0, 100, 199] + [200 + i for i in range(0, 340, 31)] + list(range(540, 564)), "b": [38, 39]}
     # The 32-bit bound of the tiny models (2e-5 for logits of order 1) is kept relative to the size
     # of the logits here: sums run over 1,024 to 3,072 terms instead of 64 to 224.
     scale = max(1.0, max(float(np.abs(want[r]).max()) for r in requests))
