@@ -482,6 +482,31 @@ attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ pa
   const float* po = part_o + ((size_t)ridx * n_head + head) * n_splits * HD + d;
   // every thread works the weights of the splits out for itself: they are few, and no thread waits
   // for another
+  if (n_splits <= 8) {
+    // everything asked for at once (splits beyond the last repeat it and count for nothing)
+    float v[8];
+    float2 ml[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int sj = j < n_splits ? j : n_splits - 1;
+      ml[j] = pm[sj];
+      v[j] = po[(size_t)sj * HD];
+    }
+    float mm = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < n_splits) mm = fmaxf(mm, ml[j].x);
+    float acc = 0.f, lt = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < n_splits) {
+        const float w = split_weight(ml[j].x, mm);
+        lt = fmaf(ml[j].y, w, lt);
+        acc = split_accumulate(acc, v[j], w);
+      }
+    out[((size_t)m_row * n_head + head) * HD + d] = f2bf(acc * (1.0f / lt));
+    return;
+  }
   float mm = -INFINITY;
   for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, pm[s].x);
   float acc = 0.f, lt = 0.f;
