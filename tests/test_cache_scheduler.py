@@ -125,6 +125,61 @@ def test_state_slots_are_cleared_on_admission():
     assert [i for i, _ in m.state_groups()] == [1]
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_decode_steps_reserved_in_one_call_match_the_calls_per_request(seed):
+    """`reserve_one_each` / `commit_one_each` leave the manager in the state that `reserve` and
+    `commit` per request leave it in (tables, free pages, lengths), with a window group giving
+    pages back, and take nothing when the pages do not suffice."""
+    rng = random.Random(seed)
+    a = manager(groups=((FULL, 2), (WIN, 1)), page_size=4, pages=30, slots=6, max_seq=80)
+    b = manager(groups=((FULL, 2), (WIN, 1)), page_size=4, pages=30, slots=6, max_seq=80)
+    live = []
+    for n in range(5):
+        k = rng.choice([1, 3, 4, 9, 17])
+        for m in (a, b):
+            m.admit(n)
+            m.reserve(n, k)
+            m.commit(n, k)
+        live.append(n)
+    for _ in range(70):
+        some = [q for q in live if rng.random() < 0.7]
+        if not some:
+            continue
+        if any(a.length(q) + 1 > 80 for q in some):
+            with pytest.raises(CacheError):
+                a.reserve_one_each(some)
+            for q in [q for q in some if a.length(q) + 1 > 80]:
+                a.release(q)
+                b.release(q)
+                live.remove(q)
+            continue
+        try:
+            starts = a.reserve_one_each(some)
+        except OutOfPages:
+            free = a.num_free_pages()
+            a.check()
+            assert a.num_free_pages() == free
+            q = rng.choice(live)                      # make room in both and go on
+            a.release(q)
+            b.release(q)
+            live.remove(q)
+            continue
+        assert starts == [b.length(q) for q in some]
+        for q in some:
+            b.reserve(q, 1)
+        a.commit_one_each(some)
+        for q in some:
+            b.commit(q, 1)
+        a.check()
+        b.check()
+        for gi in (0, 1):
+            for q in live:
+                assert a.table(gi, q) == b.table(gi, q), (gi, q)
+        assert a.num_free_pages() == b.num_free_pages()
+    with pytest.raises(CacheError):
+        a.reserve_one_each(["nobody"])
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_random_orders_lose_no_page(seed):
     """Admissions, portions, decoding, ends and failed reservations in random order:

@@ -269,6 +269,57 @@ class CacheManager:
                 if t[i] >= 0:
                     g.give_back_page(req, i)
 
+    # ---- a decode step: one token for each of several admitted requests.  The same as `reserve`
+    # (for all of them or for none) and `commit` per request, without their per-request overhead.
+    def reserve_one_each(self, reqs: Sequence[Hashable]) -> List[int]:
+        """Make one more position writable for every request of `reqs` (all admitted, each
+        once), or raise OutOfPages and take nothing.  Returns their lengths (the positions
+        the new tokens take)."""
+        try:
+            rs = [self._requests[q] for q in reqs]
+        except KeyError as e:
+            raise CacheError(f"request {e.args[0]!r} is not admitted") from None
+        P = self.page_size
+        starts = []
+        for r, q in zip(rs, reqs):
+            if r.reserved != r.length:
+                raise CacheError(f"request {q!r} has a reservation that was not committed")
+            if r.reserved + 1 > self.max_seq:
+                raise CacheError(f"request {q!r}: {r.reserved + 1} tokens exceed max_seq = {self.max_seq}")
+            starts.append(r.length)
+        todo = []
+        for _, g in self._paged:
+            tables = g.tables
+            short = [q for r, q in zip(rs, reqs) if len(tables[q]) * P <= r.reserved]
+            if len(short) > g.pool.num_free:
+                raise OutOfPages(f"the step needs {len(short)} new pages, {g.pool.num_free} are free")
+            if short:
+                todo.append((g, short))
+        for g, short in todo:
+            for q in short:
+                g.append_page(q)
+        for r in rs:
+            r.reserved += 1
+        return starts
+
+    def commit_one_each(self, reqs: Sequence[Hashable]) -> None:
+        """The step wrote one more token of every request of `reqs` (see `commit`)."""
+        P = self.page_size
+        windowed = [g for _, g in self._paged if g.need.window is not None]
+        for q in reqs:
+            r = self._requests[q]
+            if r.length + 1 > r.reserved:
+                raise CacheError(f"request {q!r}: committing a token beyond its reservation")
+            r.length += 1
+            for g in windowed:
+                # a page falls behind the window only when the window's first position enters a new page
+                lo = r.length - g.need.window + 1
+                if lo > 0 and lo % P == 0:
+                    t = g.tables[q]
+                    for i in range(min(lo // P, len(t))):
+                        if t[i] >= 0:
+                            g.give_back_page(q, i)
+
     def release(self, req: Hashable) -> None:
         """The request is over (finished, aborted or preempted): every page and
         its slot go back."""

@@ -20,7 +20,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..cache import CacheManager, CacheStorage, OutOfPages, PagedGroup
+from ..cache import CacheError, CacheManager, CacheStorage, OutOfPages, PagedGroup
 from ..models.model import Model
 from ..ops.kernels import get_ops
 from ..weights.loader import DTYPES
@@ -70,6 +70,7 @@ class StepContext:
         self.entry_meta = None
         self.tiles = None                 # int32 [n_tiles, 2]: (entry, first row) of each query tile
         self.n_tiles = 0
+        self._decode_fast = False         # the step was reserved by CacheManager.reserve_one_each
         self.tiles_small = None           # the same in tiles of PREFILL_TILE_SMALL rows, from the tile whose
         self.n_tiles_small = 0            # last row sees the most keys to the one that sees the fewest
         self.decode_only = False
@@ -216,10 +217,11 @@ class Engine:
             raise EngineError("a step needs at least one entry")
         V = self.model.vocab_size
         cache = self.cache
+        starts_fast = self._reserve_decode_step(entries)
         seen = set()
         M = 0
         n_want = 0
-        for e in entries:
+        for e in (entries if starts_fast is None else ()):
             toks = e.tokens
             n = len(toks)
             if e.request in seen:
@@ -236,12 +238,15 @@ class Engine:
             M += n
             n_want += len(e.want)
 
-        # all or nothing: see that every group can cover every entry before taking a page
         paged = cache.paged_groups()
-        n_new = sum(1 for e in entries if not cache.has(e.request))
+        if starts_fast is not None:
+            M = len(entries)
+            n_want = sum(len(e.want) for e in entries)
+        # all or nothing: see that every group can cover every entry before taking a page
+        n_new = 0 if starts_fast is not None else sum(1 for e in entries if not cache.has(e.request))
         if n_new > cache.num_free_slots():
             raise EngineError(f"{n_new} new requests but only {cache.num_free_slots()} free request slots")
-        for gi, g in paged:
+        for gi, g in (paged if starts_fast is None else ()):
             need = 0
             for e in entries:
                 known = cache.has(e.request)
@@ -251,7 +256,7 @@ class Engine:
                 need += g.pages_to_cover(e.request if known else None, upto)
             if need > g.pool.num_free:
                 raise OutOfPages(f"the step needs {need} new pages in cache group {gi}, {g.pool.num_free} are free")
-        for e in entries:
+        for e in (entries if starts_fast is None else ()):
             if not cache.has(e.request):
                 cache.admit(e.request)
             cache.reserve(e.request, len(e.tokens))
@@ -284,16 +289,20 @@ class Engine:
         ent_flat: List[int] = []
         if ctx.decode_only:
             # single tokens only: three short lists, one assignment each
-            starts = [cache.length(e.request) for e in entries]
+            starts = starts_fast if starts_fast is not None else [cache.length(e.request) for e in entries]
             h[o_tok:o_pos] = [e.tokens[0] for e in entries]
             h[o_pos:o_slot] = starts
             h[o_slot:o_out] = range(R)
-            for i, (e, start) in enumerate(zip(entries, starts)):
-                rec = (i, 1, start, cache.slot(e.request))
-                ctx.entries.append(rec)
-                ent_flat.extend(rec)
-                for _ in e.want:
-                    out_rows.append(i)
+            known = cache._requests
+            slots = [known[e.request].slot for e in entries]
+            ctx.entries = list(zip(range(R), [1] * R, starts, slots))
+            ent = np.empty((R, 4), dtype=np.int32)
+            ent[:, 0] = np.arange(R, dtype=np.int32)
+            ent[:, 1] = 1
+            ent[:, 2] = starts
+            ent[:, 3] = slots
+            ent_flat = ent.ravel()
+            out_rows = [i for i, e in enumerate(entries) for _ in e.want]
             ctx.max_context = max(starts) + 1
         else:
             tiles: List[int] = []         # (entry, first row) pairs, flat
@@ -326,12 +335,12 @@ class Engine:
             small.sort(key=lambda t: -t[0])
             h[o_tile:o_tab] = tiles + [v for t in small for v in t[1:]] + dec_rows
         ctx.split_context = ctx.max_context
-        h[o_out:o_tile] = out_rows + ent_flat
+        h[o_out:o_ent] = out_rows
+        h[o_ent:o_tile] = ent_flat
         for k, (gi, g) in enumerate(paged):
             base = o_tab + k * R * W
             rows = g.rows
-            for i, e in enumerate(entries):
-                h[base + i * W:base + (i + 1) * W] = rows[e.request]
+            h[base:base + R * W].reshape(R, W)[:] = [rows[e.request] for e in entries]
         dev[:total].copy_(host[:total], non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
@@ -349,7 +358,34 @@ class Engine:
             base = o_tab + k * R * W
             ctx._views[gi] = CacheView(dev[base:base + R * W].view(R, W), self.page_size)
         ctx._entries_in = list(entries)
+        ctx._decode_fast = starts_fast is not None
         return ctx
+
+    def _reserve_decode_step(self, entries: Sequence[StepEntry]) -> Optional[List[int]]:
+        """The common step, checked and reserved in one pass: every entry is one token of a
+        request that is admitted already.  Returns the tokens' positions, or None for any
+        other step (nothing has been done then; `prepare` takes its general path)."""
+        cache = self.cache
+        known = cache._requests
+        for e in entries:
+            if len(e.tokens) != 1 or e.request not in known:
+                return None
+        reqs = [e.request for e in entries]
+        if len(set(reqs)) != len(reqs):
+            return None                                   # the general path names the request
+        toks = [e.tokens[0] for e in entries]
+        if not (0 <= min(toks) and max(toks) < self.model.vocab_size):
+            return None                                   # the general path names the token
+        for e in entries:
+            for w in e.want:
+                if w != 0:
+                    return None
+        try:
+            return cache.reserve_one_each(reqs)
+        except CacheError as err:
+            if isinstance(err, OutOfPages):
+                raise
+            raise EngineError(str(err)) from None
 
     def run(self, ctx: StepContext) -> Optional[torch.Tensor]:
         """The model over the step's tokens: embedding, the layers in run order,
@@ -366,8 +402,11 @@ class Engine:
         return model.head.forward(ctx, h)
 
     def finish(self, ctx: StepContext) -> None:
-        for e in ctx._entries_in:
-            self.cache.commit(e.request, len(e.tokens))
+        if ctx._decode_fast:
+            self.cache.commit_one_each([e.request for e in ctx._entries_in])
+        else:
+            for e in ctx._entries_in:
+                self.cache.commit(e.request, len(e.tokens))
         self.steps_run += 1
 
     # ------------------------------------------------------------ decode graphs
