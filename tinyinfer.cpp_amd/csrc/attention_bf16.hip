@@ -188,14 +188,31 @@ __device__ __forceinline__ void attend_pair(KVPair<HD>& f, const Frag8* qf, Bloc
 // run the loads of the next pair are in flight while a pair is computed (two fragment
 // sets take turns; loads past the end repeat the last block and are not used).
 // `check(block)` tells whether a block needs masks.
-template <int HD, typename Check>
+struct NoHook {
+  __device__ __forceinline__ void operator()() const {}
+};
+
+// `after_table` runs once, right after the first load of page ids has been issued, and
+// `before_attend` once, after the loads of the first pair have been issued and before the
+// first pair is computed (both also when there is no block to walk; every wavefront of a
+// workgroup runs each exactly once, so they may hold a barrier).  Loads come back in the
+// order they were issued: what a caller asks for in `after_table` arrives before the keys
+// and values, and what it computes in `before_attend` runs while those are in flight.
+template <int HD, typename Check, typename AfterTable = NoHook, typename BeforeAttend = NoHook>
 __device__ __forceinline__ void walk_blocks(const PagedKV& kv, const Frag8* qf, int first, int stride, int n,
                                             int lo, int hi, int kv_last, float scale, Check check, float& m,
-                                            float& l, floatx4* o) {
+                                            float& l, floatx4* o, AfterTable after_table = NoHook{},
+                                            BeforeAttend before_attend = NoHook{}) {
   const int lane = threadIdx.x & 63;
+  bool hooks_due = true;
   for (int c0 = 0; c0 < n; c0 += 64) {
     const int nc = min(64, n - c0);
     const int mine = (lane < nc) ? kv.table[((first + (c0 + lane) * stride) * 16) / kv.P] : -1;
+    if (hooks_due) {
+      __builtin_amdgcn_sched_barrier(0);
+      after_table();
+      __builtin_amdgcn_sched_barrier(0);
+    }
     KVPair<HD> f0, f1;
     BlockInfo a0, b0, a1, b1;
     // block j of this run, clamped to the run's last block
@@ -212,12 +229,22 @@ __device__ __forceinline__ void walk_blocks(const PagedKV& kv, const Frag8* qf, 
       load_pair<HD>(kv, max(pa, 0), A.key0, max(pb, 0), B.key0, f);
     };
     issue(0, f0, a0, b0);
+    if (hooks_due) {
+      __builtin_amdgcn_sched_barrier(0);
+      before_attend();
+      __builtin_amdgcn_sched_barrier(0);
+      hooks_due = false;
+    }
     for (int i = 0; i < nc; i += 4) {
       issue(i + 2, f1, a1, b1);
       attend_pair<HD>(f0, qf, a0, b0, lo, hi, kv_last, scale, m, l, o);
       issue(i + 4, f0, a0, b0);
       if (i + 2 < nc) attend_pair<HD>(f1, qf, a1, b1, lo, hi, kv_last, scale, m, l, o);
     }
+  }
+  if (hooks_due) {
+    after_table();
+    before_attend();
   }
 }
 
@@ -237,95 +264,110 @@ struct QKPrep {
   bf16_t* pool_w;            // the cache to write the new key and value into; nullptr: nothing is written
 };
 
-// Q^T fragments of this lane's column (one q head) from the 32-bit projection: the same
-// arithmetic as qk_head_wave, in the layout of the first product.  A lane holds the dims
-// 32 s + 8 quad + j (s < HD / 32, j < 8), which are both halves of its rotation pairs; the
-// sum of squares goes up the same tree as the butterfly of a wavefront with one pair per lane.
 template <int HD>
-__device__ __forceinline__ void prepare_q(const QKPrep& pr, const float* __restrict__ src, int p, bool valid,
-                                          Frag8* qf) {
+struct QueryLoads {
   static_assert(HD == 64 || HD == 128, "a lane holds whole rotation pairs for these head sizes only");
-  constexpr int NS = HD / 32, NP = NS / 2, HALF = HD / 2;
-  const int lane = threadIdx.x & 63, quad = lane >> 4;
+  static constexpr int NS = HD / 32, NP = NS / 2, HALF = HD / 2;
   float x[NS][8];
-#pragma unroll
-  for (int s = 0; s < NS; ++s) {
-    const float4 a = *reinterpret_cast<const float4*>(src + s * 32 + quad * 8);
-    const float4 b = *reinterpret_cast<const float4*>(src + s * 32 + quad * 8 + 4);
-    x[s][0] = a.x; x[s][1] = a.y; x[s][2] = a.z; x[s][3] = a.w;
-    x[s][4] = b.x; x[s][5] = b.y; x[s][6] = b.z; x[s][7] = b.w;
-  }
-  float scale = 1.f;
-  if (pr.q_w) {
-    float u[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      u[j] = qk_pair_square(x[0][j], x[NP][j]);
-      if (NP == 2) u[j] += qk_pair_square(x[1][j], x[1 + NP][j]);   // pairs i and i + 32
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) u[j] += __shfl_xor(u[j], 32, 64);   // pairs i and i ^ 16
-#pragma unroll
-    for (int j = 0; j < 8; ++j) u[j] += __shfl_xor(u[j], 16, 64);   // i ^ 8
-#pragma unroll
-    for (int j = 0; j < 4; ++j) u[j] += u[j + 4];                   // i ^ 4
-    u[0] += u[2];                                                   // i ^ 2
-    u[1] += u[3];
-    scale = qk_norm_scale(u[0] + u[1], HD, pr.eps);                 // i ^ 1
-  }
-  // weights and angles of this lane's pairs: fetched in one go (the table case and the computed
-  // case are told apart once, not per element, so that the loads go out together)
   float wl[NP][8], wh[NP][8];
   float2 cs[NP][8];
-  const bool from_table = pr.inv_freq && pr.rope_table && p < pr.table_len;   // the same in every lane
+  bool from_table;
+
+  // everything the preparation reads, asked for in one go (the table case and the computed case
+  // of the angles are told apart once, not per element, so that the loads go out together)
+  __device__ __forceinline__ void load(const QKPrep& pr, const float* __restrict__ src, int p) {
+    const int lane = threadIdx.x & 63, quad = lane >> 4;
 #pragma unroll
-  for (int sp = 0; sp < NP; ++sp) {
-    const int i0 = sp * 32 + quad * 8;
-    if (pr.q_w) {
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const float4 a = *reinterpret_cast<const float4*>(pr.q_w + i0 + 4 * h);
-        const float4 b = *reinterpret_cast<const float4*>(pr.q_w + i0 + HALF + 4 * h);
-        wl[sp][4 * h] = a.x; wl[sp][4 * h + 1] = a.y; wl[sp][4 * h + 2] = a.z; wl[sp][4 * h + 3] = a.w;
-        wh[sp][4 * h] = b.x; wh[sp][4 * h + 1] = b.y; wh[sp][4 * h + 2] = b.z; wh[sp][4 * h + 3] = b.w;
-      }
+    for (int s = 0; s < NS; ++s) {
+      const float4 a = *reinterpret_cast<const float4*>(src + s * 32 + quad * 8);
+      const float4 b = *reinterpret_cast<const float4*>(src + s * 32 + quad * 8 + 4);
+      x[s][0] = a.x; x[s][1] = a.y; x[s][2] = a.z; x[s][3] = a.w;
+      x[s][4] = b.x; x[s][5] = b.y; x[s][6] = b.z; x[s][7] = b.w;
     }
-    if (from_table) {
-      const float4* t = reinterpret_cast<const float4*>(pr.rope_table + (size_t)p * HALF + i0);
+    from_table = pr.inv_freq && pr.rope_table && p < pr.table_len;   // the same in every lane
 #pragma unroll
-      for (int h = 0; h < 4; ++h) {
-        const float4 v = t[h];
-        cs[sp][2 * h] = make_float2(v.x, v.y);
-        cs[sp][2 * h + 1] = make_float2(v.z, v.w);
-      }
-    } else if (pr.inv_freq) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) cs[sp][j] = qk_cos_sin(i0 + j, HALF, p, pr.inv_freq, nullptr, 0);
-    }
-  }
-#pragma unroll
-  for (int sp = 0; sp < NP; ++sp) {
-    bf16_t* lo_h = reinterpret_cast<bf16_t*>(&qf[sp].u);
-    bf16_t* hi_h = reinterpret_cast<bf16_t*>(&qf[sp + NP].u);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      float lo = x[sp][j] * scale, hi = x[sp + NP][j] * scale;
+    for (int sp = 0; sp < NP; ++sp) {
+      const int i0 = sp * 32 + quad * 8;
       if (pr.q_w) {
-        lo *= wl[sp][j];
-        hi *= wh[sp][j];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const float4 a = *reinterpret_cast<const float4*>(pr.q_w + i0 + 4 * h);
+          const float4 b = *reinterpret_cast<const float4*>(pr.q_w + i0 + HALF + 4 * h);
+          wl[sp][4 * h] = a.x; wl[sp][4 * h + 1] = a.y; wl[sp][4 * h + 2] = a.z; wl[sp][4 * h + 3] = a.w;
+          wh[sp][4 * h] = b.x; wh[sp][4 * h + 1] = b.y; wh[sp][4 * h + 2] = b.z; wh[sp][4 * h + 3] = b.w;
+        }
       }
-      if (pr.inv_freq) qk_rotate(lo, hi, cs[sp][j]);
-      lo_h[j] = f2bf(valid ? lo : 0.f);
-      hi_h[j] = f2bf(valid ? hi : 0.f);
+      if (from_table) {
+        const float4* t = reinterpret_cast<const float4*>(pr.rope_table + (size_t)p * HALF + i0);
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          const float4 v = t[h];
+          cs[sp][2 * h] = make_float2(v.x, v.y);
+          cs[sp][2 * h + 1] = make_float2(v.z, v.w);
+        }
+      }
     }
   }
-}
+
+  // Q^T fragments of this lane's column (one q head): the same arithmetic as qk_head_wave, in
+  // the layout of the first product.  A lane holds the dims 32 s + 8 quad + j (s < HD / 32,
+  // j < 8), which are both halves of its rotation pairs; the sum of squares goes up the same
+  // tree as the butterfly of a wavefront with one pair per lane.
+  __device__ __forceinline__ void finish(const QKPrep& pr, int p, bool valid, Frag8* qf) {
+    const int lane = threadIdx.x & 63, quad = lane >> 4;
+    float scale = 1.f;
+    if (pr.q_w) {
+      float u[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        u[j] = qk_pair_square(x[0][j], x[NP][j]);
+        if (NP == 2) u[j] += qk_pair_square(x[1][j], x[1 + NP][j]);   // pairs i and i + 32
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) u[j] += __shfl_xor(u[j], 32, 64);   // pairs i and i ^ 16
+#pragma unroll
+      for (int j = 0; j < 8; ++j) u[j] += __shfl_xor(u[j], 16, 64);   // i ^ 8
+#pragma unroll
+      for (int j = 0; j < 4; ++j) u[j] += u[j + 4];                   // i ^ 4
+      u[0] += u[2];                                                   // i ^ 2
+      u[1] += u[3];
+      scale = qk_norm_scale(u[0] + u[1], HD, pr.eps);                 // i ^ 1
+    }
+    if (pr.inv_freq && !from_table) {
+#pragma unroll
+      for (int sp = 0; sp < NP; ++sp)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) cs[sp][j] = qk_cos_sin(sp * 32 + quad * 8 + j, HALF, p, pr.inv_freq, nullptr, 0);
+    }
+#pragma unroll
+    for (int sp = 0; sp < NP; ++sp) {
+      bf16_t* lo_h = reinterpret_cast<bf16_t*>(&qf[sp].u);
+      bf16_t* hi_h = reinterpret_cast<bf16_t*>(&qf[sp + NP].u);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float lo = x[sp][j] * scale, hi = x[sp + NP][j] * scale;
+        if (pr.q_w) {
+          lo *= wl[sp][j];
+          hi *= wh[sp][j];
+        }
+        if (pr.inv_freq) qk_rotate(lo, hi, cs[sp][j]);
+        lo_h[j] = f2bf(valid ? lo : 0.f);
+        hi_h[j] = f2bf(valid ? hi : 0.f);
+      }
+    }
+  }
+};
 
 // =================================================================== decode
 // grid (rows, n_kv * head_parts, splits), 256 threads.  Partials (splits > 1):
 //   part_o [row][head][split][hd], part_ml [row][head][split][2] = (max, sum)
 // PREP: the queries come from the 32-bit projections (see QKPrep); needs parts == 1.
-template <int HD, bool PREP>
+// SHARED (with PREP): the four wavefronts need the same query; one prepares it, after the
+// first keys and values have been asked for by all four, and hands it over through LDS.  The
+// others' load units are then free for keys and values from the start, and the preparation
+// runs while those are on their way.  It costs registers (one wavefront per SIMD): for launches
+// of at most one workgroup per compute unit, where the start of the kernel is most of its time.
+template <int HD, bool PREP, bool SHARED = false>
 __global__ void __launch_bounds__(256)
 attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool, const int* __restrict__ table,
                    int table_stride, const int* __restrict__ pos, const int* __restrict__ slot,
@@ -356,23 +398,29 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
 
   PagedKV kv{pool, table + (size_t)slot[m_row] * table_stride, P, n_kv, kvh};
   Frag8 qf[HD / 32];
+  float mx = -INFINITY, l = 0.f;
+  floatx4 o[HD / 16];
+#pragma unroll
+  for (int d = 0; d < HD / 16; ++d) o[d] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int mine = (b1 - (b0 + wave) + 3) / 4;   // blocks b0 + wave, + 4, ... below b1
+  auto edge = [=](int b) { return b == blk_lo || b == blk_hi; };
   bool own_key = false;   // PREP: this workgroup takes the row's own key and value from LDS, not from the cache
   if constexpr (PREP) {
     const float* row = prep.qkv + (size_t)m_row * prep.row_width;
     own_key = prep.pool_w && blk_hi >= b0 && blk_hi < b1;
-    if (own_key) {
-      // this workgroup walks the block of the row's own position.  The position's key and value
-      // are computed here (by the code that prepares whole steps) into LDS; from there they go
-      // into the cache for later steps, and into this step's attention as a block of their own,
-      // so nothing waits for the cache to hold them.
-      if (wave == 0)
+    const int last = own_key ? p_q - 1 : p_q;      // what the cache holds for this workgroup
+    const float* q_src = row + (size_t)(r16 < n_cols ? head : kvh * G) * HD;
+    // this workgroup walks the block of the row's own position: the position's key and value
+    // are computed here (by the code that prepares whole steps) into LDS; from there they go
+    // into the cache for later steps, and into this step's attention as a block of their own,
+    // so nothing waits for the cache to hold them.
+    auto own_key_to_lds = [&]() {
+      if (wave == (SHARED ? 1 : 0))
         qk_head_wave<bf16_t>(row + (size_t)(n_head + kvh) * HD, s_kv, 1, prep.k_w, prep.eps, prep.inv_freq,
                              prep.rope_table, prep.table_len, p_q, HD);
-      if (wave == 1) v_head_wave<bf16_t>(row + (size_t)(n_head + n_kv + kvh) * HD, s_kv + HD, 1, HD);
-    }
-    prepare_q<HD>(prep, row + (size_t)(r16 < n_cols ? head : kvh * G) * HD, p_q, r16 < n_cols, qf);
-    if (own_key) {
-      __syncthreads();
+      if (wave == (SHARED ? 2 : 1)) v_head_wave<bf16_t>(row + (size_t)(n_head + n_kv + kvh) * HD, s_kv + HD, 1, HD);
+    };
+    auto own_key_to_cache = [&]() {          // after a barrier
       const int page = kv.table[p_q / P];
       if (page >= 0) {    // the host reserves pages first; never write astray
         bf16_t* kd = kv_page_slot<bf16_t>(prep.pool_w, page, 0, kvh, p_q % P, n_kv, P, HD);
@@ -382,6 +430,39 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
           vd[(size_t)i * P] = s_kv[HD + i];
         }
       }
+    };
+    if constexpr (SHARED) {
+      __shared__ uint4 s_q[HD / 32][64];
+      QueryLoads<HD> ql;
+      walk_blocks<HD>(
+          kv, qf, b0 + wave, 4, mine, lo, last, last, scale * TI_LOG2E, edge, mx, l, o,
+          [&]() {
+            if (wave == 0) ql.load(prep, q_src, p_q);   // the same for every lane of the wavefront
+          },
+          [&]() {
+            if (own_key) own_key_to_lds();
+            if (wave == 0) {
+              ql.finish(prep, p_q, r16 < n_cols, qf);
+#pragma unroll
+              for (int s = 0; s < HD / 32; ++s) s_q[s][lane] = qf[s].u;
+            }
+            __syncthreads();
+            if (wave != 0) {
+#pragma unroll
+              for (int s = 0; s < HD / 32; ++s) qf[s].u = s_q[s][lane];
+            }
+            if (own_key) own_key_to_cache();
+          });
+    } else {
+      if (own_key) own_key_to_lds();
+      QueryLoads<HD> ql;
+      ql.load(prep, q_src, p_q);
+      ql.finish(prep, p_q, r16 < n_cols, qf);
+      if (own_key) {
+        __syncthreads();
+        own_key_to_cache();
+      }
+      walk_blocks<HD>(kv, qf, b0 + wave, 4, mine, lo, last, last, scale * TI_LOG2E, edge, mx, l, o);
     }
   } else {
 #pragma unroll
@@ -390,17 +471,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
       if (r16 < n_cols)
         qf[s].u = *reinterpret_cast<const uint4*>(q + ((size_t)m_row * n_head + head) * HD + s * 32 + quad * 8);
     }
-  }
-  float mx = -INFINITY, l = 0.f;
-  floatx4 o[HD / 16];
-#pragma unroll
-  for (int d = 0; d < HD / 16; ++d) o[d] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  {
-    const int mine = (b1 - (b0 + wave) + 3) / 4;   // blocks b0 + wave, + 4, ... below b1
-    const int last = own_key ? p_q - 1 : p_q;      // what the cache holds for this workgroup
-    walk_blocks<HD>(kv, qf, b0 + wave, 4, mine, lo, last, last, scale * TI_LOG2E,
-                    [=](int b) { return b == blk_lo || b == blk_hi; }, mx, l, o);
+    walk_blocks<HD>(kv, qf, b0 + wave, 4, mine, lo, p_q, p_q, scale * TI_LOG2E, edge, mx, l, o);
   }
   if (PREP && own_key && wave == 0) {
     // the row's own key and value: a block whose first key is the only one that counts
@@ -1028,6 +1099,23 @@ static int check_common(const char* what, int n_head, int n_kv, int hd, int P, i
   return 0;
 }
 
+// compute units of the current device (asked once)
+static int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      n = v;
+    else
+      n = 256;
+  }
+  return n;
+}
+// 1 (default): small decode launches from the projections let one wavefront prepare the query
+static int g_decode_shared_query = 1;
+extern "C" void ti_attention_decode_shared_query(int on) { g_decode_shared_query = on; }
+
 // Decode rows.  rows: which rows of the step (nullptr: rows 0..n_rows-1).  n_splits > 1 needs
 // part_o (float [n_rows, n_head, n_splits, hd]) and part_ml (float [n_rows, n_head, n_splits, 2]).
 // Returns 3 for sizes these kernels do not serve.
@@ -1042,12 +1130,19 @@ static int launch_decode(const void* q, const void* pool, const int* table, int 
   const int parts = (n_head / n_kv + 15) / 16;
   TI_REQUIRE(n_kv * parts <= 65535, "attention_decode: too many heads");
   dim3 grid(n_rows, n_kv * parts, n_splits);
+  // at most one workgroup per compute unit: one wavefront prepares the query for all four
+  const bool shared = PREP && g_decode_shared_query && (long)n_rows * n_kv * parts * n_splits <= compute_units();
 #define TI_DEC(H)                                                                                          \
   case H:                                                                                                  \
-    attn_decode_kernel<H, PREP><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,     \
-                                                          table_stride, pos, slot, rows, (bf16_t*)out,      \
-                                                          part_o, part_ml, n_head, n_kv, page_size, scale,  \
-                                                          window, n_splits, prep);                          \
+    if (shared)                                                                                            \
+      attn_decode_kernel<H, PREP, PREP><<<grid, 256, 0, stream>>>(                                         \
+          (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, pos, slot, rows, (bf16_t*)out,        \
+          part_o, part_ml, n_head, n_kv, page_size, scale, window, n_splits, prep);                         \
+    else                                                                                                   \
+      attn_decode_kernel<H, PREP><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,   \
+                                                            table_stride, pos, slot, rows, (bf16_t*)out,    \
+                                                            part_o, part_ml, n_head, n_kv, page_size,       \
+                                                            scale, window, n_splits, prep);                 \
     if (n_splits > 1)                                                                                       \
       attn_merge_kernel<H><<<dim3(n_rows, n_head), (H < 64 ? 64 : H), 0, stream>>>(part_o, part_ml, rows,   \
                                                                                   (bf16_t*)out, n_head,    \

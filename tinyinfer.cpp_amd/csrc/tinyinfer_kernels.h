@@ -92,6 +92,7 @@ int ti_attention_prefill_bf16(const void* q, const void* pool, const int* table,
 int ti_attention_prefill_paired_bf16(const void* q, const void* pool, const int* table, int table_stride,
                                      const int* tiles, const int* entries, void* out, int n_tiles, int n_head,
                                      int n_kv, int hd, int page_size, float scale, int window, hipStream_t stream);
+void ti_attention_decode_shared_query(int on);   // 0: every wavefront of a decode workgroup prepares the query itself
 void ti_attention_prefill_groups(int groups);  // 1 or 2 groups of wavefronts per workgroup, 0: by the launch
 void ti_attention_prefill_use_lds(int on);     // 0: the kernel without LDS for every head size
 
