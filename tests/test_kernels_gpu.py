@@ -459,6 +459,45 @@ def test_linear_bf16_matrix_cores(ops, M, N, K):
         assert (f64(out) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 1, 8), (1, 1024, 2048), (8, 1024, 3072), (3, 7, 4096), (2, 4095, 520),
+                                   (4, 33, 1032), (8, 5, 24), (5, 1000, 2056), (7, 130, 3080)])
+def test_linear_bf16_weight_row_per_wavefront(ops, M, N, K):
+    """Up to 8 tokens and a weight of fewer than 4,096 rows: the kernel with a weight row per
+    wavefront, at the edges of what it serves (one row, one piece of K, the longest K, every
+    template variant of M and K), with strided token rows, against float64 and against the
+    kernels that take these sizes when it is switched off (same values up to rounding)."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    g = torch.Generator().manual_seed(M * 11 + N + K)
+    wide = (torch.rand(M, K + 24, generator=g) * 2 - 1).to(torch.bfloat16)
+    a = dev(wide)[:, 8:8 + K]                                    # rows 16 bytes into a wider matrix
+    w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    ref = ref_linear(wide[:, 8:8 + K], w.cpu())
+    tol = 2e-5 * K
+    lib = ops.lib("gemm_bf16")
+    base = torch.randn(M, N, generator=g)
+    results = {}
+    try:
+        for on in (1, 0):
+            lib.ti_gemm_bf16_row_per_wave(on)
+            out = torch.full((M + 1, N), 7.0, device="cuda")     # a row beyond: must stay untouched
+            ops.linear(a, w, out[:M], "store")
+            assert (f64(out[:M]) - ref).abs().max() < tol
+            assert bool((out[M] == 7.0).all())
+            acc = dev(base.clone())
+            ops.linear(a, w, acc, "add")
+            assert (f64(acc) - (ref + f64(base))).abs().max() < tol
+            results[on] = (out[:M].clone(), acc)
+    finally:
+        lib.ti_gemm_bf16_row_per_wave(1)
+    assert (results[1][0] - results[0][0]).abs().max() < tol
+    # a row's bits do not depend on the rows beside it
+    if M > 1:
+        one = torch.empty(1, N, device="cuda")
+        ops.linear(a[M - 1:M], w, one, "store")
+        assert torch.equal(one[0], results[1][0][M - 1])
+
+
 @pytest.mark.parametrize("tile", [1, 3, 6])
 @pytest.mark.parametrize("M,N,K", [(300, 520, 128), (257, 384, 192), (130, 200, 64), (700, 96, 320)])
 def test_linear_bf16_every_tile(ops, tile, M, N, K):
