@@ -368,7 +368,8 @@ class Engine:
         cache = self.cache
         known = cache._requests
         for e in entries:
-            if len(e.tokens) != 1 or e.request not in known:
+            r = known.get(e.request)
+            if len(e.tokens) != 1 or r is None or r.reserved != r.length:
                 return None
         reqs = [e.request for e in entries]
         if len(set(reqs)) != len(reqs):
