@@ -641,6 +641,59 @@ struct QKVEpilogue {
   int n_head, n_kv, hd, P;
 };
 
+// A q or k head (unit u of the fused projection, head hh of the tile) of all BM rows of a tile that
+// lies in LDS in 32-bit (row stride FS): eight lanes a row, 8 NWV rows a pass.  The angles of the
+// next pass are asked for before a pass is finished; a row's bfloat16 then leave LDS in pieces of
+// 16 bytes, the eight lanes writing 128 consecutive bytes.
+template <int HD, int BM, int NWV, int FS, bool NORMED, bool ROTATE>
+__device__ __forceinline__ void qkv_rows_by_lanes(const QKVEpilogue& ep, float* ft, const int* s_pos,
+                                                  const int* s_page, const int* s_prow, const int* s_live, int hh,
+                                                  int u, int m0) {
+  constexpr int NP = HD / 16, PASSES = BM / (NWV * 8);
+  const int tid = threadIdx.x;
+  const bool is_q = u < ep.n_head;
+  float wlo[NP], whi[NP];
+  qk_lanes_weights<HD>(wlo, whi, NORMED ? (is_q ? ep.q_w : ep.k_w) : nullptr);
+  float2 cs[NP], next[NP];
+#pragma unroll 1
+  for (int ps = -1; ps < PASSES; ++ps) {
+    if (ROTATE && ps + 1 < PASSES)
+      qk_lanes_angles<HD>(next, s_pos[(ps + 1) * NWV * 8 + tid / 8], ep.inv_freq, ep.rope_table, ep.table_len);
+    if (ps >= 0) {
+      const int r = ps * NWV * 8 + tid / 8;
+      float* row = ft + r * FS + hh * HD;
+      qk_head_lanes<HD, NORMED, ROTATE>(row, wlo, whi, ep.eps, cs);
+      bf16_t* dst = nullptr;
+      if (is_q) {
+        if (s_live[r] >= 0) dst = ep.q_out + ((size_t)(m0 + r) * ep.n_head + u) * HD;
+      } else if (s_page[r] >= 0) {
+        dst = kv_page_slot<bf16_t>(ep.pool, s_page[r], 0, u - ep.n_head, s_prow[r], ep.n_kv, ep.P, HD);
+      }
+      if (dst)
+#pragma unroll
+        for (int pc = tid & 7; pc < HD / 8; pc += 8)
+          reinterpret_cast<uint4*>(dst)[pc] = reinterpret_cast<const uint4*>(row)[pc];
+    }
+#pragma unroll
+    for (int k = 0; k < NP; ++k) cs[k] = next[k];
+  }
+}
+
+template <int HD, int BM, int NWV, int FS>
+__device__ __forceinline__ void qkv_rows_by_lanes(const QKVEpilogue& ep, float* ft, const int* s_pos,
+                                                  const int* s_page, const int* s_prow, const int* s_live, int hh,
+                                                  int u, int m0) {
+  const bool normed = (u < ep.n_head ? ep.q_w : ep.k_w) != nullptr, rotate = ep.inv_freq != nullptr;
+  if (normed && rotate)
+    qkv_rows_by_lanes<HD, BM, NWV, FS, true, true>(ep, ft, s_pos, s_page, s_prow, s_live, hh, u, m0);
+  else if (normed)
+    qkv_rows_by_lanes<HD, BM, NWV, FS, true, false>(ep, ft, s_pos, s_page, s_prow, s_live, hh, u, m0);
+  else if (rotate)
+    qkv_rows_by_lanes<HD, BM, NWV, FS, false, true>(ep, ft, s_pos, s_page, s_prow, s_live, hh, u, m0);
+  else
+    qkv_rows_by_lanes<HD, BM, NWV, FS, false, false>(ep, ft, s_pos, s_page, s_prow, s_live, hh, u, m0);
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_,
@@ -796,11 +849,14 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
   // acc[a][b][i]: row wm*(BM/WAVES_M) + a*32 + 8*(i/4) + 4*(lane/32) + i%4, column wn*(BN/WAVES_N) + b*32 + lane%32
   const int ccol = lane & 31, crow = (lane >> 5) * 4;
   if constexpr (EPI == TI_EPI_QKV_PREP) {
-    // The tile goes to LDS in 32-bit (the stages are free now), then every thread finishes one row:
-    // for each head of the tile, the arithmetic of the kernel that prepares whole steps.
-    static_assert(BM == 256, "a row per thread");
-    constexpr int FS = BN + 1;                              // row stride: threads of a wavefront read different rows
-    static_assert(BM * FS * 4 + 3 * BM * 4 <= PSTAGES * (BM + BN) * PBK * 2, "the 32-bit tile fits into the stages");
+    // The tile goes to LDS in 32-bit (the stages are free now); then, head by head of the tile, eight
+    // lanes finish a row of a q or k head (the arithmetic of the kernel that prepares whole steps; a
+    // row's eight lanes read its angles and write its result as runs of consecutive bytes), and a
+    // thread a dim of a v head.
+    static_assert(BM == 256 && NWV == 8, "a row per thread of the first four wavefronts, 64 rows per pass of all eight");
+    constexpr int FS = BN + 8;                              // row stride: the eight rows x eight lanes of a wavefront
+                                                            // read 64 different banks
+    static_assert(BM * FS * 4 + 4 * BM * 4 <= PSTAGES * (BM + BN) * PBK * 2, "the 32-bit tile fits into the stages");
     float* ft = reinterpret_cast<float*>(smem);
     __syncthreads();
 #pragma unroll
@@ -811,35 +867,33 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
         for (int b = 0; b < TN; ++b)
           ft[(wm * (BM / WAVES_M) + a * 32 + (i >> 2) * 8 + crow + (i & 3)) * FS + wn * (BN / WAVES_N) + b * 32 + ccol] =
               acc[a][b][i];
-    __syncthreads();
-    // each thread's row: its position, and where its key and value go
+    // each row's position, and where its key and value go
     int* s_page = reinterpret_cast<int*>(ft + BM * FS);     // [BM] page of the row's position, -1: none
     int* s_prow = s_page + BM;                              // [BM] row of the position in that page
     int* s_live = s_prow + BM;                              // [BM] block-table row (request) of the row, -1: none
-    const int m = m0 + tid;
-    const bool live = tid < BM && m < M;                    // (eight wavefronts: the upper four have no row)
-    const int p = live ? ep.pos[m] : 0;
+    int* s_pos = s_live + BM;                               // [BM] position of the row
     const int hd = ep.hd, units = ep.n_head + 2 * ep.n_kv;
-    // the host reserves pages first; a row without one (-1) writes nothing
-    const int page = (live && ep.n_kv > 0) ? ep.table[(size_t)ep.slot[m] * ep.table_stride + p / ep.P] : -1;
     if (tid < BM) {
-      s_page[tid] = page;
+      const int m = m0 + tid;
+      const bool live = m < M;
+      const int p = live ? ep.pos[m] : 0;
+      // the host reserves pages first; a row without one (-1) writes nothing
+      s_page[tid] = (live && ep.n_kv > 0) ? ep.table[(size_t)ep.slot[m] * ep.table_stride + p / ep.P] : -1;
       s_prow[tid] = p % ep.P;
       s_live[tid] = live ? ep.slot[m] : -1;
+      s_pos[tid] = p;
     }
     __syncthreads();
-    if (tid >= BM) return;
     for (int hh = 0; hh < BN / hd; ++hh) {
       const int u = n0 / hd + hh;                            // the same in every thread
       if (u >= units) break;
-      const float* src = ft + tid * FS + hh * hd;
       const bool is_q = u < ep.n_head, is_v = u >= ep.n_head + ep.n_kv;
       if (is_v) {
         // values go in transposed, [dim][row of the page]: thread -> one dim, for runs of 16 rows of
         // the tile; a run that is 16 consecutive rows of one page leaves as 32 contiguous bytes
         const int kvh = u - ep.n_head - ep.n_kv;
         const int d = tid % hd;
-        for (int r0 = (tid / hd) * 16; r0 < BM; r0 += (BM / hd) * 16) {
+        for (int r0 = (tid / hd) * 16; r0 < BM; r0 += (NWV * 64 / hd) * 16) {
           const int pg = s_page[r0], pr = s_prow[r0];
           // rows of a run are consecutive positions of one request: its first and last row tell
           bool run = (pg >= 0) & (pr % 16 == 0) & (s_page[r0 + 15] == pg) & (s_prow[r0 + 15] == pr + 15) &
@@ -865,21 +919,10 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
         }
         continue;
       }
-      if (!live) continue;
-      if (is_q) {
-        bf16_t* dst = ep.q_out + ((size_t)m * ep.n_head + u) * hd;
-        if (hd == 128)
-          qk_head_thread<128>(src, dst, ep.q_w, ep.eps, ep.inv_freq, ep.rope_table, ep.table_len, p);
-        else
-          qk_head_thread<64>(src, dst, ep.q_w, ep.eps, ep.inv_freq, ep.rope_table, ep.table_len, p);
-        continue;
-      }
-      if (page < 0) continue;
-      bf16_t* dst = kv_page_slot<bf16_t>(ep.pool, page, 0, u - ep.n_head, p % ep.P, ep.n_kv, ep.P, hd);
       if (hd == 128)
-        qk_head_thread<128>(src, dst, ep.k_w, ep.eps, ep.inv_freq, ep.rope_table, ep.table_len, p);
+        qkv_rows_by_lanes<128, BM, NWV, FS>(ep, ft, s_pos, s_page, s_prow, s_live, hh, u, m0);
       else
-        qk_head_thread<64>(src, dst, ep.k_w, ep.eps, ep.inv_freq, ep.rope_table, ep.table_len, p);
+        qkv_rows_by_lanes<64, BM, NWV, FS>(ep, ft, s_pos, s_page, s_prow, s_live, hh, u, m0);
     }
     return;
   }

@@ -120,6 +120,87 @@ __device__ __forceinline__ void qk_head_thread(const float* src, bf16_t* dst, co
   }
 }
 
+// One head by eight adjacent lanes of a wavefront: lane j of the eight takes the pairs j, j + 8, ...
+// of the row.  The three functions below give such a lane its norm weights, its angles, and the
+// finished row.  The loads of the first two do not wait for one another, and a caller with several
+// rows asks for all their angles before it finishes the first.
+template <int HD>
+__device__ __forceinline__ void qk_lanes_weights(float (&wlo)[HD / 16], float (&whi)[HD / 16], const float* w) {
+  const int j = threadIdx.x & 7;
+#pragma unroll
+  for (int k = 0; k < HD / 16; ++k) {
+    wlo[k] = w ? w[j + 8 * k] : 1.f;
+    whi[k] = w ? w[HD / 2 + j + 8 * k] : 1.f;
+  }
+}
+
+// (cos, sin) of this lane's pairs at position p; inv_freq must not be nullptr
+template <int HD>
+__device__ __forceinline__ void qk_lanes_angles(float2 (&cs)[HD / 16], int p, const float* inv_freq,
+                                                const float2* rope_table, int table_len) {
+  constexpr int HALF = HD / 2;
+  const int j = threadIdx.x & 7;
+  const bool held = rope_table && p < table_len;
+  if (rope_table) {
+    // every lane loads (a row beyond the table reads the last one and computes below)
+    const float2* tp = rope_table + (size_t)min(p, table_len - 1) * HALF;
+#pragma unroll
+    for (int k = 0; k < HD / 16; ++k) cs[k] = tp[j + 8 * k];
+  }
+  if (!held) {
+#pragma unroll
+    for (int k = 0; k < HD / 16; ++k) cs[k] = qk_cos_sin(j + 8 * k, HALF, p, inv_freq, nullptr, 0);
+  }
+}
+
+// From HD floats at `row` (LDS, 16-byte aligned) to HD bfloat16 that overwrite the first half of the
+// same floats.  A lane's own pairs go up the tree of the sum of squares in the lane (partners at
+// distance 32, 16, 8), the rest across the eight lanes (4, 2, 1): the tree of qk_head_wave's
+// butterfly, so the bits are the same.  All lanes of the wavefront call it together; a row that
+// is not wanted is computed and left in LDS.  NORMED: with the norm (weights wlo, whi); ROTATE:
+// with the rotation by cs.
+template <int HD, bool NORMED, bool ROTATE>
+__device__ __forceinline__ void qk_head_lanes(float* row, const float (&wlo)[HD / 16], const float (&whi)[HD / 16],
+                                              float eps, const float2 (&cs)[HD / 16]) {
+  constexpr int HALF = HD / 2, NP = HALF / 8;
+  static_assert(NP == 4 || NP == 8, "the tree below is that of a 64-lane butterfly with one pair a lane");
+  const int j = threadIdx.x & 7;
+  float lo[NP], hi[NP];
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    lo[k] = row[j + 8 * k];
+    hi[k] = row[HALF + j + 8 * k];
+  }
+  // the eight lanes read all of the row before any of them writes into it (a wavefront runs its
+  // LDS instructions in order; the compiler is told not to move them)
+  asm volatile("" ::: "memory");
+  float scale = 1.f;
+  if (NORMED) {
+    float t[NP];
+#pragma unroll
+    for (int k = 0; k < NP; ++k) t[k] = qk_pair_square(lo[k], hi[k]);
+#pragma unroll
+    for (int o = NP / 2; o >= 1; o >>= 1)
+#pragma unroll
+      for (int k = 0; k < o; ++k) t[k] += t[k + o];
+    scale = qk_norm_scale(group_sum<8>(t[0]), HD, eps);
+  }
+  bf16_t* rb = reinterpret_cast<bf16_t*>(row);
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    const int i = j + 8 * k;
+    float a = lo[k] * scale, b = hi[k] * scale;
+    if (NORMED) {
+      a *= wlo[k];
+      b *= whi[k];
+    }
+    if (ROTATE) qk_rotate(a, b, cs[k]);
+    rb[i] = f2bf(a);
+    rb[i + HALF] = f2bf(b);
+  }
+  asm volatile("" ::: "memory");
+}
+
 // A value head: copied (rounded to T), element d to dst[d * dst_stride]
 template <typename T>
 __device__ __forceinline__ void v_head_wave(const float* __restrict__ src, T* __restrict__ dst, size_t dst_stride,
