@@ -853,7 +853,7 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
     // lanes finish a row of a q or k head (the arithmetic of the kernel that prepares whole steps; a
     // row's eight lanes read its angles and write its result as runs of consecutive bytes), and a
     // thread a dim of a v head.
-    static_assert(BM == 256 && NWV == 8, "a row per thread of the first four wavefronts, 64 rows per pass of all eight");
+    static_assert(BM == 256 && NWV == 8, "the first four wavefronts look up a row each; 64 rows per pass of all eight");
     constexpr int FS = BN + 8;                              // row stride: the eight rows x eight lanes of a wavefront
                                                             // read 64 different banks
     static_assert(BM * FS * 4 + 4 * BM * 4 <= PSTAGES * (BM + BN) * PBK * 2, "the 32-bit tile fits into the stages");
