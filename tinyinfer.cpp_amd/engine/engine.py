@@ -219,6 +219,7 @@ class Engine:
         cache = self.cache
         starts_fast = self._reserve_decode_step(entries)
         seen = set()
+        token_arrays: Dict[Hashable, np.ndarray] = {}
         M = 0
         n_want = 0
         for e in (entries if starts_fast is None else ()):
@@ -229,7 +230,16 @@ class Engine:
             seen.add(e.request)
             if n == 0:
                 raise EngineError(f"request {e.request!r}: an entry needs at least one token")
-            if not (0 <= min(toks) and max(toks) < V):
+            if n > 64:
+                # a long portion: one conversion serves the check here and the upload below
+                arr = np.asarray(toks)
+                if arr.ndim != 1 or arr.dtype.kind not in "iu":
+                    raise EngineError(f"request {e.request!r}: token ids must be a flat sequence of integers")
+                in_vocab = 0 <= int(arr.min()) and int(arr.max()) < V
+                token_arrays[e.request] = arr
+            else:
+                in_vocab = 0 <= min(toks) and max(toks) < V
+            if not in_vocab:
                 bad = next(t for t in toks if not (0 <= int(t) < V))
                 raise EngineError(f"request {e.request!r}: token id {bad} is outside the vocabulary [0, {V})")
             if e.want and not (0 <= min(e.want) and max(e.want) < n):
@@ -315,7 +325,7 @@ class Engine:
                 rec = (row0, n, start, cache.slot(e.request))
                 ctx.entries.append(rec)
                 ent_flat.extend(rec)
-                h[o_tok + row0:o_tok + row0 + n] = e.tokens
+                h[o_tok + row0:o_tok + row0 + n] = token_arrays.get(e.request, e.tokens)
                 h[o_slot + row0:o_slot + row0 + n] = i
                 if n > 1:
                     h[o_pos + row0:o_pos + row0 + n] = np.arange(start, start + n, dtype=np.int32)

@@ -23,6 +23,9 @@ class KernelError(RuntimeError):
     pass
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _code(dt: torch.dtype) -> int:
     if dt == torch.float32:
         return F32
@@ -98,6 +101,11 @@ class Ops:
 
     @staticmethod
     def _stream():
+        """The current stream's handle.  Every launch asks for it; torch's raw accessor, where this
+        build of torch has it, answers in well under a microsecond (the public one builds a
+        Stream object: ~8 us a call)."""
+        if _RAW_STREAM is not None:
+            return ctypes.c_void_p(_RAW_STREAM(torch.cuda.current_device()))
         return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
     @staticmethod
