@@ -40,15 +40,16 @@ _plain_cache = {}
 
 def plain_logits(folder, requests, dtype):
     """({request: logits [T, V]}, tolerance) of the plain model for this dtype."""
+    key = (folder, tuple((r, tuple(t)) for r, t in sorted(requests.items())))
     for d in ("float32", "bfloat16"):
-        if (folder, d) not in _plain_cache:
+        if key + (d,) not in _plain_cache:
             cfg, w = read_folder(folder)
             rnd = ROUNDED if d == "bfloat16" else plain.no_rounding
-            _plain_cache[(folder, d)] = {r: plain.forward(w, cfg, t, rnd) for r, t in requests.items()}
-    want = _plain_cache[(folder, dtype)]
+            _plain_cache[key + (d,)] = {r: plain.forward(w, cfg, t, rnd) for r, t in requests.items()}
+    want = _plain_cache[key + (dtype,)]
     if dtype == "float32":
         return want, TOL["float32"]
-    exact = _plain_cache[(folder, "float32")]
+    exact = _plain_cache[key + ("float32",)]
     noise = max(float(np.abs(want[r] - exact[r]).max()) for r in want)
     return want, BF16_NOISE_FACTOR * noise
 
@@ -59,7 +60,7 @@ def replay(engine, trace):
     got = {}
     for step in trace:
         logits = engine.step([StepEntry(r, t, w) for r, t, w in step["entries"]])
-        rows = logits.cpu().numpy().astype(np.float64)
+        rows = None if logits is None else logits.cpu().numpy().astype(np.float64)     # None: nothing wanted
         i = 0
         for r, t, w in step["entries"]:
             for _ in w:
@@ -263,6 +264,46 @@ def test_layers_of_real_width_match_plain(model_folders, dtype):
         err = np.abs(got[r] - want[r][rows[r]]).max()
         print(f"\n[E {dtype} {r}] max |engine - plain| = {err:.3e} (allowed {tol:.3e}, logits up to {scale:.1f})")
         assert err < tol, (r, err, tol)
+
+
+def test_steps_of_17_to_64_tokens_at_real_width(model_folders):
+    """Steps of 17 to 64 tokens at the widths of Qwen3-0.6B: the products into the residual split
+    K over workgroups and leave their partial sums to the norm that follows (the last one to a
+    kernel of their own, before the final norm of the wanted rows).  A prompt in portions of 40,
+    17, 64 and 33 tokens, one of them beside another request's token, then a step that wants
+    nothing: against the plain model; with the sums added at once the bits are the same, and
+    with the kernels without MFMA the logits agree within the same bound."""
+    from tinyinfer_amd.ops.kernels import get_ops
+    folder = model_folders("E", "bfloat16", True)
+    V = CONFIGS["E"]["vocab_size"]
+    requests = {"a": random_tokens(154, V, 41), "b": random_tokens(3, V, 42)}
+    want, tol = plain_logits(folder, requests, "bfloat16")
+    a, b = requests["a"], requests["b"]
+    trace = [{"entries": [("a", a[:40], [0, 39])], "end": []},
+             {"entries": [("a", a[40:57], [16])], "end": []},
+             {"entries": [("b", b[:2], []), ("a", a[57:119], [0, 61])], "end": []},
+             {"entries": [("a", a[119:152], [])], "end": []},                   # wants nothing
+             {"entries": [("a", a[152:154], [0, 1]), ("b", b[2:3], [0])], "end": ["a", "b"]}]
+    rows = {"a": [0, 39, 56, 57, 118, 152, 153], "b": [2]}
+    ops = get_ops()
+    results = {}
+    try:
+        for how in ("left to the norm", "added at once", "without MFMA"):
+            ops.use_deferred_add = how == "left to the norm"
+            ops.use_mfma_rows = how != "without MFMA"
+            results[how] = replay(build_engine(folder, "bfloat16", 256), trace)
+            assert ops._pending is None
+    finally:
+        ops.use_deferred_add = ops.use_mfma_rows = True
+    for r in requests:
+        got = results["left to the norm"][r]
+        err = np.abs(got - want[r][rows[r]]).max()
+        print(f"\n[E 17..64 tokens {r}] max |engine - plain| = {err:.3e} (allowed {tol:.3e})")
+        assert err < tol, (r, err, tol)
+        assert np.array_equal(got, results["added at once"][r]), r
+        assert np.abs(results["without MFMA"][r] - want[r][rows[r]]).max() < tol, r
+    assert not np.array_equal(results["left to the norm"]["a"], results["without MFMA"]["a"]), \
+        "the switch did not change the kernel"
 
 
 def test_step_refuses_what_it_cannot_run(model_folders):

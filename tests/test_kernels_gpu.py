@@ -498,6 +498,107 @@ def test_linear_bf16_weight_row_per_wavefront(ops, M, N, K):
         assert torch.equal(one[0], results[1][0][M - 1])
 
 
+@pytest.mark.parametrize("M,N,K,ks", [(1, 16, 64, 1), (17, 1024, 2048, 4), (64, 1024, 3072, 8), (33, 50, 256, 3),
+                                      (48, 7, 128, 2), (5, 40, 192, 1), (64, 130, 1024, 5)])
+def test_linear_bf16_mfma_fed_from_memory(ops, M, N, K, ks):
+    """The kernel for 17 to 64 rows alone (16x16x32 MFMAs whose operands come straight from
+    memory), through its test entry point: every epilogue, 1 to 4 blocks of 16 rows, columns that
+    do not fill a tile, K split over workgroups with the partial sums added afterwards, strided
+    rows; against float64.  A row's bits do not depend on the rows beside it."""
+    import ctypes
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    lib = ops.lib("gemm_bf16")
+    g = torch.Generator().manual_seed(M * 7 + N + K + ks)
+    wide = (torch.rand(M, K + 24, generator=g) * 2 - 1).to(torch.bfloat16)
+    a = dev(wide)[:, 8:8 + K]
+    w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    ref = ref_linear(wide[:, 8:8 + K], w.cpu())
+    tol = 2e-5 * K
+    partial = torch.empty(ks * M * N, device="cuda")
+
+    def run(rows, out, epi, splits=1):
+        ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+        rc = lib.ti_gemm_bf16_mblocks_any(ptr(rows), ptr(w), ptr(out), rows.shape[0], out.shape[1], K,
+                                          ctypes.c_long(rows.stride(0)), epi, ptr(partial), splits, None)
+        assert rc == 0, lib.ti_last_error()
+    out = torch.full((M + 1, N), 7.0, device="cuda")
+    run(a, out[:M], 0)
+    assert (f64(out[:M]) - ref).abs().max() < tol
+    assert bool((out[M] == 7.0).all())
+    one = torch.empty(1, N, device="cuda")
+    run(a[M - 1:M], one, 0)
+    assert torch.equal(one[0], out[M - 1])
+    base = torch.randn(M, N, generator=g)
+    for splits in sorted({1, ks}):
+        acc = dev(base.clone())
+        run(a, acc, 1, splits)
+        assert (f64(acc) - (ref + f64(base))).abs().max() < tol
+    act = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+    run(a, act, 2)
+    assert (f64(act) - ref).abs().max() < 0.005 * ref.abs().max() + tol
+    if N % 2 == 0:
+        F = N // 2
+        sw = torch.empty(M, F, device="cuda", dtype=torch.bfloat16)
+        run(a, sw, 3)
+        gte, up = ref[:, :F], ref[:, F:]
+        want = gte / (1 + torch.exp(-gte)) * up
+        assert (f64(sw) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 1024, 2048), (64, 1024, 3072), (40, 512, 1024), (33, 96, 1024)])
+def test_partial_sums_left_to_the_next_norm(ops, M, N, K):
+    """A product into the residual at 17..64 rows with few columns splits K over workgroups.
+    With `may_defer` its partial sums wait for whatever reads the residual next: the norm adds
+    them on its way, any other launch (or `flush`) adds them with a kernel of their own.  All
+    three give the bits of the product that adds them at once, and match float64."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    g = torch.Generator().manual_seed(M + N + K)
+    a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    base = torch.randn(M, N, generator=g)
+    nw = dev(torch.rand(N, generator=g) + 0.5)
+    ref = ref_linear(a.cpu(), w.cpu()) + f64(base)
+    eps = 1e-5
+
+    def product_then_norm(how):
+        x = dev(base.clone())
+        h = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+        ops.use_deferred_add = how != "at once"
+        try:
+            ops.linear(a, w, x, "add", may_defer=True)
+        finally:
+            ops.use_deferred_add = True
+        if how == "flush":
+            ops.flush()
+        if how == "another launch":
+            other = torch.empty(M, N, device="cuda")
+            ops.linear(a, w, other, "store")              # reads nothing of x, but goes first
+            assert ops._pending is None
+        if how == "norm":
+            assert ops._pending is not None               # these sizes do split K
+        ops.rmsnorm(x, nw, eps, h)
+        assert ops._pending is None
+        return x, h
+    want_x, want_h = product_then_norm("at once")
+    assert (f64(want_x) - ref).abs().max() < 2e-5 * K
+    assert (f64(want_h) - ref_rmsnorm(f64(want_x), f64(nw), eps)).abs().max() < 0.02
+    for how in ("norm", "flush", "another launch"):
+        x, h = product_then_norm(how)
+        assert torch.equal(x, want_x), how
+        assert torch.equal(h, want_h), how
+    # switched off, the other kernels take these sizes: the same values up to rounding
+    try:
+        ops.use_mfma_rows = False
+        x = dev(base.clone())
+        ops.linear(a, w, x, "add", may_defer=True)
+        assert ops._pending is None
+        assert (x - want_x).abs().max() < 2e-5 * K
+    finally:
+        ops.use_mfma_rows = True
+
+
 @pytest.mark.parametrize("tile", [1, 3, 6])
 @pytest.mark.parametrize("M,N,K", [(300, 520, 128), (257, 384, 192), (130, 200, 64), (700, 96, 320)])
 def test_linear_bf16_every_tile(ops, tile, M, N, K):

@@ -103,6 +103,62 @@ extern "C" int ti_rmsnorm(int out_dtype, const float* x, const float* w, const i
   return 0;
 }
 
+// The norm of rows whose last product left its sums of a split K in `partial` [KS][n_rows][H]:
+// x[r] += partial[0][r] + ... + partial[KS - 1][r] (in that order, written back), then the norm of
+// rmsnorm_wave_kernel over the new x.  A wavefront per row, four rows a workgroup.
+template <typename T>
+__global__ void __launch_bounds__(256)
+rmsnorm_add_partials_kernel(float* __restrict__ x, const float* __restrict__ partial, int KS,
+                            const float* __restrict__ w, T* __restrict__ out, int n_rows, int H, float eps) {
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (r >= n_rows) return;
+  float* src = x + (size_t)r * H;
+  const size_t count = (size_t)n_rows * H;
+  float ss = 0.f;
+  for (int k = lane * 4; k < H; k += 256) {
+    float4 v = *reinterpret_cast<const float4*>(src + k);
+    for (int s = 0; s < KS; ++s) {
+      const float4 p = *reinterpret_cast<const float4*>(partial + s * count + (size_t)r * H + k);
+      v.x += p.x;
+      v.y += p.y;
+      v.z += p.z;
+      v.w += p.w;
+    }
+    *reinterpret_cast<float4*>(src + k) = v;
+    ss = rms_accumulate(ss, v);
+  }
+  const float scale = rms_scale(ss, H, eps);
+  T* dst = out + (size_t)r * H;
+  for (int k = lane * 4; k < H; k += 256) {
+    const float4 v = *reinterpret_cast<const float4*>(src + k);     // this lane's own store above
+    const float4 g = *reinterpret_cast<const float4*>(w + k);
+    st<T>(dst + k, v.x * scale * g.x);
+    st<T>(dst + k + 1, v.y * scale * g.y);
+    st<T>(dst + k + 2, v.z * scale * g.z);
+    st<T>(dst + k + 3, v.w * scale * g.w);
+  }
+}
+
+// Returns 3 for a width or an alignment it does not serve (the caller adds the partial sums with
+// their own kernel then, and norms with ti_rmsnorm).
+extern "C" int ti_rmsnorm_add_partials(int out_dtype, float* x, const float* partial, int KS, const float* w,
+                                       void* out, int n_rows, int H, float eps, hipStream_t stream) {
+  TI_REQUIRE(n_rows >= 0 && H > 0 && KS >= 1, "rmsnorm_add_partials: bad sizes rows=%d H=%d KS=%d", n_rows, H, KS);
+  TI_REQUIRE(out_dtype == TI_F32 || out_dtype == TI_BF16, "rmsnorm_add_partials: unknown dtype %d", out_dtype);
+  if (H % 4 != 0 || (((uintptr_t)x | (uintptr_t)w | (uintptr_t)partial) & 15) != 0) {
+    ti_set_error("rmsnorm_add_partials: serves widths that are multiples of 4 and 16-byte aligned operands");
+    return 3;
+  }
+  if (n_rows == 0) return 0;
+  const int grid = (n_rows + 3) / 4;
+  if (out_dtype == TI_F32)
+    rmsnorm_add_partials_kernel<float><<<grid, 256, 0, stream>>>(x, partial, KS, w, (float*)out, n_rows, H, eps);
+  else
+    rmsnorm_add_partials_kernel<bf16_t><<<grid, 256, 0, stream>>>(x, partial, KS, w, (bf16_t*)out, n_rows, H, eps);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
 // ----------------------------------------------------------- rotary, by itself
 // In place on f32 x[m, h, :] with row stride `row_stride` floats: pair (k, k+hd/2)
 // turns by pos[m] * inv_freq[k].

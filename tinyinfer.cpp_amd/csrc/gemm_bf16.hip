@@ -1210,6 +1210,218 @@ static int launch_skinny_copied(const bf16_t* A, const bf16_t* W, void* out, int
 
 static int g_use_pipelined = 1;
 // 1: the pipelined tiled kernel for M > 64 (default); 0: the plain tiled kernel (for comparison)
+// ---------------------------------------------------------------------------------------------
+// 17 to 64 rows: 16x16x32 MFMAs fed straight from memory.  A workgroup takes 16 rows of W (16
+// output columns; SwiGLU: 8 gate and 8 up rows) and a range of K; its four wavefronts take the
+// 64-wide k-blocks of that range in turn, each block as MB + 1 pairs of 16-byte loads per lane
+// (lane -> row lane % 16, 8 k at 8 (lane / 16), first and second half of the block) and 2 MB
+// MFMAs over all 16 MB rows of A.  The four wavefronts' sums meet in LDS, in the order 0..3.
+// With a weight of few rows the launch would fill a fraction of the compute units and every
+// workgroup would pull in all of A: then K is split over KS workgroups, which leave their sums
+// in `partial` [KS][M][N], and gemm_partials_add_kernel adds them to the residual in the order
+// 0..KS-1.  A row's bits do not depend on the other rows.
+#define MBK_STRIDE 20   // floats per row of the LDS tile: the 4 x 16 lanes of a store hit 64 banks
+
+template <int MB, int EPI>
+__global__ void __launch_bounds__(256)
+gemm_mblocks_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_,
+                    float* __restrict__ partial, int M, int N, int K, long lda) {
+  constexpr bool SW = (EPI == TI_EPI_SWIGLU);
+  constexpr int TILE = SW ? 8 : 16;                          // output columns of a workgroup
+  __shared__ __attribute__((aligned(16))) float red[4][MB * 16][MBK_STRIDE];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * TILE;
+  const int KS = gridDim.y, split = blockIdx.y;
+  const int nb = K / 64;
+  const int kb0 = (int)((long)nb * split / KS), kb1 = (int)((long)nb * (split + 1) / KS);
+
+  // rows outside the matrices read a valid row; what they give is not stored
+  const bf16_t* arow[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) arow[mb] = A + (size_t)min(mb * 16 + r, M - 1) * lda + g * 8;
+  int wr;
+  if (SW) wr = (r < 8) ? min(n0 + r, N - 1) : N + min(n0 + r - 8, N - 1);
+  else wr = min(n0 + r, N - 1);
+  const bf16_t* wrow = W + (size_t)wr * K + g * 8;
+
+  struct Block { uint4 a[MB][2]; uint4 b[2]; };
+  auto load = [&](Block& f, int kb) {
+    const int k = kb * 64;
+    f.b[0] = *reinterpret_cast<const uint4*>(wrow + k);
+    f.b[1] = *reinterpret_cast<const uint4*>(wrow + k + 32);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      f.a[mb][0] = *reinterpret_cast<const uint4*>(arow[mb] + k);
+      f.a[mb][1] = *reinterpret_cast<const uint4*>(arow[mb] + k + 32);
+    }
+  };
+  floatx4 acc[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) acc[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+  int kb = kb0 + wave;
+  if (kb < kb1) {
+    Block cur;
+    load(cur, kb);
+    while (kb < kb1) {
+      // the next block is asked for before this one is multiplied (after the last one, the last again)
+      Block next;
+      load(next, min(kb + 4, kb1 - 1));
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, cur.a[mb][h]),
+                                                            __builtin_bit_cast(bf16x8, cur.b[h]), acc[mb], 0, 0, 0);
+      cur = next;
+      kb += 4;
+    }
+  }
+  // acc[mb][q]: row 16 mb + 4 g + q, column r
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) red[wave][mb * 16 + 4 * g + q][r] = acc[mb][q];
+  __syncthreads();
+  if (SW) {
+    // thread -> a row and 4 of the 8 columns: gate in columns 0..7 of the tile, up in 8..15
+    const int row = tid >> 1, c = (tid & 1) * 4;
+    if (row >= MB * 16 || row >= M) return;
+    float gt[4] = {0.f, 0.f, 0.f, 0.f}, up[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        gt[i] += red[w][row][c + i];
+        up[i] += red[w][row][8 + c + i];
+      }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n0 + c + i < N) ((bf16_t*)out_)[(size_t)row * N + n0 + c + i] = f2bf(silu_mul(gt[i], up[i]));
+    return;
+  }
+  const int row = tid >> 2, c = (tid & 3) * 4;
+  if (row >= MB * 16 || row >= M) return;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int w = 0; w < 4; ++w)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] += red[w][row][c + i];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = n0 + c + i;
+    if (n >= N) continue;
+    const size_t o = (size_t)row * N + n;
+    if (EPI == TI_EPI_ADD_F32 && KS > 1) partial[(size_t)split * M * N + o] = v[i];
+    else if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] += v[i];
+    else if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = v[i];
+    else ((bf16_t*)out_)[o] = f2bf(v[i]);
+  }
+}
+
+// out[i] += partial[0][i] + ... + partial[KS - 1][i], in that order
+__global__ void __launch_bounds__(256)
+gemm_partials_add_kernel(float* __restrict__ out, const float* __restrict__ partial, int KS, size_t count) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  float v = out[i];
+  for (int s = 0; s < KS; ++s) v += partial[(size_t)s * count + i];
+  out[i] = v;
+}
+
+static int g_mblocks = 1;        // a hook for measurements: 0 leaves 17..64 rows to the kernels without MFMA
+extern "C" void ti_gemm_bf16_mblocks_on(int on) { g_mblocks = on; }
+
+template <int EPI>
+static void launch_mblocks(const bf16_t* a, const bf16_t* w, void* out, float* partial, int M, int N, int K,
+                           long lda, int KS, hipStream_t s) {
+  const int tile = (EPI == TI_EPI_SWIGLU) ? 8 : 16;
+  dim3 grid((N + tile - 1) / tile, KS);
+  const int mb = (M + 15) / 16;
+  if (mb == 1) gemm_mblocks_kernel<1, EPI><<<grid, 256, 0, s>>>(a, w, out, partial, M, N, K, lda);
+  else if (mb == 2) gemm_mblocks_kernel<2, EPI><<<grid, 256, 0, s>>>(a, w, out, partial, M, N, K, lda);
+  else if (mb == 3) gemm_mblocks_kernel<3, EPI><<<grid, 256, 0, s>>>(a, w, out, partial, M, N, K, lda);
+  else gemm_mblocks_kernel<4, EPI><<<grid, 256, 0, s>>>(a, w, out, partial, M, N, K, lda);
+}
+
+// out[i] += partial[0][i] + ... + partial[KS - 1][i] for count elements: what a product with a split
+// K leaves to do (see ti_gemm_bf16_mblocks)
+extern "C" int ti_gemm_bf16_partials_add(float* out, const float* partial, int KS, long count, hipStream_t stream) {
+  TI_REQUIRE(KS >= 1 && count >= 0, "gemm_bf16_partials_add: bad sizes KS=%d count=%ld", KS, count);
+  if (count == 0) return 0;
+  gemm_partials_add_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(out, partial, KS, (size_t)count);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// The product for 17..64 rows that adds into the 32-bit residual, where the weight has so few rows
+// that K is split over workgroups (see gemm_mblocks_kernel; measured against the kernels without
+// MFMA at 64 rows: 1024 x 3072 19.7 -> 9.7 us with the addition of the partial sums as a kernel of
+// its own, ~5.5 us without; with more columns, or another epilogue, it gains nothing and returns 3).
+// partial: workspace of partial_bytes.  defer = 0: the partial sums are added to `out` here, and
+// only products large enough to gain with that are served.  defer = 1: they are left in `partial`,
+// *splits gets their number, and the caller sees to the addition (ti_gemm_bf16_partials_add, or a
+// kernel that reads the residual next and adds them on the way).  defer = 2: what defer = 1
+// serves, added here (the same bits).  Returns 3 for what it does not serve.
+extern "C" int ti_gemm_bf16_mblocks(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
+                                    void* partial, long partial_bytes, int defer, int* splits, hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K, "gemm_bf16_mblocks: bad sizes M=%d N=%d K=%d lda=%ld", M, N, K, lda);
+  TI_REQUIRE(splits != nullptr, "gemm_bf16_mblocks: splits must point to an int");
+  *splits = 0;
+  int KS = 1;
+  if (g_mblocks && epi == TI_EPI_ADD_F32 && partial && M > 16 && M <= 64 && K % 64 == 0 && lda % 8 == 0 &&
+      !((uintptr_t)A & 15) && !((uintptr_t)W & 15) && !((uintptr_t)partial & 15)) {
+    // split K until the launch has about a workgroup per compute unit
+    const int tiles = (N + 15) / 16, nb = K / 64;
+    while (KS < 8 && tiles * KS * 2 <= 256 && nb / (KS * 2) >= 4) KS *= 2;
+    if ((long)KS * M * N * 4 > partial_bytes) KS = 1;
+    // with the addition as a kernel of its own, only large products gain
+    if (!defer && !((long)M * K >= 128 * 1024 || (K >= 3072 && (long)M * K >= 96 * 1024))) KS = 1;
+  }
+  if (KS == 1) {
+    ti_set_error("gemm_bf16_mblocks: serves 17..64 rows added into few columns, K a multiple of 64");
+    return 3;
+  }
+  launch_mblocks<TI_EPI_ADD_F32>((const bf16_t*)A, (const bf16_t*)W, out, (float*)partial, M, N, K, lda, KS, stream);
+  if (defer == 1) {
+    *splits = KS;
+  } else {
+    const size_t count = (size_t)M * N;
+    gemm_partials_add_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>((float*)out, (const float*)partial,
+                                                                                KS, count);
+  }
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// hooks for tests of the kernel alone: any epilogue, K split `ks` ways (1: not split; partial sums
+// are added here)
+extern "C" int ti_gemm_bf16_mblocks_any(const void* A, const void* W, void* out, int M, int N, int K, long lda,
+                                        int epi, void* partial, int ks, hipStream_t stream) {
+  TI_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0 && K % 64 == 0 && lda >= K && lda % 8 == 0 && ks >= 1 && ks <= K / 64,
+             "gemm_bf16_mblocks_any: bad sizes M=%d N=%d K=%d lda=%ld ks=%d", M, N, K, lda, ks);
+  TI_REQUIRE(ks == 1 || (epi == TI_EPI_ADD_F32 && partial), "gemm_bf16_mblocks_any: a split K needs the adding epilogue");
+  const bf16_t* a = (const bf16_t*)A;
+  const bf16_t* w = (const bf16_t*)W;
+  switch (epi) {
+    case TI_EPI_STORE_F32: launch_mblocks<TI_EPI_STORE_F32>(a, w, out, nullptr, M, N, K, lda, 1, stream); break;
+    case TI_EPI_STORE_ACT: launch_mblocks<TI_EPI_STORE_ACT>(a, w, out, nullptr, M, N, K, lda, 1, stream); break;
+    case TI_EPI_SWIGLU: launch_mblocks<TI_EPI_SWIGLU>(a, w, out, nullptr, M, N, K, lda, 1, stream); break;
+    case TI_EPI_ADD_F32:
+      launch_mblocks<TI_EPI_ADD_F32>(a, w, out, (float*)partial, M, N, K, lda, ks, stream);
+      if (ks > 1) {
+        const size_t count = (size_t)M * N;
+        gemm_partials_add_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>((float*)out, (const float*)partial,
+                                                                                    ks, count);
+      }
+      break;
+    default:
+      TI_REQUIRE(false, "gemm_bf16_mblocks_any: unknown epilogue %d", epi);
+  }
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
 extern "C" void ti_gemm_bf16_use_pipelined(int on) { g_use_pipelined = on; }
 
 // N: output columns (SwiGLU: F, with W holding 2F rows).  Returns 3 for a shape

@@ -25,6 +25,10 @@ int ti_embed(int dtype, const void* table, const int* tok, float* x, int M, int 
 // out[r] = rmsnorm(x[rows ? rows[r] : r]) * w, in `out_dtype`
 int ti_rmsnorm(int out_dtype, const float* x, const float* w, const int* rows, void* out, int n_rows, int H, float eps,
                hipStream_t stream);
+// x[r] += partial[0][r] + ... + partial[KS - 1][r] (partial: [KS][n_rows][H], what a product with a
+// split K left), written back, then the same norm of the new x.  Returns 3 for what it does not serve.
+int ti_rmsnorm_add_partials(int out_dtype, float* x, const float* partial, int KS, const float* w, void* out,
+                            int n_rows, int H, float eps, hipStream_t stream);
 // half-split rotation in place on f32 [M, heads, hd] (rows `row_stride` floats apart)
 int ti_rope_neox(float* x, const int* pos, const float* inv_freq, int M, int heads, int hd, long row_stride,
                  hipStream_t stream);
@@ -46,6 +50,18 @@ int ti_gemm_generic(int dtype, const void* A, const void* W, void* out, int M, i
 
 // ---- libti_gemm_bf16: the same on the matrix cores (K a multiple of 8)
 int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi, hipStream_t stream);
+// The adding product for 17..64 rows and a weight of few rows: MFMAs fed straight from memory, K
+// split over workgroups whose sums go through `partial` (workspace of partial_bytes).  defer = 0:
+// they are added to out here (served: products large enough to gain even so); defer = 1: they stay
+// in partial [*splits][M][N] and the caller adds them (ti_gemm_bf16_partials_add, or
+// ti_rmsnorm_add_partials on the way to the next norm); defer = 2: as 1, but added here.
+// Returns 3 for what it does not serve.
+int ti_gemm_bf16_mblocks(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
+                         void* partial, long partial_bytes, int defer, int* splits, hipStream_t stream);
+int ti_gemm_bf16_partials_add(float* out, const float* partial, int KS, long count, hipStream_t stream);
+// the kernel of ti_gemm_bf16_mblocks alone, for tests: any epilogue, 1..64 rows, K split ks ways
+int ti_gemm_bf16_mblocks_any(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
+                             void* partial, int ks, hipStream_t stream);
 // out (op)= rmsnorm(x; nw, eps) W^T for M <= 16, K a multiple of 64
 int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, const void* W, void* out, int M, int N, int K, int epi,
                         hipStream_t stream);
@@ -57,6 +73,7 @@ int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K, long lda, 
 // switches for measurements and tests (0 restores the choice by shape)
 void ti_gemm_bf16_force_tile(int which);      // 1: 256 x 128, 3: 128 x 64, 6: 64 x 64
 void ti_gemm_bf16_skinny_waves(int waves);    // 4 or 8 wavefronts in the kernel for M <= 64
+void ti_gemm_bf16_mblocks_on(int on);         // 0: ti_gemm_bf16_mblocks serves nothing
 void ti_gemm_bf16_use_pipelined(int on);      // 0: the plain tiled kernel for every K
 void ti_gemm_bf16_row_per_wave(int on);        // 0: few tokens and a weight of few rows take the 16-row kernels too
 void ti_gemm_bf16_skinny_copy(int on);        // 0: up to 16 tokens, fragments of the token rows straight from memory

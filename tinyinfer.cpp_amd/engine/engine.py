@@ -408,6 +408,7 @@ class Engine:
             ctx.run = r
             model.blocks[li].forward(ctx, x)
         if ctx.out_rows is None:
+            self.ops.flush()
             return None
         h = model.final_norm.forward(ctx, x, rows=ctx.out_rows)
         return model.head.forward(ctx, h)

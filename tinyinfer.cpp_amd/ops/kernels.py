@@ -70,6 +70,10 @@ class Ops:
         self.use_fused_norm = True       # the norm before a product inside the product's kernel (few tokens)
         self.use_fused_qk_decode = True  # per-head norm, rotation and cache write inside the decode attention
         self.use_fused_qkv_prefill = True  # the same in the epilogue of the q/k/v product (steps of many tokens)
+        self.use_mfma_rows = True          # 17..64 rows: the product by MFMAs fed from memory
+        self.use_deferred_add = True       # ... and its partial sums added by the norm that comes next
+        self._partials = None
+        self._pending = None               # (residual, splits): partial sums not yet added
         self.use_paired_prefill = True   # small prefill launches: a heavy and a light tile per workgroup
 
     # ------------------------------------------------------------------ loading
@@ -99,14 +103,35 @@ class Ops:
         if rc != 0:
             raise KernelError(f"{what}: {lib.ti_last_error().decode()}")
 
-    @staticmethod
-    def _stream():
+    def _stream(self):
         """The current stream's handle.  Every launch asks for it; torch's raw accessor, where this
         build of torch has it, answers in well under a microsecond (the public one builds a
-        Stream object: ~8 us a call)."""
+        Stream object: ~8 us a call).  Partial sums that a product left for later (see `flush`)
+        are added first: whatever is launched next finds the residual complete."""
+        if self._pending is not None:
+            self.flush()
+        return self._raw_stream()
+
+    @staticmethod
+    def _raw_stream():
         if _RAW_STREAM is not None:
             return ctypes.c_void_p(_RAW_STREAM(torch.cuda.current_device()))
         return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def flush(self):
+        """A product into the residual whose K was split over workgroups (17..64 rows, few
+        columns) may leave its partial sums in a workspace, for the norm that reads the residual
+        next to add on its way (`linear(..., may_defer=True)`).  Every other launch through this
+        object adds them first, with a kernel of their own, in the same order: the same bits.
+        Code that reads such a residual without going through this object calls `flush` itself."""
+        pend, self._pending = self._pending, None
+        if pend is None:
+            return
+        out, ks = pend
+        lib = self.lib("gemm_bf16")
+        rc = lib.ti_gemm_bf16_partials_add(_ptr(out), _ptr(self._partials), ks, ctypes.c_long(out.numel()),
+                                           self._raw_stream())
+        self._check(lib, rc, "linear(bf16): adding the partial sums")
 
     @staticmethod
     def _dev(*ts):
@@ -138,6 +163,16 @@ class Ops:
         if rows is not None and rows.dtype != torch.int32:
             raise KernelError("rmsnorm: rows must be int32")
         lib = self.lib("core")
+        pend = self._pending
+        if pend is not None and rows is None and pend[0].data_ptr() == x.data_ptr() and pend[0].shape == x.shape:
+            # the product before left its partial sums: this norm adds them on its way
+            rc = lib.ti_rmsnorm_add_partials(_code(out.dtype), _ptr(x), _ptr(self._partials), pend[1], _ptr(w),
+                                             _ptr(out), n, H, ctypes.c_float(eps), self._raw_stream())
+            if rc == 0:
+                self._pending = None
+                return
+            if rc != 3:
+                self._check(lib, rc, "rmsnorm")
         rc = lib.ti_rmsnorm(_code(out.dtype), _ptr(x), _ptr(w), _ptr(rows), _ptr(out), n, H,
                             ctypes.c_float(eps), self._stream())
         self._check(lib, rc, "rmsnorm")
@@ -214,10 +249,11 @@ class Ops:
         self._check(lib, rc, "qk_norm_inplace")
 
     # ---------------------------------------------------------- matrix products
-    def linear(self, a, w, out, epilogue: str):
+    def linear(self, a, w, out, epilogue: str, may_defer: bool = False):
         """out (op)= a w^T.  a: T [M, K] (rows may be strided); w: T [N, K] contiguous.
         epilogue: "store" f32 out = ; "add" f32 out += ; "store_act" T out = ;
-        "swiglu": w is [2F, K] = [gate; up], T out [M, F] = silu(gate) * up."""
+        "swiglu": w is [2F, K] = [gate; up], T out [M, F] = silu(gate) * up.
+        may_defer (with "add"): the caller reads `out` next through this object (see `flush`)."""
         epi = EPI[epilogue]
         if isinstance(a, NormedRows):
             if self._linear_normed(a, w, out, epilogue):
@@ -237,7 +273,7 @@ class Ops:
         if M == 0:
             return
         code = _code(a.dtype)
-        if code == BF16 and self.use_fast_gemm and self._linear_bf16(a, w, out, epi, M, N, K):
+        if code == BF16 and self.use_fast_gemm and self._linear_bf16(a, w, out, epi, M, N, K, may_defer):
             return
         lib = self.lib("gemm_generic")
         rc = lib.ti_gemm_generic(code, _ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi,
@@ -287,6 +323,7 @@ class Ops:
         return True
 
     NORMED_MAX_ROWS = 16
+    PARTIALS_BYTES = 1 << 20
 
     def can_fuse_norm(self, n_rows: int, dtype: torch.dtype) -> bool:
         """Whether `linear` has a kernel that takes the norm of this many rows in."""
@@ -317,11 +354,29 @@ class Ops:
         self._check(lib, rc, "linear(normed)")
         return True
 
-    def _linear_bf16(self, a, w, out, epi, M, N, K) -> bool:
+    def _linear_bf16(self, a, w, out, epi, M, N, K, may_defer=False) -> bool:
         """The MFMA kernels; False if they refuse the shape (the generic kernel takes it)."""
         if K % 8 or a.stride(0) % 8 or a.data_ptr() % 16 or w.data_ptr() % 16:
             return False
         lib = self.lib("gemm_bf16")
+        if 16 < M <= 64 and epi == EPI["add"] and self.use_mfma_rows:
+            # MFMAs fed from memory, K split over workgroups; their sums go through a workspace
+            stream = self._stream()
+            ws = self._partials
+            if ws is None or ws.device != a.device:
+                ws = self._partials = torch.empty(self.PARTIALS_BYTES // 4, dtype=torch.float32, device=a.device)
+            # 1: the sums are left for the next norm; 2: the same product, added at once
+            defer = 0 if not may_defer else 1 if self.use_deferred_add else 2
+            splits = ctypes.c_int(0)
+            rc = lib.ti_gemm_bf16_mblocks(_ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi,
+                                          _ptr(ws), ctypes.c_long(self.PARTIALS_BYTES), defer,
+                                          ctypes.byref(splits), stream)
+            if rc == 0:
+                if splits.value:
+                    self._pending = (out, splits.value)
+                return True
+            if rc != 3:
+                self._check(lib, rc, "linear(bf16, 17..64 rows)")
         rc = lib.ti_gemm_bf16(_ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi, self._stream())
         if rc == 3:          # "shape not served": not an error
             return False

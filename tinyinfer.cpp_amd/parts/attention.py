@@ -96,7 +96,7 @@ class Attention(Part):
                 0 if self.shares_kv else self.kv_heads, self.head_dim):
             # a step of many tokens: the projection's epilogue prepared q and wrote the cache
             ctx.ops.attention(ctx, view, q, pool, a, self.heads, self.kv_heads, self.head_dim, self.scale, self.window)
-            ctx.ops.linear(a, self.w_o, x, "add")
+            ctx.ops.linear(a, self.w_o, x, "add", may_defer=True)
             return
         qkv = ctx.buf("attn.qkv", (M, width), ctx.f32)
         ctx.ops.linear(h, self.w_qkv, qkv, "store")
@@ -104,7 +104,8 @@ class Attention(Part):
                 ctx, view, qkv, self.q_norm_w, self.k_norm_w, self.eps,
                 None if rot is None else rot["inv_freq"], None if rot is None else rot.get("table"),
                 pool, not self.shares_kv, a, self.heads, self.kv_heads, self.head_dim, self.scale, self.window):
-            ctx.ops.linear(a, self.w_o, x, "add")        # a step of single tokens: one kernel did it all
+            # a step of single tokens: one kernel did it all
+            ctx.ops.linear(a, self.w_o, x, "add", may_defer=True)
             return
         q_w, k_w = self.q_norm_w, self.k_norm_w
         if self.pos is not None and rot is None:
@@ -125,7 +126,7 @@ class Attention(Part):
             None if rot is None else rot.get("table"))
         ctx.ops.attention(ctx, view, q, pool, a, self.heads, self.kv_heads, self.head_dim,
                           self.scale, self.window)
-        ctx.ops.linear(a, self.w_o, x, "add")
+        ctx.ops.linear(a, self.w_o, x, "add", may_defer=True)
 
 
 register_part("mixer", "attention", Attention)

@@ -3,6 +3,9 @@
 `pre_norm`: x += mixer(norm1(x)); x += ffn(norm2(x))
 (/root/reference/src/inference.cu:35-66).  The mixer and the feed-forward add
 into x themselves, so the residual sum happens in 32-bit in their last kernel.
+The framework's own mixers and feed-forwards let that kernel leave part of the sum
+to the norm that reads x next (`ops.linear(..., may_defer=True)`); a part that reads
+x other than through `ctx.ops` calls `ctx.ops.flush()` first.
 """
 from __future__ import annotations
 

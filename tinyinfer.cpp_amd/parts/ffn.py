@@ -40,7 +40,7 @@ class SwiGLU(Part):
         M = h.shape[0]
         y = ctx.buf("ffn.y", (M, self.intermediate), ctx.act_dtype)
         ctx.ops.linear(h, self.w_gate_up, y, "swiglu")
-        ctx.ops.linear(y, self.w_down, x, "add")
+        ctx.ops.linear(y, self.w_down, x, "add", may_defer=True)
 
 
 register_part("ffn", "swiglu", SwiGLU)
