@@ -546,7 +546,8 @@ def test_linear_bf16_mfma_fed_from_memory(ops, M, N, K, ks):
         assert (f64(sw) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
 
 
-@pytest.mark.parametrize("M,N,K", [(17, 1024, 2048), (64, 1024, 3072), (40, 512, 1024), (33, 96, 1024)])
+@pytest.mark.parametrize("M,N,K", [(17, 1024, 2048), (64, 1024, 3072), (40, 512, 1024), (33, 96, 1024),
+                                   (20, 2048, 1024), (24, 256, 2048)])
 def test_partial_sums_left_to_the_next_norm(ops, M, N, K):
     """A product into the residual at 17..64 rows with few columns splits K over workgroups.
     With `may_defer` its partial sums wait for whatever reads the residual next: the norm adds
@@ -597,6 +598,35 @@ def test_partial_sums_left_to_the_next_norm(ops, M, N, K):
         assert (x - want_x).abs().max() < 2e-5 * K
     finally:
         ops.use_mfma_rows = True
+
+
+@pytest.mark.parametrize("rows,H,KS", [(5, 2304, 3), (3, 1028, 5), (9, 64, 1), (2, 1024, 4), (70, 1536, 2)])
+def test_rmsnorm_that_adds_partial_sums(ops, rows, H, KS):
+    """The norm that first adds KS partial sums to its rows, alone, at widths and counts that the
+    products of the engine do not produce: the rows afterwards are x + p0 + ... in that order
+    (bit for bit), and the output is the norm of them, in the bits of the plain norm kernel."""
+    import ctypes
+    g = torch.Generator().manual_seed(rows + H + KS)
+    x0 = torch.randn(rows, H, generator=g)
+    parts = torch.randn(KS, rows, H, generator=g)
+    w = dev(torch.rand(H, generator=g) + 0.5)
+    want_x = x0.clone()
+    for s in range(KS):
+        want_x += parts[s]
+    lib = ops.lib("core")
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+    for dtype, code in ((torch.float32, 0), (torch.bfloat16, 1)):
+        x = dev(x0.clone())
+        out = torch.empty(rows, H, device="cuda", dtype=dtype)
+        rc = lib.ti_rmsnorm_add_partials(code, ptr(x), ptr(dev(parts)), KS, ptr(w), ptr(out), rows, H,
+                                         ctypes.c_float(1e-6), None)
+        assert rc == 0, lib.ti_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(x.cpu(), want_x)
+        plain = torch.empty_like(out)
+        ops.rmsnorm(x, w, 1e-6, plain)
+        assert torch.equal(out, plain)
+        assert (f64(out) - ref_rmsnorm(want_x, w, 1e-6)).abs().max() < (1e-5 if dtype == torch.float32 else 0.03)
 
 
 @pytest.mark.parametrize("tile", [1, 3, 6])

@@ -106,7 +106,10 @@ extern "C" int ti_rmsnorm(int out_dtype, const float* x, const float* w, const i
 // The norm of rows whose last product left its sums of a split K in `partial` [KS][n_rows][H]:
 // x[r] += partial[0][r] + ... + partial[KS - 1][r] (in that order, written back), then the norm of
 // rmsnorm_wave_kernel over the new x.  A wavefront per row, four rows a workgroup.
-template <typename T>
+// KS_T: the number of partial sums if known when compiled (their loads then do not wait for one
+// another), 0: KS.  PIECES: 16-byte pieces of a row a lane keeps in registers between the sum and
+// the scaling (rows up to 1024 PIECES wide), 0: it reads them again.
+template <typename T, int KS_T, int PIECES>
 __global__ void __launch_bounds__(256)
 rmsnorm_add_partials_kernel(float* __restrict__ x, const float* __restrict__ partial, int KS,
                             const float* __restrict__ w, T* __restrict__ out, int n_rows, int H, float eps) {
@@ -114,29 +117,86 @@ rmsnorm_add_partials_kernel(float* __restrict__ x, const float* __restrict__ par
   if (r >= n_rows) return;
   float* src = x + (size_t)r * H;
   const size_t count = (size_t)n_rows * H;
-  float ss = 0.f;
-  for (int k = lane * 4; k < H; k += 256) {
+  const float* prow = partial + (size_t)r * H;
+  if (KS_T) KS = KS_T;
+  auto summed = [&](int k) {
     float4 v = *reinterpret_cast<const float4*>(src + k);
-    for (int s = 0; s < KS; ++s) {
-      const float4 p = *reinterpret_cast<const float4*>(partial + s * count + (size_t)r * H + k);
-      v.x += p.x;
-      v.y += p.y;
-      v.z += p.z;
-      v.w += p.w;
+    if (KS_T) {
+      float4 p[KS_T ? KS_T : 1];
+#pragma unroll
+      for (int s = 0; s < KS_T; ++s) p[s] = *reinterpret_cast<const float4*>(prow + s * count + k);
+#pragma unroll
+      for (int s = 0; s < KS_T; ++s) {
+        v.x += p[s].x;
+        v.y += p[s].y;
+        v.z += p[s].z;
+        v.w += p[s].w;
+      }
+    } else {
+      for (int s = 0; s < KS; ++s) {
+        const float4 p = *reinterpret_cast<const float4*>(prow + s * count + k);
+        v.x += p.x;
+        v.y += p.y;
+        v.z += p.z;
+        v.w += p.w;
+      }
     }
-    *reinterpret_cast<float4*>(src + k) = v;
-    ss = rms_accumulate(ss, v);
-  }
-  const float scale = rms_scale(ss, H, eps);
-  T* dst = out + (size_t)r * H;
-  for (int k = lane * 4; k < H; k += 256) {
-    const float4 v = *reinterpret_cast<const float4*>(src + k);     // this lane's own store above
+    return v;
+  };
+  auto scaled = [&](int k, float4 v, float scale) {
     const float4 g = *reinterpret_cast<const float4*>(w + k);
+    T* dst = out + (size_t)r * H;
     st<T>(dst + k, v.x * scale * g.x);
     st<T>(dst + k + 1, v.y * scale * g.y);
     st<T>(dst + k + 2, v.z * scale * g.z);
     st<T>(dst + k + 3, v.w * scale * g.w);
+  };
+  float ss = 0.f;
+  if (PIECES) {
+    float4 v[PIECES ? PIECES : 1];
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int k = lane * 4 + i * 256;
+      if (k < H) v[i] = summed(k);
+    }
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int k = lane * 4 + i * 256;
+      if (k < H) {
+        *reinterpret_cast<float4*>(src + k) = v[i];
+        ss = rms_accumulate(ss, v[i]);
+      }
+    }
+    const float scale = rms_scale(ss, H, eps);
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int k = lane * 4 + i * 256;
+      if (k < H) scaled(k, v[i], scale);
+    }
+    return;
   }
+  for (int k = lane * 4; k < H; k += 256) {
+    const float4 v = summed(k);
+    *reinterpret_cast<float4*>(src + k) = v;
+    ss = rms_accumulate(ss, v);
+  }
+  const float scale = rms_scale(ss, H, eps);
+  for (int k = lane * 4; k < H; k += 256)
+    scaled(k, *reinterpret_cast<const float4*>(src + k), scale);     // this lane's own store above
+}
+
+template <typename T>
+static void launch_rmsnorm_add_partials(float* x, const float* partial, int KS, const float* w, T* out, int n_rows,
+                                        int H, float eps, hipStream_t stream) {
+  const int grid = (n_rows + 3) / 4;
+#define TI_GO(KS_T, PIECES) \
+  rmsnorm_add_partials_kernel<T, KS_T, PIECES><<<grid, 256, 0, stream>>>(x, partial, KS, w, out, n_rows, H, eps)
+  if (H <= 1024 && KS == 4) TI_GO(4, 4);
+  else if (H <= 1024 && KS == 2) TI_GO(2, 4);
+  else if (H <= 1024 && KS == 8) TI_GO(8, 4);
+  else if (H <= 2048) TI_GO(0, 8);
+  else TI_GO(0, 0);
+#undef TI_GO
 }
 
 // Returns 3 for a width or an alignment it does not serve (the caller adds the partial sums with
@@ -150,11 +210,10 @@ extern "C" int ti_rmsnorm_add_partials(int out_dtype, float* x, const float* par
     return 3;
   }
   if (n_rows == 0) return 0;
-  const int grid = (n_rows + 3) / 4;
   if (out_dtype == TI_F32)
-    rmsnorm_add_partials_kernel<float><<<grid, 256, 0, stream>>>(x, partial, KS, w, (float*)out, n_rows, H, eps);
+    launch_rmsnorm_add_partials<float>(x, partial, KS, w, (float*)out, n_rows, H, eps, stream);
   else
-    rmsnorm_add_partials_kernel<bf16_t><<<grid, 256, 0, stream>>>(x, partial, KS, w, (bf16_t*)out, n_rows, H, eps);
+    launch_rmsnorm_add_partials<bf16_t>(x, partial, KS, w, (bf16_t*)out, n_rows, H, eps, stream);
   TI_LAUNCH_CHECK();
   return 0;
 }
