@@ -696,7 +696,7 @@ __device__ __forceinline__ void qkv_rows_by_lanes(const QKVEpilogue& ep, float* 
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
-gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_,
+gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_arg,
                       int M, int N, int K, long lda, QKVEpilogue ep = QKVEpilogue{}) {
   constexpr bool SW = (EPI == TI_EPI_SWIGLU);
   constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
@@ -709,6 +709,11 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
   constexpr int LOADS = (GROUPS_A + GROUPS_B) / NWV;         // per wavefront and k-tile
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
+  // gridDim.z > 1 (storing epilogue only): K is split; workgroup z takes its share of the k-tiles and
+  // stores its sums into the z-th [M, N] of out
+  const int kt0 = (int)((long)(K / PBK) * blockIdx.z / gridDim.z);
+  const int n_k = (int)((long)(K / PBK) * (blockIdx.z + 1) / gridDim.z) - kt0;
+  void* __restrict__ out_ = (EPI == TI_EPI_STORE_F32) ? (void*)((float*)out_arg + (size_t)blockIdx.z * M * N) : out_arg;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int m0 = blockIdx.y * BM;
@@ -744,7 +749,7 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
 
   auto issue = [&](int kt) {
     unsigned char* stage = smem + (kt % PSTAGES) * STAGE_BYTES;
-    const int k0 = kt * PBK;
+    const int k0 = (kt0 + kt) * PBK;
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int g = wave + NWV * i;
@@ -782,7 +787,6 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
   // the residual an adding epilogue adds to: asked for while the last k-tile is multiplied
   // (elements outside the matrix read a valid one and are not stored)
   float prev[EPI == TI_EPI_ADD_F32 ? TM : 1][EPI == TI_EPI_ADD_F32 ? TN : 1][16];
-  const int n_k = K / PBK;
   issue(0);
   if (n_k > 1) issue(1);
   for (int kt = 0; kt < n_k; ++kt) {
@@ -853,7 +857,7 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
     // lanes finish a row of a q or k head (the arithmetic of the kernel that prepares whole steps; a
     // row's eight lanes read its angles and write its result as runs of consecutive bytes), and a
     // thread a dim of a v head.
-    static_assert(BM == 256 && NWV == 8, "the first four wavefronts look up a row each; 64 rows per pass of all eight");
+    static_assert((BM == 256 || BM == 128) && NWV == 8, "the first wavefronts look up a row each; 64 rows per pass of all eight");
     constexpr int FS = BN + 8;                              // row stride: the eight rows x eight lanes of a wavefront
                                                             // read 64 different banks
     static_assert(BM * FS * 4 + 4 * BM * 4 <= PSTAGES * (BM + BN) * PBK * 2, "the 32-bit tile fits into the stages");
@@ -953,7 +957,7 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
 static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
-                            hipStream_t s) {
+                            hipStream_t s, int ksplit = 1) {
   constexpr int bytes = PSTAGES * (BM + BN) * PBK * 2;
   auto kernel = gemm_pipelined_kernel<BM, BN, WAVES_M, WAVES_N, EPI>;
   static bool ready = false;          // per instantiation: allow more than 64 KiB of dynamic LDS
@@ -965,8 +969,41 @@ static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, 
     ready = true;
   }
   const int bn = (EPI == TI_EPI_SWIGLU) ? BN / 2 : BN;
-  dim3 grid((N + bn - 1) / bn, (M + BM - 1) / BM);
+  dim3 grid((N + bn - 1) / bn, (M + BM - 1) / BM, (EPI == TI_EPI_STORE_F32) ? ksplit : 1);
   kernel<<<grid, WAVES_M * WAVES_N * 64, bytes, s>>>(A, W, out, M, N, K, lda, QKVEpilogue{});
+  return 0;
+}
+
+static int g_qkv_rows = 0;       // a hook for measurements: 128 or 256 forces the tile's rows
+extern "C" void ti_gemm_bf16_qkv_prep_rows(int rows) { g_qkv_rows = rows; }
+
+static int compute_units() {
+  static int n = 0;
+  if (!n) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
+    if (n <= 0) n = 256;
+  }
+  return n;
+}
+
+template <int BM, int WAVES_M, int WAVES_N>
+static int launch_qkv_prep(const void* A, const void* W, int M, int N, int K, long lda, const QKVEpilogue& ep,
+                           hipStream_t stream) {
+  constexpr int BN = 128;
+  constexpr int bytes = PSTAGES * (BM + BN) * PBK * 2;
+  auto kernel = gemm_pipelined_kernel<BM, BN, WAVES_M, WAVES_N, TI_EPI_QKV_PREP>;
+  static bool ready = false;
+  if (!ready) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+      ti_set_error("gemm_bf16_qkv_prep: cannot reserve %d bytes of LDS", bytes);
+      return 2;
+    }
+    ready = true;
+  }
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
+  kernel<<<grid, 512, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, nullptr, M, N, K, lda, ep);
   return 0;
 }
 
@@ -992,19 +1029,13 @@ extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K,
   QKVEpilogue ep{q_w, k_w, eps, inv_freq, (const float2*)rope_table, table_len, pos, slot, table, table_stride,
                  (bf16_t*)pool, (bf16_t*)q_out, n_head, n_kv, hd, page_size};
   const int N = (n_head + 2 * n_kv) * hd;
-  constexpr int BM = 256, BN = 128;
-  constexpr int bytes = PSTAGES * (BM + BN) * PBK * 2;
-  auto kernel = gemm_pipelined_kernel<BM, BN, 4, 2, TI_EPI_QKV_PREP>;
-  static bool ready = false;
-  if (!ready) {
-    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
-      ti_set_error("gemm_bf16_qkv_prep: cannot reserve %d bytes of LDS", bytes);
-      return 2;
-    }
-    ready = true;
-  }
-  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
-  kernel<<<grid, 512, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, nullptr, M, N, K, lda, ep);
+  // 128-row tiles while they make no more workgroups than there are compute units (1,024 rows of
+  // the 32 column tiles of Qwen3-0.6B), else 256-row tiles, which load less per flop
+  const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+  const bool rows128 = g_qkv_rows ? g_qkv_rows == 128 : tiles128 <= compute_units();
+  int rc_ = rows128 ? launch_qkv_prep<128, 2, 4>(A, W, M, N, K, lda, ep, stream)
+                    : launch_qkv_prep<256, 4, 2>(A, W, M, N, K, lda, ep, stream);
+  if (rc_) return rc_;
   TI_LAUNCH_CHECK();
   return 0;
 }
@@ -1354,35 +1385,46 @@ extern "C" int ti_gemm_bf16_partials_add(float* out, const float* partial, int K
   return 0;
 }
 
-// The product for 17..64 rows that adds into the 32-bit residual, where the weight has so few rows
-// that K is split over workgroups (see gemm_mblocks_kernel; measured against the kernels without
-// MFMA at 64 rows: 1024 x 3072 19.7 -> 9.7 us with the addition of the partial sums as a kernel of
-// its own, ~5.5 us without; with more columns, or another epilogue, it gains nothing and returns 3).
-// partial: workspace of partial_bytes.  defer = 0: the partial sums are added to `out` here, and
-// only products large enough to gain with that are served.  defer = 1: they are left in `partial`,
-// *splits gets their number, and the caller sees to the addition (ti_gemm_bf16_partials_add, or a
-// kernel that reads the residual next and adds them on the way).  defer = 2: what defer = 1
-// serves, added here (the same bits).  Returns 3 for what it does not serve.
+// The product that adds into the 32-bit residual, for steps of more than 16 rows whose launch would
+// leave most compute units idle (few rows times a weight of few rows): K is split over workgroups,
+// which leave their sums in `partial` [KS][M][N] (workspace of partial_bytes).  17..64 rows:
+// gemm_mblocks_kernel (measured against the kernels without MFMA at 64 rows: 1024 x 3072 19.7 ->
+// 9.7 us with the addition of the partial sums as a kernel of its own, ~6 us without).  More rows:
+// the pipelined kernel with 64 x 64 tiles, storing (136 rows: 18.5 -> ~8 us).
+// defer = 0: the partial sums are added to `out` here, and only what gains even so is served.
+// defer = 1: they are left in `partial`, *splits gets their number, and the caller sees to the
+// addition (ti_gemm_bf16_partials_add, or a kernel that reads the residual next and adds them on
+// the way).  defer = 2: what defer = 1 serves, added here (the same bits).  Returns 3 for what
+// it does not serve.
 extern "C" int ti_gemm_bf16_mblocks(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
                                     void* partial, long partial_bytes, int defer, int* splits, hipStream_t stream) {
   TI_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K, "gemm_bf16_mblocks: bad sizes M=%d N=%d K=%d lda=%ld", M, N, K, lda);
   TI_REQUIRE(splits != nullptr, "gemm_bf16_mblocks: splits must point to an int");
   *splits = 0;
   int KS = 1;
-  if (g_mblocks && epi == TI_EPI_ADD_F32 && partial && M > 16 && M <= 64 && K % 64 == 0 && lda % 8 == 0 &&
-      !((uintptr_t)A & 15) && !((uintptr_t)W & 15) && !((uintptr_t)partial & 15)) {
+  const bool small = M <= 64;
+  if (g_mblocks && epi == TI_EPI_ADD_F32 && partial && M > 16 && K % 64 == 0 && lda % 8 == 0 &&
+      !((uintptr_t)A & 15) && !((uintptr_t)W & 15) && !((uintptr_t)partial & 15) && (small || g_use_pipelined)) {
     // split K until the launch has about a workgroup per compute unit
-    const int tiles = (N + 15) / 16, nb = K / 64;
+    const long tiles = small ? (N + 15) / 16 : (long)((M + 63) / 64) * ((N + 63) / 64);
+    const int nb = K / 64;
     while (KS < 8 && tiles * KS * 2 <= 256 && nb / (KS * 2) >= 4) KS *= 2;
     if ((long)KS * M * N * 4 > partial_bytes) KS = 1;
     // with the addition as a kernel of its own, only large products gain
-    if (!defer && !((long)M * K >= 128 * 1024 || (K >= 3072 && (long)M * K >= 96 * 1024))) KS = 1;
+    if (!defer && small && !((long)M * K >= 128 * 1024 || (K >= 3072 && (long)M * K >= 96 * 1024))) KS = 1;
+    if (!defer && !small && KS < 4) KS = 1;
   }
   if (KS == 1) {
-    ti_set_error("gemm_bf16_mblocks: serves 17..64 rows added into few columns, K a multiple of 64");
+    ti_set_error("gemm_bf16_mblocks: serves more than 16 rows added into a product of few tiles, K a multiple of 64");
     return 3;
   }
-  launch_mblocks<TI_EPI_ADD_F32>((const bf16_t*)A, (const bf16_t*)W, out, (float*)partial, M, N, K, lda, KS, stream);
+  if (small) {
+    launch_mblocks<TI_EPI_ADD_F32>((const bf16_t*)A, (const bf16_t*)W, out, (float*)partial, M, N, K, lda, KS, stream);
+  } else {
+    int rc_ = launch_pipelined<64, 64, 2, 2, TI_EPI_STORE_F32>((const bf16_t*)A, (const bf16_t*)W, partial, M, N, K, lda,
+                                                               stream, KS);
+    if (rc_) return rc_;
+  }
   if (defer == 1) {
     *splits = KS;
   } else {

@@ -73,6 +73,7 @@ int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K, long lda, 
 // switches for measurements and tests (0 restores the choice by shape)
 void ti_gemm_bf16_force_tile(int which);      // 1: 256 x 128, 3: 128 x 64, 6: 64 x 64
 void ti_gemm_bf16_skinny_waves(int waves);    // 4 or 8 wavefronts in the kernel for M <= 64
+void ti_gemm_bf16_qkv_prep_rows(int rows);    // 128 / 256: the rows of ti_gemm_bf16_qkv_prep's tile; 0: by the shape
 void ti_gemm_bf16_mblocks_on(int on);         // 0: ti_gemm_bf16_mblocks serves nothing
 void ti_gemm_bf16_use_pipelined(int on);      // 0: the plain tiled kernel for every K
 void ti_gemm_bf16_row_per_wave(int on);        // 0: few tokens and a weight of few rows take the 16-row kernels too

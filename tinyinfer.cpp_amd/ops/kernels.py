@@ -70,7 +70,7 @@ class Ops:
         self.use_fused_norm = True       # the norm before a product inside the product's kernel (few tokens)
         self.use_fused_qk_decode = True  # per-head norm, rotation and cache write inside the decode attention
         self.use_fused_qkv_prefill = True  # the same in the epilogue of the q/k/v product (steps of many tokens)
-        self.use_mfma_rows = True          # 17..64 rows: the product by MFMAs fed from memory
+        self.use_mfma_rows = True          # products into the residual of few tiles: K split over workgroups
         self.use_deferred_add = True       # ... and its partial sums added by the norm that comes next
         self._partials = None
         self._pending = None               # (residual, splits): partial sums not yet added
@@ -323,7 +323,7 @@ class Ops:
         return True
 
     NORMED_MAX_ROWS = 16
-    PARTIALS_BYTES = 1 << 20
+    PARTIALS_BYTES = 4 << 20
 
     def can_fuse_norm(self, n_rows: int, dtype: torch.dtype) -> bool:
         """Whether `linear` has a kernel that takes the norm of this many rows in."""
@@ -359,8 +359,8 @@ class Ops:
         if K % 8 or a.stride(0) % 8 or a.data_ptr() % 16 or w.data_ptr() % 16:
             return False
         lib = self.lib("gemm_bf16")
-        if 16 < M <= 64 and epi == EPI["add"] and self.use_mfma_rows:
-            # MFMAs fed from memory, K split over workgroups; their sums go through a workspace
+        if M > 16 and epi == EPI["add"] and self.use_mfma_rows:
+            # a product of few tiles: K split over workgroups; their sums go through a workspace
             stream = self._stream()
             ws = self._partials
             if ws is None or ws.device != a.device:
@@ -376,7 +376,7 @@ class Ops:
                     self._pending = (out, splits.value)
                 return True
             if rc != 3:
-                self._check(lib, rc, "linear(bf16, 17..64 rows)")
+                self._check(lib, rc, "linear(bf16, split K)")
         rc = lib.ti_gemm_bf16(_ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi, self._stream())
         if rc == 3:          # "shape not served": not an error
             return False
