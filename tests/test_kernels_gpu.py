@@ -547,9 +547,11 @@ def test_linear_bf16_mfma_fed_from_memory(ops, M, N, K, ks):
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 1024, 2048), (64, 1024, 3072), (40, 512, 1024), (33, 96, 1024),
-                                   (20, 2048, 1024), (24, 256, 2048)])
+                                   (20, 2048, 1024), (24, 256, 2048), (136, 1024, 2048), (300, 1000, 3072),
+                                   (65, 520, 1024), (512, 1024, 2048)])
 def test_partial_sums_left_to_the_next_norm(ops, M, N, K):
-    """A product into the residual at 17..64 rows with few columns splits K over workgroups.
+    """A product into the residual whose launch would have few tiles (17..64 rows and few columns:
+    MFMAs fed from memory; up to ~512 rows: 64 x 64 tiles) splits K over workgroups.
     With `may_defer` its partial sums wait for whatever reads the residual next: the norm adds
     them on its way, any other launch (or `flush`) adds them with a kernel of their own.  All
     three give the bits of the product that adds them at once, and match float64."""
@@ -975,10 +977,13 @@ def test_attention_bf16_decode_from_projections(ops, nh, nkv, hd, P, window, nor
 @pytest.mark.parametrize("M,nh,nkv,hd,K,P,norm,rope", [
     (300, 3, 1, 64, 192, 16, True, "table"), (257, 4, 2, 128, 128, 16, True, "table"),
     (100, 2, 2, 128, 64, 32, False, "computed"), (513, 5, 1, 64, 256, 16, True, None), (70, 2, 0, 128, 64, 16, True, "table")])
-def test_qkv_product_with_prepared_heads(ops, M, nh, nkv, hd, K, P, norm, rope):
-    """The q/k/v product whose epilogue norms, rotates and caches, against the product followed
-    by the kernel that prepares whole steps: the same bits in q and in the cache (rows that
-    are no multiple of the tile, a last tile with a head beyond the matrix, no k/v heads)."""
+@pytest.mark.parametrize("tile_rows", [128, 256])
+def test_qkv_product_with_prepared_heads(ops, tile_rows, M, nh, nkv, hd, K, P, norm, rope):
+    """The q/k/v product whose epilogue norms, rotates and caches, with tiles of 128 and of 256
+    rows (the dispatch takes the first while it makes no more workgroups than the chip has
+    units), against the product followed by the kernel that prepares whole steps: the same bits
+    in q and in the cache (rows that are no multiple of the tile, a last tile with a head beyond
+    the matrix, no k/v heads)."""
     if not ops.use_fast_gemm:
         pytest.skip("bfloat16 MFMA kernels are switched off")
     g = torch.Generator().manual_seed(M + nh)
@@ -1010,7 +1015,12 @@ def test_qkv_product_with_prepared_heads(ops, M, nh, nkv, hd, K, P, norm, rope):
     q_a = torch.zeros(M, nh * hd, device="cuda", dtype=torch.bfloat16)
     ops.qk_norm_rope_kv_write(qkv, q_w, k_w, 1e-5, inv_freq, pos, slot, view, pool_a, q_a, nh, nkv, hd, tab)
     q_b = torch.zeros_like(q_a)
-    assert ops.qkv_prepared(a, w, q_w, k_w, 1e-5, inv_freq, tab, pos, slot, view, pool_b, q_b, nh, nkv, hd)
+    lib = ops.lib("gemm_bf16")
+    lib.ti_gemm_bf16_qkv_prep_rows(tile_rows)
+    try:
+        assert ops.qkv_prepared(a, w, q_w, k_w, 1e-5, inv_freq, tab, pos, slot, view, pool_b, q_b, nh, nkv, hd)
+    finally:
+        lib.ti_gemm_bf16_qkv_prep_rows(0)
     assert torch.equal(q_a.view(torch.int16), q_b.view(torch.int16))
     assert torch.equal(pool_a.view(torch.int16), pool_b.view(torch.int16))
     if nkv:
