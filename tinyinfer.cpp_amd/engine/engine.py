@@ -129,7 +129,7 @@ class Engine:
         for part in model.parts():
             if hasattr(part, "prepare"):
                 part.prepare(self.ops, self.max_seq)      # tables that depend on the longest sequence
-        self._ws: Dict[str, torch.Tensor] = {}
+        self._ws: Dict[tuple, object] = {}        # (name, dtype) -> tensor; (name, shape, dtype) -> (tensor, view)
         self._meta_dev = None
         self._meta_host: List[torch.Tensor] = []
         self._meta_events: List[Optional[torch.cuda.Event]] = []
@@ -167,18 +167,27 @@ class Engine:
 
     # ---------------------------------------------------------------- workspace
     def _workspace(self, name: str, shape, dtype) -> torch.Tensor:
+        """A named scratch tensor of this shape; the same memory for the same name in every layer
+        and step (it grows when a larger one is asked for).  The views handed out are kept: a
+        layer asks for the shapes the layer before asked for."""
+        ws = self._ws
+        shape = tuple(shape)
+        hit = ws.get((name, shape, dtype))
+        if hit is not None and hit[0] is ws.get((name, dtype)):
+            return hit[1]
         n = 1
         for s in shape:
             n *= int(s)
-        key = f"{name}/{dtype}"
-        t = self._ws.get(key)
+        t = ws.get((name, dtype))
         if t is None or t.numel() < n:
             cap = max(n, 1)
             if t is not None:
                 cap = max(cap, int(t.numel() * 1.5))
             t = torch.empty(cap, dtype=dtype, device=self.device)
-            self._ws[key] = t
-        return t[:n].view(*shape)
+            ws[(name, dtype)] = t
+        view = t[:n].view(*shape)
+        ws[(name, shape, dtype)] = (t, view)
+        return view
 
     def _meta_buffers(self, n_ints: int, dev_fixed: Optional[torch.Tensor] = None):
         """A pinned host buffer (two take turns) and the device buffer, both >= n_ints.
@@ -485,7 +494,7 @@ class _DecodeGraph:
     def __init__(self):
         self.graph = None
         self.meta: Optional[torch.Tensor] = None
-        self.workspace: Dict[str, torch.Tensor] = {}
+        self.workspace: Dict[tuple, object] = {}
         self.logits: Optional[torch.Tensor] = None
 
 
