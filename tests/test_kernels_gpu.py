@@ -912,6 +912,33 @@ def test_attention_bf16_paired_tiles_of_one_long_prompt(ops):
     assert (outs[0] - outs[1]).abs().max() < 2e-2
 
 
+@pytest.mark.parametrize("nh,nkv,hd,P,window", [(2, 1, 128, 16, None), (4, 2, 64, 32, None), (2, 2, 128, 16, 1500)])
+def test_attention_bf16_short_portions_against_a_long_context(ops, nh, nkv, hd, P, window):
+    """Few tiles, thousands of keys: the keys of every tile are cut into runs with a workgroup
+    each, and a kernel merges their results.  A portion deep in a long request, one at the
+    start of a request (its later runs are empty), one in between, and a single token (its
+    row is written by the decode kernel after the merge has passed over it); against float64
+    and against the same launch with one run."""
+    if not ops.use_fast_attention:
+        pytest.skip("bfloat16 attention kernels are switched off")
+    from tinyinfer_amd.ops import attention_bf16
+    entries = [(70, 3000), (40, 0), (1, 2500), (130, 1000)]
+    ctx = FakeCtx(entries)
+    assert attention_bf16.portion_splits(ctx, nh, int(window or 0)) >= 3
+    outs = []
+    try:
+        for split in (True, False):
+            ops.use_portion_splits = split
+            got, want = fast_attention_case(ops, entries, nh, nkv, hd, P, window, seed=hd + nh)
+            assert torch.isfinite(got).all()
+            assert (got - want).abs().max() < 2e-2
+            outs.append(got)
+    finally:
+        ops.use_portion_splits = True
+    assert (outs[0] - outs[1]).abs().max() < 2e-2
+    assert not torch.equal(outs[0], outs[1]), "the switch did not change the launch"
+
+
 @pytest.mark.parametrize("nh,nkv,hd,P,window,norm,rope", [
     (16, 8, 128, 16, None, True, "table"), (4, 2, 64, 16, None, True, "table"), (3, 1, 128, 32, 50, True, "computed"),
     (4, 4, 64, 16, 40, False, "table"), (16, 1, 64, 16, None, True, None), (8, 2, 128, 16, None, False, None)])

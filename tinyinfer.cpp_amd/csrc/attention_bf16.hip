@@ -732,7 +732,12 @@ __global__ void __launch_bounds__(64 * NW * NG)
 attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool,
                         const int* __restrict__ table, int table_stride, const int* __restrict__ tiles,
                         int n_tiles, const int* __restrict__ entries, bf16_t* __restrict__ out, int n_head,
-                        int n_kv, int P, float scale, int window) {
+                        int n_kv, int P, float scale, int window, float* __restrict__ part_o = nullptr,
+                        float* __restrict__ part_ml = nullptr) {
+  // gridDim.z > 1: the keys a tile sees are cut into gridDim.z runs of whole turns, workgroup z takes
+  // run z and leaves its maxima, sums and unscaled outputs in part_ml [row][head][z] = (m, l) and
+  // part_o [row][head][z][HD] for the kernel that merges them
+  const int n_splits = gridDim.z, split = blockIdx.z;
   constexpr int CB = 1;                               // column blocks (of 32 tokens) per wavefront
   constexpr int WROWS = 32 * CB;                      // tokens per wavefront
   constexpr int TROWS = NW * WROWS;                   // tokens per tile
@@ -849,8 +854,13 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
       for (int i = 0; i < 16; ++i) o[cb][d][i] = 0.f;
   }
 
-  const int blk_lo = (g_lo / PF_KEYS) * 2, blk_hi = g_pos_last / 16;   // 16-key blocks, starting on a turn
+  int blk_lo = (g_lo / PF_KEYS) * 2, blk_hi = g_pos_last / 16;         // 16-key blocks, starting on a turn
   const int v_limit = min(kv_last, blk_hi * 16 + 15);               // last key whose value row is real
+  if (n_splits > 1) {
+    const int per = (((blk_hi + 1 - blk_lo) + n_splits - 1) / n_splits + 1) & ~1;   // whole turns
+    blk_lo += split * per;
+    blk_hi = min(blk_hi, blk_lo + per - 1);                         // a run past the end is empty
+  }
   for (int c0 = blk_lo; c0 <= blk_hi; c0 += 64) {
     const int nblk = min(64, blk_hi + 1 - c0);
     const int n_turns = (nblk + 1) / 2;
@@ -1064,8 +1074,20 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     for (int cb = 0; cb < CB; ++cb) {
       const float lt = l[cb] + __shfl_xor(l[cb], 32, 64);
       if (!col_ok[cb]) continue;
-      const float inv = 1.0f / lt;
       const int row = w_first + cb * 32 + r32;
+      if (n_splits > 1) {
+        const size_t at = ((size_t)row * n_head + head) * n_splits + split;
+        float* po = part_o + at * HD;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4)
+            *reinterpret_cast<float4*>(po + 32 * d + 8 * g4 + 4 * h) =
+                make_float4(o[cb][d][4 * g4], o[cb][d][4 * g4 + 1], o[cb][d][4 * g4 + 2], o[cb][d][4 * g4 + 3]);
+        if (h == 0) reinterpret_cast<float2*>(part_ml)[at] = make_float2(mx[cb], lt);
+        continue;
+      }
+      const float inv = 1.0f / lt;
       bf16_t* dst = out + ((size_t)row * n_head + head) * HD;
 #pragma unroll
       for (int d = 0; d < DB; ++d)
@@ -1281,7 +1303,8 @@ extern "C" int ti_attention_prefill_bf16(const void* q, const void* pool, const 
 extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool, const int* table, int table_stride,
                                                 const int* tiles, const int* entries, void* out, int n_tiles,
                                                 int n_head, int n_kv, int hd, int page_size, float scale,
-                                                int window, hipStream_t stream) {
+                                                int window, int n_rows, float* part_o, float* part_ml,
+                                                int n_splits, hipStream_t stream) {
   int rc = check_common("attention_prefill_paired", n_head, n_kv, hd, page_size, table_stride);
   if (rc) return rc;
   if (hd == 32) {
@@ -1289,6 +1312,8 @@ extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool,
     return 3;
   }
   TI_REQUIRE(n_head <= 65535, "attention_prefill_paired: too many heads");
+  TI_REQUIRE(n_splits >= 1 && n_splits <= 8 && (n_splits == 1 || (part_o && part_ml && n_rows > 0)),
+             "attention_prefill_paired: 1 to 8 runs of keys, more than one with buffers for their results");
   if (n_tiles == 0) return 0;
   constexpr int NG = 4, NW = 2, ST = 2;
   const int lds = NG * ST * 2 * PF_KEYS * hd * 2;
@@ -1303,15 +1328,24 @@ extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool,
     }
     ready = true;
   }
-  dim3 grid((n_tiles + 1) / 2, n_head);
+  dim3 grid((n_tiles + 1) / 2, n_head, n_splits);
   if (hd == 128)
     attn_prefill_lds_kernel<128, NG, NW, ST, true><<<grid, 64 * NW * NG, lds, stream>>>(
         (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, n_tiles, entries, (bf16_t*)out, n_head,
-        n_kv, page_size, scale, window);
+        n_kv, page_size, scale, window, part_o, part_ml);
   else
     attn_prefill_lds_kernel<64, NG, NW, ST, true><<<grid, 64 * NW * NG, lds, stream>>>(
         (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, n_tiles, entries, (bf16_t*)out, n_head,
-        n_kv, page_size, scale, window);
+        n_kv, page_size, scale, window, part_o, part_ml);
+  if (n_splits > 1) {
+    // every row of the step has its runs (rows of single tokens too: theirs are not read by anyone)
+    if (hd == 128)
+      attn_merge_kernel<128><<<dim3(n_rows, n_head), 128, 0, stream>>>(part_o, part_ml, nullptr, (bf16_t*)out, n_head,
+                                                                     n_splits);
+    else
+      attn_merge_kernel<64><<<dim3(n_rows, n_head), 64, 0, stream>>>(part_o, part_ml, nullptr, (bf16_t*)out, n_head,
+                                                                   n_splits);
+  }
   TI_LAUNCH_CHECK();
   return 0;
 }

@@ -107,9 +107,14 @@ int ti_attention_prefill_bf16(const void* q, const void* pool, const int* table,
                               float scale, int window, hipStream_t stream);
 // the same for launches of few tiles (head sizes 64, 128): tiles of 64 rows ordered from the most visible
 // keys to the fewest; a workgroup takes tile b and tile n_tiles - 1 - b, so that all have about the same work
+// n_splits > 1 (up to 8): the keys of every tile are cut into that many runs, each with a workgroup of its
+// own, for launches of few tiles against a long context; their results go through part_o [n_rows][n_head]
+// [n_splits][hd] and part_ml [n_rows][n_head][n_splits][2] and are merged into out for all n_rows rows of the
+// step (rows of no tile get what lies in the buffers: whoever owns them writes them afterwards).
 int ti_attention_prefill_paired_bf16(const void* q, const void* pool, const int* table, int table_stride,
                                      const int* tiles, const int* entries, void* out, int n_tiles, int n_head,
-                                     int n_kv, int hd, int page_size, float scale, int window, hipStream_t stream);
+                                     int n_kv, int hd, int page_size, float scale, int window, int n_rows,
+                                     float* part_o, float* part_ml, int n_splits, hipStream_t stream);
 void ti_attention_decode_shared_query(int on);   // 0: every wavefront of a decode workgroup prepares the query itself
 void ti_attention_prefill_groups(int groups);  // 1 or 2 groups of wavefronts per workgroup, 0: by the launch
 void ti_attention_prefill_use_lds(int on);     // 0: the kernel without LDS for every head size

@@ -62,6 +62,33 @@ def run_decode_prepared(ops, ctx, view, qkv, q_w, k_w, eps, inv_freq, rope_table
     return True
 
 
+PORTION_SPLIT_KEYS = 512         # a portion's keys are cut into runs of at least this many ...
+PORTION_SPLIT_MAX = 8            # ... at most this many runs
+
+
+def portion_splits(ctx, heads: int, window: int) -> int:
+    """Into how many runs the paired prefill kernel cuts the keys of its tiles: 1 unless the launch
+    would leave most compute units idle (a short portion) while every workgroup walks a long
+    context (191 us a layer for 512 rows against 6,144 cached tokens in one run)."""
+    longest = getattr(ctx, "max_context", 0)
+    context = longest if window == 0 else min(longest, window + 64)
+    workgroups = ((ctx.n_tiles_small + 1) // 2) * heads
+    units = compute_units()
+    if workgroups * 2 > units or context < 2 * PORTION_SPLIT_KEYS:
+        return 1
+    return max(1, min(PORTION_SPLIT_MAX, units // workgroups, context // PORTION_SPLIT_KEYS))
+
+
+_units = {}
+
+
+def compute_units() -> int:
+    dev = torch.cuda.current_device()
+    if dev not in _units:
+        _units[dev] = torch.cuda.get_device_properties(dev).multi_processor_count
+    return _units[dev]
+
+
 def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) -> bool:
     P = pool.shape[3]
     if head_dim not in SERVED_HEAD_DIMS or P % 16 != 0:
@@ -70,6 +97,31 @@ def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) 
     stream = ops._stream()
     table = view.table
     win = int(window or 0)
+    # the portions first: with their keys cut into runs, the merge writes every row of the step, and
+    # the rows of single tokens get their own result afterwards
+    if ctx.n_tiles and head_dim in PAIRED_HEAD_DIMS and ctx.n_tiles * heads < PAIRED_BELOW \
+            and getattr(ctx, "tiles_small", None) is not None and ops.use_paired_prefill:
+        # few tiles: under a causal mask they differ much in work, and a launch lasts as long as its
+        # heaviest workgroup; the paired kernel gives every workgroup a heavy and a light tile
+        S = portion_splits(ctx, heads, win) if ops.use_portion_splits else 1
+        part_o = part_ml = None
+        if S > 1:
+            part_o = ctx.buf("attn.portion_o", (ctx.M, heads, S, head_dim), torch.float32)
+            part_ml = ctx.buf("attn.portion_ml", (ctx.M, heads, S, 2), torch.float32)
+        rc = lib.ti_attention_prefill_paired_bf16(
+            _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.tiles_small), _ptr(ctx.entry_meta), _ptr(out),
+            ctx.n_tiles_small, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, ctx.M, _ptr(part_o),
+            _ptr(part_ml), S, stream)
+        if rc == 3:
+            return False
+        ops._check(lib, rc, "attention(prefill, paired)")
+    elif ctx.n_tiles:
+        rc = lib.ti_attention_prefill_bf16(
+            _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.tiles), _ptr(ctx.entry_meta), _ptr(out),
+            ctx.n_tiles, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, stream)
+        if rc == 3:
+            return False
+        ops._check(lib, rc, "attention(prefill)")
     n_dec = ctx.M if ctx.decode_only else ctx.n_decode_rows
     if n_dec:
         rows = None if ctx.decode_only else ctx.decode_rows
@@ -86,21 +138,4 @@ def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) 
         if rc == 3:
             return False
         ops._check(lib, rc, "attention(decode)")
-    if ctx.n_tiles and head_dim in PAIRED_HEAD_DIMS and ctx.n_tiles * heads < PAIRED_BELOW \
-            and getattr(ctx, "tiles_small", None) is not None and ops.use_paired_prefill:
-        # few tiles: under a causal mask they differ much in work, and a launch lasts as long as its
-        # heaviest workgroup; the paired kernel gives every workgroup a heavy and a light tile
-        rc = lib.ti_attention_prefill_paired_bf16(
-            _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.tiles_small), _ptr(ctx.entry_meta), _ptr(out),
-            ctx.n_tiles_small, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, stream)
-        if rc == 3:
-            return False
-        ops._check(lib, rc, "attention(prefill, paired)")
-    elif ctx.n_tiles:
-        rc = lib.ti_attention_prefill_bf16(
-            _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.tiles), _ptr(ctx.entry_meta), _ptr(out),
-            ctx.n_tiles, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, stream)
-        if rc == 3:
-            return False
-        ops._check(lib, rc, "attention(prefill)")
     return True

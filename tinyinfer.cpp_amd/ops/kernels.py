@@ -75,6 +75,7 @@ class Ops:
         self._partials = None
         self._pending = None               # (residual, splits): partial sums not yet added
         self.use_paired_prefill = True   # small prefill launches: a heavy and a light tile per workgroup
+        self.use_portion_splits = True   # ... and the keys of a short portion against a long context cut into runs
 
     # ------------------------------------------------------------------ loading
     def lib(self, name: str) -> ctypes.CDLL:
