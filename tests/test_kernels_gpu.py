@@ -1003,7 +1003,8 @@ def test_attention_bf16_decode_from_projections(ops, nh, nkv, hd, P, window, nor
 
 @pytest.mark.parametrize("M,nh,nkv,hd,K,P,norm,rope", [
     (300, 3, 1, 64, 192, 16, True, "table"), (257, 4, 2, 128, 128, 16, True, "table"),
-    (100, 2, 2, 128, 64, 32, False, "computed"), (513, 5, 1, 64, 256, 16, True, None), (70, 2, 0, 128, 64, 16, True, "table")])
+    (100, 2, 2, 128, 64, 32, False, "computed"), (513, 5, 1, 64, 256, 16, True, None), (70, 2, 0, 128, 64, 16, True, "table"),
+    (40, 2, 1, 128, 64, 16, True, "table"), (17, 3, 1, 64, 128, 16, True, "computed")])
 @pytest.mark.parametrize("tile_rows", [128, 256])
 def test_qkv_product_with_prepared_heads(ops, tile_rows, M, nh, nkv, hd, K, P, norm, rope):
     """The q/k/v product whose epilogue norms, rotates and caches, with tiles of 128 and of 256
@@ -1048,8 +1049,17 @@ def test_qkv_product_with_prepared_heads(ops, tile_rows, M, nh, nkv, hd, K, P, n
         assert ops.qkv_prepared(a, w, q_w, k_w, 1e-5, inv_freq, tab, pos, slot, view, pool_b, q_b, nh, nkv, hd)
     finally:
         lib.ti_gemm_bf16_qkv_prep_rows(0)
-    assert torch.equal(q_a.view(torch.int16), q_b.view(torch.int16))
-    assert torch.equal(pool_a.view(torch.int16), pool_b.view(torch.int16))
+    if M > 64:
+        assert torch.equal(q_a.view(torch.int16), q_b.view(torch.int16))
+        assert torch.equal(pool_a.view(torch.int16), pool_b.view(torch.int16))
+    else:
+        # up to 64 rows the product alone comes from kernels that sum in another order: the same
+        # values up to the rounding of the result (rubbish in untouched cache rows may be NaN: bits there)
+        assert (f64(q_a) - f64(q_b)).abs().max() <= 2 ** -7 * f64(q_a).abs().max()
+        touched = pool_a.view(torch.int16) != dev(pool0).view(torch.int16)
+        assert torch.equal(touched, pool_b.view(torch.int16) != dev(pool0).view(torch.int16)) or nkv == 0
+        da, db = f64(pool_a)[touched.cpu()], f64(pool_b)[touched.cpu()]
+        assert nkv == 0 or (da - db).abs().max() <= 2 ** -7 * da.abs().max()
     if nkv:
         assert not torch.equal(pool_a.view(torch.int16), dev(pool0).view(torch.int16))
 

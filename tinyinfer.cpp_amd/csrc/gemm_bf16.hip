@@ -974,7 +974,9 @@ static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, 
   return 0;
 }
 
-static int g_qkv_rows = 0;       // a hook for measurements: 128 or 256 forces the tile's rows
+static int g_qkv_rows = 0;       // hooks for measurements: 128 or 256 forces the tile's rows;
+static int g_qkv_min_rows = 17;  // the fewest rows served (fewer take the kernels with the norm in front)
+extern "C" void ti_gemm_bf16_qkv_prep_min_rows(int rows) { g_qkv_min_rows = rows; }
 extern "C" void ti_gemm_bf16_qkv_prep_rows(int rows) { g_qkv_rows = rows; }
 
 static int compute_units() {
@@ -1009,7 +1011,7 @@ static int launch_qkv_prep(const void* A, const void* W, int M, int N, int K, lo
 
 // The fused q/k/v projection of a step's rows with the per-head work in its epilogue (see
 // QKVEpilogue): A [M, K] bf16, W [(n_head + 2 n_kv) hd, K] bf16 (n_kv = 0: q heads only, nothing is
-// written to the cache).  Returns 3 for what it does not serve: M <= 64, K not a multiple of 64,
+// written to the cache).  Returns 3 for what it does not serve: M <= 16, K not a multiple of 64,
 // head sizes other than 64 and 128.
 extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K, long lda, const float* q_w,
                                      const float* k_w, float eps, const float* inv_freq, const float* rope_table,
@@ -1018,9 +1020,9 @@ extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K,
                                      int page_size, hipStream_t stream) {
   TI_REQUIRE(M >= 0 && K > 0 && lda >= K && n_head > 0 && n_kv >= 0 && hd > 0 && page_size > 0 && table_stride > 0,
              "gemm_bf16_qkv_prep: bad sizes");
-  if (M <= 64 || K % 64 != 0 || lda % 8 != 0 || !(hd == 64 || hd == 128) || ((uintptr_t)A & 15) ||
+  if (M < g_qkv_min_rows || K % 64 != 0 || lda % 8 != 0 || !(hd == 64 || hd == 128) || ((uintptr_t)A & 15) ||
       ((uintptr_t)W & 15) || ((uintptr_t)q_out & 15) || ((uintptr_t)pool & 15) || ((uintptr_t)rope_table & 15)) {
-    ti_set_error("gemm_bf16_qkv_prep: M=%d K=%d head_dim=%d is not served (M > 64, K %% 64 == 0, head_dim 64 or 128)",
+    ti_set_error("gemm_bf16_qkv_prep: M=%d K=%d head_dim=%d is not served (M > 16, K %% 64 == 0, head_dim 64 or 128)",
                  M, K, hd);
     return 3;
   }

@@ -65,7 +65,7 @@ int ti_gemm_bf16_mblocks_any(const void* A, const void* W, void* out, int M, int
 // out (op)= rmsnorm(x; nw, eps) W^T for M <= 16, K a multiple of 64
 int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, const void* W, void* out, int M, int N, int K, int epi,
                         hipStream_t stream);
-// the q/k/v product of a step (M > 64) that finishes its heads itself: see ti_qk_norm_rope_kv_write
+// the q/k/v product of a step (M > 16) that finishes its heads itself: see ti_qk_norm_rope_kv_write
 int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K, long lda, const float* q_w, const float* k_w,
                           float eps, const float* inv_freq, const float* rope_table, int table_len, const int* pos,
                           const int* slot, const int* table, int table_stride, void* pool, void* q_out, int n_head,
@@ -73,6 +73,7 @@ int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K, long lda, 
 // switches for measurements and tests (0 restores the choice by shape)
 void ti_gemm_bf16_force_tile(int which);      // 1: 256 x 128, 3: 128 x 64, 6: 64 x 64
 void ti_gemm_bf16_skinny_waves(int waves);    // 4 or 8 wavefronts in the kernel for M <= 64
+void ti_gemm_bf16_qkv_prep_min_rows(int rows); // the fewest rows ti_gemm_bf16_qkv_prep serves (17)
 void ti_gemm_bf16_qkv_prep_rows(int rows);    // 128 / 256: the rows of ti_gemm_bf16_qkv_prep's tile; 0: by the shape
 void ti_gemm_bf16_mblocks_on(int on);         // 0: ti_gemm_bf16_mblocks serves nothing
 void ti_gemm_bf16_use_pipelined(int on);      // 0: the plain tiled kernel for every K
