@@ -113,6 +113,34 @@ def measure_prefill(engine, rng, reps=5):
     return times[len(times) // 2]
 
 
+def measure_mixed(engine, batch, portion, cached, rng, reps=8):
+    """ms of a step that holds one decoded token of each of `batch` requests (CONTEXT tokens
+    each) beside `portion` tokens of a prompt of which `cached` tokens are in the cache already:
+    what the scheduler runs while a prompt arrives in portions.  Not a captured graph."""
+    import torch
+    from tinyinfer_amd.engine import StepEntry
+    V = engine.model.vocab_size
+    rids = [f"x{i}" for i in range(batch)]
+    fill(engine, rids, CONTEXT, rng)
+    times = []
+    for i in range(reps + 3):
+        if cached:
+            engine.step([StepEntry("long", rng.integers(0, V, size=cached).tolist(), ())])
+        entries = [StepEntry(r, [int(rng.integers(0, V))], (0,)) for r in rids]
+        entries.append(StepEntry("long", rng.integers(0, V, size=portion).tolist(), (portion - 1,)))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = engine.step(entries)
+        logits[0, :8].cpu()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        engine.release("long")
+    for r in rids:
+        engine.release(r)
+    times = sorted(times[3:])
+    return times[len(times) // 2] * 1e3
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -121,8 +149,11 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
-    ap.add_argument("--only", choices=["all", "decode", "prefill"], default="all",
-                    help="measure one phase only (for profiles): the other's fields are null")
+    ap.add_argument("--only", choices=["all", "decode", "prefill", "mixed"], default="all",
+                    help="measure one phase only (for profiles): the other's fields are null; "
+                         "mixed: a step of --batch decoded tokens beside --portion tokens of a prompt, a line of its own")
+    ap.add_argument("--portion", type=int, default=128, help="--only mixed: tokens of the prompt in the step")
+    ap.add_argument("--cached", type=int, default=0, help="--only mixed: tokens of that prompt already in the cache")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not served (this engine runs on a single GPU)")
@@ -142,11 +173,19 @@ def main() -> int:
     biggest = max(args.batch, 1 if (args.no_points or args.only != "all") else 64)
     say("building the model (random weights on the device) ...")
     engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", page_size=PAGE,
-                                max_tokens=biggest * (CONTEXT + 512) + PREFILL_TOKENS, max_requests=biggest + 1,
+                                max_tokens=biggest * (CONTEXT + 512) + PREFILL_TOKENS + args.cached + args.portion,
+                                max_requests=biggest + 1,
                                 max_seq=MAX_SEQ)
     sampler = Sampler(engine.ops, engine.device)
     nums = model_numbers(cfg)
 
+    if args.only == "mixed":
+        say(f"a step of {args.batch} decoded tokens beside a portion of {args.portion} (after {args.cached} cached) ...")
+        ms = measure_mixed(engine, args.batch, args.portion, args.cached, rng)
+        print(json.dumps({"mixed": {"ms_per_step": round(ms, 3), "tokens": args.batch + args.portion,
+                                    "decoded": args.batch, "portion": args.portion, "cached": args.cached,
+                                    "decode_context": CONTEXT}}), flush=True)
+        return 0
     p_s = tps = ms = None
     if args.only != "decode":
         say(f"prefill of {PREFILL_TOKENS} tokens ...")

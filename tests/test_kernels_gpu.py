@@ -808,6 +808,7 @@ class FakeCtx:
         self.decode_rows = None if self.decode_only else (dev(torch.tensor(dec, dtype=torch.int32)) if dec else None)
         self.n_decode_rows = 0 if self.decode_only else len(dec)
         self.max_context = self.split_context = max(s + n for n, s in entries)
+        self.portion_context = max([s + n for n, s in entries if n > 1], default=0)
         self._bufs = {}
 
     def buf(self, name, shape, dtype):

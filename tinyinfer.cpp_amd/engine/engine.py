@@ -77,6 +77,7 @@ class StepContext:
         self.decode_rows = None           # int32: rows of single-token entries (None if decode_only)
         self.n_decode_rows = 0
         self.max_context = 0              # longest context (tokens) any row reads in this step
+        self.portion_context = 0          # the same over the rows of portions (entries of several tokens) only
         self.split_context = 0            # the context length the decode kernel's split count is sized for
         self.run = 0                      # index into the model's run order
         self._views: Dict[int, CacheView] = {}
@@ -343,6 +344,8 @@ class Engine:
                         tiles.append(row0 + q0)
                     for q0 in range(0, n, PREFILL_TILE_SMALL):
                         small.append((start + min(q0 + PREFILL_TILE_SMALL, n) - 1, i, row0 + q0))
+                    if start + n > ctx.portion_context:
+                        ctx.portion_context = start + n
                 else:
                     h[o_pos + row0] = start
                     dec_rows.append(row0)

@@ -70,7 +70,7 @@ def portion_splits(ctx, heads: int, window: int) -> int:
     """Into how many runs the paired prefill kernel cuts the keys of its tiles: 1 unless the launch
     would leave most compute units idle (a short portion) while every workgroup walks a long
     context (191 us a layer for 512 rows against 6,144 cached tokens in one run)."""
-    longest = getattr(ctx, "max_context", 0)
+    longest = getattr(ctx, "portion_context", 0)
     context = longest if window == 0 else min(longest, window + 64)
     workgroups = ((ctx.n_tiles_small + 1) // 2) * heads
     units = compute_units()
