@@ -873,24 +873,26 @@ def test_attention_bf16_decode_rows(ops, nh, nkv, hd, P, window):
 @pytest.mark.parametrize("nh,nkv,hd,P,window", [
     (4, 2, 64, 16, None), (6, 2, 32, 16, None), (4, 2, 128, 16, None), (2, 1, 128, 32, None),
     (4, 4, 64, 16, 40), (2, 2, 32, 16, 7)])
-@pytest.mark.parametrize("variant", ["one group", "two groups", "paired"])
+@pytest.mark.parametrize("variant", ["one group", "two groups", "paired", "a tile each"])
 def test_attention_bf16_portions_and_mixed(ops, nh, nkv, hd, P, window, variant):
     """Portions of every size, starting anywhere (a page's edge, the middle of a
     page, the start of a request), beside decode rows; with one and with two groups of
-    wavefronts per workgroup, and with the kernel that gives a workgroup two tiles of
-    64 rows (the launch would choose by its size)."""
+    wavefronts per workgroup, and with the kernel of 64-row tiles, giving a workgroup two
+    tiles or one (the launch would choose by its size)."""
     if not ops.use_fast_attention:
         pytest.skip("bfloat16 attention kernels are switched off")
     entries = [(2, 0), (7, 30), (1, 99), (16, 16), (17, 15), (64, 0), (65, 63), (130, 41), (1, 0), (3, 300), (200, 5),
                (333, 700)]
     lib = ops.lib("attention_bf16")
-    lib.ti_attention_prefill_groups({"one group": 1, "two groups": 2, "paired": 0}[variant])
-    ops.use_paired_prefill = variant == "paired"
+    lib.ti_attention_prefill_groups({"one group": 1, "two groups": 2}.get(variant, 0))
+    ops.use_paired_prefill = variant in ("paired", "a tile each")
+    ops.force_paired_tiles = variant == "paired"
     try:
         got, want = fast_attention_case(ops, entries, nh, nkv, hd, P, window, seed=nh * 10 + hd)
     finally:
         lib.ti_attention_prefill_groups(0)
         ops.use_paired_prefill = True
+        ops.force_paired_tiles = None
     assert torch.isfinite(got).all()
     assert (got - want).abs().max() < 2e-2
 
@@ -904,17 +906,19 @@ def test_attention_bf16_paired_tiles_of_one_long_prompt(ops):
     outs = []
     try:
         for paired in (True, False):
-            ops.use_paired_prefill = paired
+            ops.use_paired_prefill = ops.force_paired_tiles = paired
             got, want = fast_attention_case(ops, [(1100, 0), (1, 40)], 4, 2, 128, 16, None, seed=5)
             assert (got - want).abs().max() < 2e-2
             outs.append(got)
     finally:
         ops.use_paired_prefill = True
+        ops.force_paired_tiles = None
     assert (outs[0] - outs[1]).abs().max() < 2e-2
 
 
+@pytest.mark.parametrize("paired", [True, False])
 @pytest.mark.parametrize("nh,nkv,hd,P,window", [(2, 1, 128, 16, None), (4, 2, 64, 32, None), (2, 2, 128, 16, 1500)])
-def test_attention_bf16_short_portions_against_a_long_context(ops, nh, nkv, hd, P, window):
+def test_attention_bf16_short_portions_against_a_long_context(ops, nh, nkv, hd, P, window, paired):
     """Few tiles, thousands of keys: the keys of every tile are cut into runs with a workgroup
     each, and a kernel merges their results.  A portion deep in a long request, one at the
     start of a request (its later runs are empty), one in between, and a single token (its
@@ -925,8 +929,9 @@ def test_attention_bf16_short_portions_against_a_long_context(ops, nh, nkv, hd, 
     from tinyinfer_amd.ops import attention_bf16
     entries = [(70, 3000), (40, 0), (1, 2500), (130, 1000)]
     ctx = FakeCtx(entries)
-    assert attention_bf16.portion_splits(ctx, nh, int(window or 0)) >= 3
+    assert attention_bf16.portion_launch(ctx, nh, int(window or 0))[0] >= 3
     outs = []
+    ops.force_paired_tiles = paired
     try:
         for split in (True, False):
             ops.use_portion_splits = split
@@ -936,6 +941,7 @@ def test_attention_bf16_short_portions_against_a_long_context(ops, nh, nkv, hd, 
             outs.append(got)
     finally:
         ops.use_portion_splits = True
+        ops.force_paired_tiles = None
     assert (outs[0] - outs[1]).abs().max() < 2e-2
     assert not torch.equal(outs[0], outs[1]), "the switch did not change the launch"
 

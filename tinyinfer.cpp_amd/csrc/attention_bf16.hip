@@ -1304,7 +1304,7 @@ extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool,
                                                 const int* tiles, const int* entries, void* out, int n_tiles,
                                                 int n_head, int n_kv, int hd, int page_size, float scale,
                                                 int window, int n_rows, float* part_o, float* part_ml,
-                                                int n_splits, hipStream_t stream) {
+                                                int n_splits, int paired, hipStream_t stream) {
   int rc = check_common("attention_prefill_paired", n_head, n_kv, hd, page_size, table_stride);
   if (rc) return rc;
   if (hd == 32) {
@@ -1322,21 +1322,28 @@ extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool,
     if (hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<128, NG, NW, ST, true>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, NG * ST * 2 * PF_KEYS * 128 * 2) != hipSuccess ||
         hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<64, NG, NW, ST, true>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, NG * ST * 2 * PF_KEYS * 64 * 2) != hipSuccess ||
+        hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<128, NG, NW, ST, false>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, NG * ST * 2 * PF_KEYS * 128 * 2) != hipSuccess ||
+        hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<64, NG, NW, ST, false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, NG * ST * 2 * PF_KEYS * 64 * 2) != hipSuccess) {
       ti_set_error("attention_prefill_paired: cannot reserve the LDS");
       return 2;
     }
     ready = true;
   }
-  dim3 grid((n_tiles + 1) / 2, n_head, n_splits);
-  if (hd == 128)
-    attn_prefill_lds_kernel<128, NG, NW, ST, true><<<grid, 64 * NW * NG, lds, stream>>>(
-        (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, n_tiles, entries, (bf16_t*)out, n_head,
-        n_kv, page_size, scale, window, part_o, part_ml);
-  else
-    attn_prefill_lds_kernel<64, NG, NW, ST, true><<<grid, 64 * NW * NG, lds, stream>>>(
-        (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, n_tiles, entries, (bf16_t*)out, n_head,
-        n_kv, page_size, scale, window, part_o, part_ml);
+  // paired = 0: a workgroup per tile (a launch that fits the chip in one round lasts as long as its
+  // heaviest tile then, not as the heaviest and the lightest together)
+  dim3 grid(paired ? (n_tiles + 1) / 2 : n_tiles, n_head, n_splits);
+#define TI_GO(H, PAIRED)                                                                                          \
+  attn_prefill_lds_kernel<H, NG, NW, ST, PAIRED><<<grid, 64 * NW * NG, lds, stream>>>(                            \
+      (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, n_tiles, entries, (bf16_t*)out, n_head, \
+      n_kv, page_size, scale, window, part_o, part_ml)
+  if (hd == 128 && paired) TI_GO(128, true);
+  else if (hd == 128) TI_GO(128, false);
+  else if (paired) TI_GO(64, true);
+  else TI_GO(64, false);
+#undef TI_GO
   if (n_splits > 1) {
     // every row of the step has its runs (rows of single tokens too: theirs are not read by anyone)
     if (hd == 128)

@@ -112,10 +112,11 @@ int ti_attention_prefill_bf16(const void* q, const void* pool, const int* table,
 // own, for launches of few tiles against a long context; their results go through part_o [n_rows][n_head]
 // [n_splits][hd] and part_ml [n_rows][n_head][n_splits][2] and are merged into out for all n_rows rows of the
 // step (rows of no tile get what lies in the buffers: whoever owns them writes them afterwards).
+// paired = 0: the same kernel with a workgroup per tile, for launches that fit the chip in one round.
 int ti_attention_prefill_paired_bf16(const void* q, const void* pool, const int* table, int table_stride,
                                      const int* tiles, const int* entries, void* out, int n_tiles, int n_head,
                                      int n_kv, int hd, int page_size, float scale, int window, int n_rows,
-                                     float* part_o, float* part_ml, int n_splits, hipStream_t stream);
+                                     float* part_o, float* part_ml, int n_splits, int paired, hipStream_t stream);
 void ti_attention_decode_shared_query(int on);   // 0: every wavefront of a decode workgroup prepares the query itself
 void ti_attention_prefill_groups(int groups);  // 1 or 2 groups of wavefronts per workgroup, 0: by the launch
 void ti_attention_prefill_use_lds(int on);     // 0: the kernel without LDS for every head size

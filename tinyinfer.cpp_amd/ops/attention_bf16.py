@@ -66,17 +66,20 @@ PORTION_SPLIT_KEYS = 512         # a portion's keys are cut into runs of at leas
 PORTION_SPLIT_MAX = 8            # ... at most this many runs
 
 
-def portion_splits(ctx, heads: int, window: int) -> int:
-    """Into how many runs the paired prefill kernel cuts the keys of its tiles: 1 unless the launch
-    would leave most compute units idle (a short portion) while every workgroup walks a long
-    context (191 us a layer for 512 rows against 6,144 cached tokens in one run)."""
+def portion_launch(ctx, heads: int, window: int):
+    """(runs of keys, paired) for the prefill kernel with 64-row tiles.  A launch whose tiles all find
+    a compute unit at once gives each tile a workgroup of its own (it lasts as long as its heaviest
+    tile then); a larger one pairs the heaviest tile with the lightest.  The keys are cut into
+    runs when the launch would leave most units idle (a short portion) while every workgroup walks a
+    long context (191 us a layer for 512 rows against 6,144 cached tokens in one run)."""
     longest = getattr(ctx, "portion_context", 0)
     context = longest if window == 0 else min(longest, window + 64)
-    workgroups = ((ctx.n_tiles_small + 1) // 2) * heads
     units = compute_units()
+    paired = ctx.n_tiles_small * heads > units
+    workgroups = ((ctx.n_tiles_small + 1) // 2 if paired else ctx.n_tiles_small) * heads
     if workgroups * 2 > units or context < 2 * PORTION_SPLIT_KEYS:
-        return 1
-    return max(1, min(PORTION_SPLIT_MAX, units // workgroups, context // PORTION_SPLIT_KEYS))
+        return 1, paired
+    return max(1, min(PORTION_SPLIT_MAX, units // workgroups, context // PORTION_SPLIT_KEYS)), paired
 
 
 _units = {}
@@ -103,7 +106,11 @@ def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) 
             and getattr(ctx, "tiles_small", None) is not None and ops.use_paired_prefill:
         # few tiles: under a causal mask they differ much in work, and a launch lasts as long as its
         # heaviest workgroup; the paired kernel gives every workgroup a heavy and a light tile
-        S = portion_splits(ctx, heads, win) if ops.use_portion_splits else 1
+        S, paired = portion_launch(ctx, heads, win)
+        if not ops.use_portion_splits:
+            S = 1
+        if ops.force_paired_tiles is not None:
+            paired = ops.force_paired_tiles
         part_o = part_ml = None
         if S > 1:
             part_o = ctx.buf("attn.portion_o", (ctx.M, heads, S, head_dim), torch.float32)
@@ -111,7 +118,7 @@ def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) 
         rc = lib.ti_attention_prefill_paired_bf16(
             _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.tiles_small), _ptr(ctx.entry_meta), _ptr(out),
             ctx.n_tiles_small, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, ctx.M, _ptr(part_o),
-            _ptr(part_ml), S, stream)
+            _ptr(part_ml), S, int(paired), stream)
         if rc == 3:
             return False
         ops._check(lib, rc, "attention(prefill, paired)")

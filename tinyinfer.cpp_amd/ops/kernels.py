@@ -76,6 +76,7 @@ class Ops:
         self._pending = None               # (residual, splits): partial sums not yet added
         self.use_paired_prefill = True   # small prefill launches: a heavy and a light tile per workgroup
         self.use_portion_splits = True   # ... and the keys of a short portion against a long context cut into runs
+        self.force_paired_tiles = None   # True / False: that kernel with / without pairs, whatever the launch
 
     # ------------------------------------------------------------------ loading
     def lib(self, name: str) -> ctypes.CDLL:
