@@ -24,7 +24,7 @@ def decode_splits(n_rows: int, kv_heads: int, heads: int, context: int) -> int:
 
 
 def _ptr(t):
-    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+    return None if t is None else t.data_ptr()       # argument types are declared: see kernels.declare_signatures
 
 
 PREPARED_HEAD_DIMS = (64, 128)   # head sizes whose queries the decode kernel prepares itself

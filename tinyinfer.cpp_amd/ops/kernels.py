@@ -35,7 +35,55 @@ def _code(dt: torch.dtype) -> int:
 
 
 def _ptr(t: Optional[torch.Tensor]):
-    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+    """The tensor's address as a plain int (None: a null pointer).  Every library function is
+    called with the argument types its declaration in tinyinfer_kernels.h gives (see
+    `declare_signatures`), so no ctypes object has to be built per pointer."""
+    return None if t is None else t.data_ptr()
+
+
+_C_TYPES = {"int": ctypes.c_int, "long": ctypes.c_long, "float": ctypes.c_float}
+
+
+def header_signatures(text: str) -> Dict[str, tuple]:
+    """{function: (restype, [argtypes])} of the `int ti_...(...)` and `void ti_...(...)`
+    declarations of the kernels' header: pointers and streams as void pointers, int, long and
+    float as themselves.  A declaration with any other type raises."""
+    import re
+    text = re.sub(r"//[^\n]*", "", text)
+    out = {}
+    for ret, name, args in re.findall(r"\b(int|void)\s+(ti_\w+)\s*\(([^)]*)\)\s*;", text):
+        types = []
+        for arg in (a.strip() for a in args.split(",")):
+            if not arg or arg == "void":
+                continue
+            if "*" in arg or arg.startswith("hipStream_t"):
+                types.append(ctypes.c_void_p)
+                continue
+            words = [w for w in arg.replace("const", " ").split()]
+            if len(words) != 2 or words[0] not in _C_TYPES:
+                raise KernelError(f"tinyinfer_kernels.h: cannot read the argument {arg!r} of {name}")
+            types.append(_C_TYPES[words[0]])
+        out[name] = (ctypes.c_int if ret == "int" else None, types)
+    return out
+
+
+_signatures: Optional[Dict[str, tuple]] = None
+
+
+def declare_signatures(lib: ctypes.CDLL) -> None:
+    """Give every function of the header that this library exports its argument types."""
+    global _signatures
+    if _signatures is None:
+        import os
+        with open(os.path.join(_build.HERE, "tinyinfer_kernels.h")) as f:
+            _signatures = header_signatures(f.read())
+    for name, (restype, argtypes) in _signatures.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            continue
+        fn.restype = restype
+        fn.argtypes = argtypes
 
 
 class NormedRows:
@@ -87,6 +135,7 @@ class Ops:
             path = _build.ensure([name])[name]
             lib = ctypes.CDLL(path)
             lib.ti_last_error.restype = ctypes.c_char_p
+            declare_signatures(lib)
             self._libs[name] = lib
         return lib
 
@@ -117,8 +166,8 @@ class Ops:
     @staticmethod
     def _raw_stream():
         if _RAW_STREAM is not None:
-            return ctypes.c_void_p(_RAW_STREAM(torch.cuda.current_device()))
-        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            return _RAW_STREAM(torch.cuda.current_device()) or None      # 0, the default stream: a null pointer
+        return torch.cuda.current_stream().cuda_stream or None
 
     def flush(self):
         """A product into the residual whose K was split over workgroups (17..64 rows, few
