@@ -290,11 +290,11 @@ def test_steps_of_17_to_64_tokens_at_real_width(model_folders):
     try:
         for how in ("left to the norm", "added at once", "without MFMA"):
             ops.use_deferred_add = how == "left to the norm"
-            ops.use_mfma_rows = how != "without MFMA"
+            ops.use_split_k_add = how != "without MFMA"
             results[how] = replay(build_engine(folder, "bfloat16", 256), trace)
             assert ops._pending is None
     finally:
-        ops.use_deferred_add = ops.use_mfma_rows = True
+        ops.use_deferred_add = ops.use_split_k_add = True
     for r in requests:
         got = results["left to the norm"][r]
         err = np.abs(got - want[r][rows[r]]).max()

@@ -593,13 +593,13 @@ def test_partial_sums_left_to_the_next_norm(ops, M, N, K):
         assert torch.equal(h, want_h), how
     # switched off, the other kernels take these sizes: the same values up to rounding
     try:
-        ops.use_mfma_rows = False
+        ops.use_split_k_add = False
         x = dev(base.clone())
         ops.linear(a, w, x, "add", may_defer=True)
         assert ops._pending is None
         assert (x - want_x).abs().max() < 2e-5 * K
     finally:
-        ops.use_mfma_rows = True
+        ops.use_split_k_add = True
 
 
 @pytest.mark.parametrize("rows,H,KS", [(5, 2304, 3), (3, 1028, 5), (9, 64, 1), (2, 1024, 4), (70, 1536, 2)])

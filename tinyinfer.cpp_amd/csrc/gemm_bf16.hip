@@ -1362,8 +1362,8 @@ gemm_partials_add_kernel(float* __restrict__ out, const float* __restrict__ part
   out[i] = v;
 }
 
-static int g_mblocks = 1;        // a hook for measurements: 0 leaves 17..64 rows to the kernels without MFMA
-extern "C" void ti_gemm_bf16_mblocks_on(int on) { g_mblocks = on; }
+static int g_add_split = 1;        // a hook for measurements: 0: ti_gemm_bf16_add_split serves nothing
+extern "C" void ti_gemm_bf16_add_split_on(int on) { g_add_split = on; }
 
 template <int EPI>
 static void launch_mblocks(const bf16_t* a, const bf16_t* w, void* out, float* partial, int M, int N, int K,
@@ -1378,7 +1378,7 @@ static void launch_mblocks(const bf16_t* a, const bf16_t* w, void* out, float* p
 }
 
 // out[i] += partial[0][i] + ... + partial[KS - 1][i] for count elements: what a product with a split
-// K leaves to do (see ti_gemm_bf16_mblocks)
+// K leaves to do (see ti_gemm_bf16_add_split)
 extern "C" int ti_gemm_bf16_partials_add(float* out, const float* partial, int KS, long count, hipStream_t stream) {
   TI_REQUIRE(KS >= 1 && count >= 0, "gemm_bf16_partials_add: bad sizes KS=%d count=%ld", KS, count);
   if (count == 0) return 0;
@@ -1398,14 +1398,14 @@ extern "C" int ti_gemm_bf16_partials_add(float* out, const float* partial, int K
 // addition (ti_gemm_bf16_partials_add, or a kernel that reads the residual next and adds them on
 // the way).  defer = 2: what defer = 1 serves, added here (the same bits).  Returns 3 for what
 // it does not serve.
-extern "C" int ti_gemm_bf16_mblocks(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
+extern "C" int ti_gemm_bf16_add_split(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
                                     void* partial, long partial_bytes, int defer, int* splits, hipStream_t stream) {
-  TI_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K, "gemm_bf16_mblocks: bad sizes M=%d N=%d K=%d lda=%ld", M, N, K, lda);
-  TI_REQUIRE(splits != nullptr, "gemm_bf16_mblocks: splits must point to an int");
+  TI_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K, "gemm_bf16_add_split: bad sizes M=%d N=%d K=%d lda=%ld", M, N, K, lda);
+  TI_REQUIRE(splits != nullptr, "gemm_bf16_add_split: splits must point to an int");
   *splits = 0;
   int KS = 1;
   const bool small = M <= 64;
-  if (g_mblocks && epi == TI_EPI_ADD_F32 && partial && M > 16 && K % 64 == 0 && lda % 8 == 0 &&
+  if (g_add_split && epi == TI_EPI_ADD_F32 && partial && M > 16 && K % 64 == 0 && lda % 8 == 0 &&
       !((uintptr_t)A & 15) && !((uintptr_t)W & 15) && !((uintptr_t)partial & 15) && (small || g_use_pipelined)) {
     // split K until the launch has about a workgroup per compute unit
     const long tiles = small ? (N + 15) / 16 : (long)((M + 63) / 64) * ((N + 63) / 64);
@@ -1417,7 +1417,7 @@ extern "C" int ti_gemm_bf16_mblocks(const void* A, const void* W, void* out, int
     if (!defer && !small && KS < 4) KS = 1;
   }
   if (KS == 1) {
-    ti_set_error("gemm_bf16_mblocks: serves more than 16 rows added into a product of few tiles, K a multiple of 64");
+    ti_set_error("gemm_bf16_add_split: serves more than 16 rows added into a product of few tiles, K a multiple of 64");
     return 3;
   }
   if (small) {

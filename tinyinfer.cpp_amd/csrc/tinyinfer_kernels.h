@@ -56,10 +56,10 @@ int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int N, int K, l
 // in partial [*splits][M][N] and the caller adds them (ti_gemm_bf16_partials_add, or
 // ti_rmsnorm_add_partials on the way to the next norm); defer = 2: as 1, but added here.
 // Returns 3 for what it does not serve.
-int ti_gemm_bf16_mblocks(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
+int ti_gemm_bf16_add_split(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
                          void* partial, long partial_bytes, int defer, int* splits, hipStream_t stream);
 int ti_gemm_bf16_partials_add(float* out, const float* partial, int KS, long count, hipStream_t stream);
-// the kernel of ti_gemm_bf16_mblocks alone, for tests: any epilogue, 1..64 rows, K split ks ways
+// the kernel of ti_gemm_bf16_add_split alone, for tests: any epilogue, 1..64 rows, K split ks ways
 int ti_gemm_bf16_mblocks_any(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
                              void* partial, int ks, hipStream_t stream);
 // out (op)= rmsnorm(x; nw, eps) W^T for M <= 16, K a multiple of 64
@@ -75,7 +75,7 @@ void ti_gemm_bf16_force_tile(int which);      // 1: 256 x 128, 3: 128 x 64, 6: 6
 void ti_gemm_bf16_skinny_waves(int waves);    // 4 or 8 wavefronts in the kernel for M <= 64
 void ti_gemm_bf16_qkv_prep_min_rows(int rows); // the fewest rows ti_gemm_bf16_qkv_prep serves (17)
 void ti_gemm_bf16_qkv_prep_rows(int rows);    // 128 / 256: the rows of ti_gemm_bf16_qkv_prep's tile; 0: by the shape
-void ti_gemm_bf16_mblocks_on(int on);         // 0: ti_gemm_bf16_mblocks serves nothing
+void ti_gemm_bf16_add_split_on(int on);         // 0: ti_gemm_bf16_add_split serves nothing
 void ti_gemm_bf16_use_pipelined(int on);      // 0: the plain tiled kernel for every K
 void ti_gemm_bf16_row_per_wave(int on);        // 0: few tokens and a weight of few rows take the 16-row kernels too
 void ti_gemm_bf16_skinny_copy(int on);        // 0: up to 16 tokens, fragments of the token rows straight from memory

@@ -118,7 +118,7 @@ class Ops:
         self.use_fused_norm = True       # the norm before a product inside the product's kernel (few tokens)
         self.use_fused_qk_decode = True  # per-head norm, rotation and cache write inside the decode attention
         self.use_fused_qkv_prefill = True  # the same in the epilogue of the q/k/v product (steps of many tokens)
-        self.use_mfma_rows = True          # products into the residual of few tiles: K split over workgroups
+        self.use_split_k_add = True          # products into the residual of few tiles: K split over workgroups
         self.use_deferred_add = True       # ... and its partial sums added by the norm that comes next
         self._partials = None
         self._pending = None               # (residual, splits): partial sums not yet added
@@ -410,7 +410,7 @@ class Ops:
         if K % 8 or a.stride(0) % 8 or a.data_ptr() % 16 or w.data_ptr() % 16:
             return False
         lib = self.lib("gemm_bf16")
-        if M > 16 and epi == EPI["add"] and self.use_mfma_rows:
+        if M > 16 and epi == EPI["add"] and self.use_split_k_add:
             # a product of few tiles: K split over workgroups; their sums go through a workspace
             stream = self._stream()
             ws = self._partials
@@ -419,7 +419,7 @@ class Ops:
             # 1: the sums are left for the next norm; 2: the same product, added at once
             defer = 0 if not may_defer else 1 if self.use_deferred_add else 2
             splits = ctypes.c_int(0)
-            rc = lib.ti_gemm_bf16_mblocks(_ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi,
+            rc = lib.ti_gemm_bf16_add_split(_ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi,
                                           _ptr(ws), ctypes.c_long(self.PARTIALS_BYTES), defer,
                                           ctypes.byref(splits), stream)
             if rc == 0:
