@@ -1,6 +1,7 @@
-"""The argument types that Python gives the kernel libraries come from the declarations in
-tinyinfer_kernels.h: pointers are passed as plain ints, which ctypes would cut to 32 bits for a
-function without declared types."""
+"""What the kernels' Python side decides on the host.  The argument types that Python gives the kernel
+libraries come from the declarations in tinyinfer_kernels.h: pointers are passed as plain ints,
+which ctypes would cut to 32 bits for a function without declared types.  And the number of runs the
+decode attention cuts a context into."""
 import ctypes
 import os
 import re
@@ -51,3 +52,22 @@ def test_a_declaration_with_an_unknown_type_is_refused():
     import pytest
     with pytest.raises(kernels.KernelError):
         kernels.header_signatures("int ti_x(double y);")
+
+
+def test_context_splits_of_the_decode_kernel(monkeypatch):
+    """The number of runs the decode attention cuts the context into: bounded by the context the
+    launch is sized for, chosen for the typical one, and never just beyond a whole round of the
+    compute units when fewer runs fill one round (12 rows x 8 kv heads: 2 runs, not 3)."""
+    from tinyinfer_amd.ops import attention_bf16 as a
+    monkeypatch.setattr(a, "compute_units", lambda: 256)
+    assert a.decode_splits(8, 8, 16, 4096, 2112) == 4          # 256 workgroups
+    assert a.decode_splits(12, 8, 16, 4096, 2112) == 2         # 192, not 288
+    assert a.decode_splits(24, 8, 16, 4096, 2112) == 1         # 192 in one round, and no merge
+    assert a.decode_splits(64, 8, 16, 4096, 2112) == 1
+    assert a.decode_splits(1, 8, 16, 4096, 2112) == 16         # bounded: 16 blocks of 16 keys a run at least
+    assert a.decode_splits(1, 8, 16, 100, 100) == 1            # a short context is not split
+    assert a.decode_splits(1, 1, 64, 10 ** 6, 10 ** 6) <= a.MAX_SPLITS
+    for rows in range(1, 70):
+        for context in (300, 2000, 9000, 40000):
+            s = a.decode_splits(rows, 8, 16, context)
+            assert 1 <= s <= max(1, min(-(-context // 16) // a.MIN_BLOCKS_PER_SPLIT, a.MAX_SPLITS))

@@ -10,17 +10,43 @@ import ctypes
 import torch
 
 SERVED_HEAD_DIMS = (32, 64, 128)
-TARGET_WORKGROUPS = 256       # one per compute unit: a unit streams about as fast with 4 wavefronts as with 8
 MAX_SPLITS = 64               # the merge kernel's limit
 MIN_BLOCKS_PER_SPLIT = 16     # four 16-key blocks per wavefront at least (fewer, and the merge costs more than the split gains)
+# What a launch of the decode kernel costs, as measured on an MI355X at Qwen3-0.6B's head size (a
+# workgroup per row, kv head and split; a compute unit streams about as fast with one workgroup as
+# with two, so workgroups beyond one per unit wait for a second round):
+SPLIT_PROLOGUE_US = 5.0       # position, table row, query, page ids: before a workgroup's first key arrives
+SPLIT_TOKEN_US = 0.019        # per token of context that one workgroup walks
+SPLIT_MERGE_US = 4.0          # the merge kernel, which a launch without splits does without
 
 
-def decode_splits(n_rows: int, kv_heads: int, heads: int, context: int) -> int:
+def decode_splits(n_rows: int, kv_heads: int, heads: int, context: int, typical: int = 0) -> int:
+    """Into how many runs the decode kernel splits the context.  `context`: the longest context the
+    launch is sized for (it bounds the number); `typical`: the context the choice is made for (a
+    captured graph is sized for the longest sequence, but replayed mostly on shorter ones).
+    The number that makes rounds x (prologue + run) + merge the least, rounds being the
+    workgroups over the compute units, rounded up: 12 rows of 8 kv heads take 2 runs (192
+    workgroups, one round of half the context: 1.67 ms a step) rather than 3 (288: two rounds of
+    a third, 1.90 ms)."""
     parts = (heads // kv_heads + 15) // 16
     base = max(1, n_rows * kv_heads * parts)
-    want = -(-TARGET_WORKGROUPS // base)
     blocks = -(-max(1, context) // 16)
-    return max(1, min(want, blocks // MIN_BLOCKS_PER_SPLIT, MAX_SPLITS))
+    limit = max(1, min(blocks // MIN_BLOCKS_PER_SPLIT, MAX_SPLITS))
+    walk = SPLIT_TOKEN_US * max(1, typical or context)
+    units = compute_units()
+    best, best_cost = 1, None
+    for s in range(1, limit + 1):
+        rounds = -(-base * s // units)
+        cost = rounds * (SPLIT_PROLOGUE_US + walk / s) + (SPLIT_MERGE_US if s > 1 else 0.0)
+        if best_cost is None or cost < best_cost - 1e-9:
+            best, best_cost = s, cost
+    return best
+
+
+def typical_context(ctx) -> int:
+    """The context a launch's splits are chosen for: the step's own, but for a launch sized for more
+    than its step (a graph being captured) no less than half of that size."""
+    return max(ctx.max_context, ctx.split_context // 2) if ctx.split_context > ctx.max_context else ctx.max_context
 
 
 def _ptr(t):
@@ -46,7 +72,7 @@ def run_decode_prepared(ops, ctx, view, qkv, q_w, k_w, eps, inv_freq, rope_table
     win = int(window or 0)
     n = ctx.M
     context = ctx.split_context if win == 0 else min(ctx.split_context, win + 16)
-    S = decode_splits(n, kv_heads, heads, context)
+    S = decode_splits(n, kv_heads, heads, context, min(context, typical_context(ctx)))
     part_o = part_ml = None
     if S > 1:
         part_o = ctx.buf("attn.part_o", (n, heads, S, head_dim), torch.float32)
@@ -133,7 +159,7 @@ def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) 
     if n_dec:
         rows = None if ctx.decode_only else ctx.decode_rows
         context = ctx.split_context if win == 0 else min(ctx.split_context, win + 16)
-        S = decode_splits(n_dec, kv_heads, heads, context)
+        S = decode_splits(n_dec, kv_heads, heads, context, min(context, typical_context(ctx)))
         part_o = part_ml = None
         if S > 1:
             part_o = ctx.buf("attn.part_o", (n_dec, heads, S, head_dim), torch.float32)
