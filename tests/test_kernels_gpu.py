@@ -546,6 +546,40 @@ def test_linear_bf16_mfma_fed_from_memory(ops, M, N, K, ks):
         assert (f64(sw) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 16400, 64), (64, 20000, 1024), (40, 16387, 2048), (33, 17000, 192),
+                                   (48, 16384, 1088)])
+def test_linear_bf16_wide_weight_at_17_to_64_rows(ops, M, N, K):
+    """17 to 64 rows times a weight of 16,384 rows or more (the head of a decode step of many
+    requests): workgroups that keep their share of the token rows in registers and walk over the
+    weight's tiles.  One to four k-blocks per wavefront, four and eight wavefronts, a last tile
+    beyond the matrix, strided token rows; against float64 and against the kernels that take the
+    product when this one is switched off; a row's bits do not depend on the rows beside it."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    g = torch.Generator().manual_seed(M + N + K)
+    wide = (torch.rand(M, K + 24, generator=g) * 2 - 1).to(torch.bfloat16)
+    a = dev(wide)[:, 8:8 + K]
+    w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    ref = ref_linear(wide[:, 8:8 + K], w.cpu())
+    tol = 2e-5 * K
+    lib = ops.lib("gemm_bf16")
+    outs = {}
+    try:
+        for on in (1, 0):
+            lib.ti_gemm_bf16_wide_rows_on(on)
+            out = torch.full((M + 1, N), 7.0, device="cuda")
+            ops.linear(a, w, out[:M], "store")
+            assert (f64(out[:M]) - ref).abs().max() < tol
+            assert bool((out[M] == 7.0).all())
+            outs[on] = out[:M].clone()
+    finally:
+        lib.ti_gemm_bf16_wide_rows_on(1)
+    assert (outs[1] - outs[0]).abs().max() < tol
+    fewer = torch.empty(17, N, device="cuda")
+    ops.linear(a[M - 17:], w, fewer, "store")
+    assert torch.equal(fewer, outs[1][M - 17:])
+
+
 @pytest.mark.parametrize("M,N,K", [(17, 1024, 2048), (64, 1024, 3072), (40, 512, 1024), (33, 96, 1024),
                                    (20, 2048, 1024), (24, 256, 2048), (136, 1024, 2048), (300, 1000, 3072),
                                    (65, 520, 1024), (512, 1024, 2048)])

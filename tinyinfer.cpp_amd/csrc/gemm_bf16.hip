@@ -1362,6 +1362,134 @@ gemm_partials_add_kernel(float* __restrict__ out, const float* __restrict__ part
   out[i] = v;
 }
 
+// 17 to 64 rows times a weight of very many rows (the head: 151,936): the same MFMAs, but a
+// workgroup keeps its share of A in registers (wavefront w of NW the k-blocks w, w + NW, ..., at
+// most four) and walks over tiles of 16 weight rows, blockIdx.x, blockIdx.x + gridDim.x, ...: the
+// weight streams through once, and A is read once per workgroup instead of once per tile (with a
+// workgroup per tile the 9,496 tiles of the head pulled 1.2 GB of A through the caches: 170 us at
+// 64 rows, against ~60 us for the weight alone).  The next tile's weight fragments are asked for
+// before this tile is multiplied.  Stores 32-bit results; a row's bits do not depend on the others.
+template <int MB, int NW>
+__global__ void __launch_bounds__(64 * NW)
+gemm_wide_rows_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, float* __restrict__ out, int M,
+                      int N, int K, long lda) {
+  constexpr int BPW = 4;                                     // k-blocks of 64 per wavefront at most
+  __shared__ __attribute__((aligned(16))) float red[2][NW][MB * 16][MBK_STRIDE];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int nb = K / 64, tiles = (N + 15) / 16;
+  // this wavefront's k-blocks: block j is k-block wave + NW j (one past the end repeats the last
+  // and is not multiplied)
+  int kof[BPW];
+  bool live[BPW];
+#pragma unroll
+  for (int j = 0; j < BPW; ++j) {
+    live[j] = wave + NW * j < nb;
+    kof[j] = min(wave + NW * j, nb - 1) * 64 + g * 8;
+  }
+  uint4 a[BPW][MB][2];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const bf16_t* arow = A + (size_t)min(mb * 16 + r, M - 1) * lda;
+#pragma unroll
+    for (int j = 0; j < BPW; ++j) {
+      a[j][mb][0] = *reinterpret_cast<const uint4*>(arow + kof[j]);
+      a[j][mb][1] = *reinterpret_cast<const uint4*>(arow + kof[j] + 32);
+    }
+  }
+  auto load_w = [&](uint4 (&b)[BPW][2], int tile) {
+    const bf16_t* wrow = W + (size_t)min(tile * 16 + r, N - 1) * K;
+#pragma unroll
+    for (int j = 0; j < BPW; ++j) {
+      b[j][0] = *reinterpret_cast<const uint4*>(wrow + kof[j]);
+      b[j][1] = *reinterpret_cast<const uint4*>(wrow + kof[j] + 32);
+    }
+  };
+  int tile = blockIdx.x;
+  if (tile >= tiles) return;
+  uint4 cur[BPW][2];
+  load_w(cur, tile);
+  for (int it = 0; tile < tiles; ++it, tile += gridDim.x) {
+    uint4 next[BPW][2];
+    load_w(next, min(tile + (int)gridDim.x, tiles - 1));
+    floatx4 acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < BPW; ++j)
+      if (live[j]) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[j][mb][h]),
+                                                              __builtin_bit_cast(bf16x8, cur[j][h]), acc[mb], 0, 0, 0);
+      }
+    // the wavefronts' sums meet in LDS, in the order 0..NW-1; two buffers take turns, so that one
+    // barrier a tile is enough (a wavefront two tiles ahead would have to pass the barrier between)
+    float (*rd)[MB * 16][MBK_STRIDE] = red[it & 1];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) rd[wave][mb * 16 + 4 * g + q][r] = acc[mb][q];
+    __syncthreads();
+    for (int e = tid; e < MB * 16 * 4; e += 64 * NW) {
+      const int row = e >> 2, c = (e & 3) * 4;
+      if (row >= M) continue;
+      float v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < NW; ++w)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] += rd[w][row][c + i];
+      const int n = tile * 16 + c;
+      float* dst = out + (size_t)row * N + n;
+      if (n + 3 < N && (N & 3) == 0) {
+        *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) dst[i] = v[i];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < BPW; ++j) {
+      cur[j][0] = next[j][0];
+      cur[j][1] = next[j][1];
+    }
+  }
+}
+
+static int g_wide_rows = 1;      // a hook for measurements: 0: the kernel above serves nothing
+extern "C" void ti_gemm_bf16_wide_rows_on(int on) { g_wide_rows = on; }
+#define WIDE_ROWS_MIN_N 16384
+
+// whether gemm_wide_rows_kernel takes the product (storing 32-bit results)
+static bool wide_rows_serves(int M, int N, int K, int epi) {
+  return g_wide_rows && epi == TI_EPI_STORE_F32 && M > 16 && M <= 64 && N >= WIDE_ROWS_MIN_N && K % 64 == 0 &&
+         K / 64 <= 4 * 8;
+}
+
+static void launch_wide_rows(const bf16_t* a, const bf16_t* w, float* out, int M, int N, int K, long lda,
+                             hipStream_t s) {
+  const int mb = (M + 15) / 16, tiles = (N + 15) / 16;
+  const bool eight = K / 64 > 4 * 4;                         // more than 16 k-blocks: eight wavefronts
+  int dev = 0, units = 256;
+  hipDeviceProp_t prop;
+  static int cached_units = 0;
+  if (!cached_units) {
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) units = prop.multiProcessorCount;
+    cached_units = units > 0 ? units : 256;
+  }
+  const int grid = min(tiles, cached_units);
+#define TI_GO(MBV)                                                                                   \
+  if (eight) gemm_wide_rows_kernel<MBV, 8><<<grid, 512, 0, s>>>(a, w, out, M, N, K, lda);            \
+  else gemm_wide_rows_kernel<MBV, 4><<<grid, 256, 0, s>>>(a, w, out, M, N, K, lda)
+  if (mb == 2) { TI_GO(2); }
+  else if (mb == 3) { TI_GO(3); }
+  else { TI_GO(4); }
+#undef TI_GO
+}
+
 static int g_add_split = 1;        // a hook for measurements: 0: ti_gemm_bf16_add_split serves nothing
 extern "C" void ti_gemm_bf16_add_split_on(int on) { g_add_split = on; }
 
@@ -1486,6 +1614,11 @@ extern "C" int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int 
   const bf16_t* w = (const bf16_t*)W;
   const bool skinny = M <= 64;
   const bool copied = g_skinny_copy && M <= 16 && K % 64 == 0 && K <= 4096;
+  if (wide_rows_serves(M, N, K, epi)) {
+    launch_wide_rows(a, w, (float*)out, M, N, K, lda, stream);
+    TI_LAUNCH_CHECK();
+    return 0;
+  }
   if (row_per_wave_serves(M, N, K, epi)) {
     int rc_ = 0;
     if (epi == TI_EPI_STORE_F32) rc_ = launch_rows<TI_EPI_STORE_F32>(a, w, out, M, N, K, lda, stream);

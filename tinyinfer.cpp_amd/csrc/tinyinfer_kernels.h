@@ -75,6 +75,7 @@ void ti_gemm_bf16_force_tile(int which);      // 1: 256 x 128, 3: 128 x 64, 6: 6
 void ti_gemm_bf16_skinny_waves(int waves);    // 4 or 8 wavefronts in the kernel for M <= 64
 void ti_gemm_bf16_qkv_prep_min_rows(int rows); // the fewest rows ti_gemm_bf16_qkv_prep serves (17)
 void ti_gemm_bf16_qkv_prep_rows(int rows);    // 128 / 256: the rows of ti_gemm_bf16_qkv_prep's tile; 0: by the shape
+void ti_gemm_bf16_wide_rows_on(int on);       // 0: 17..64 rows times a weight of 16,384 rows or more take the other kernels
 void ti_gemm_bf16_add_split_on(int on);         // 0: ti_gemm_bf16_add_split serves nothing
 void ti_gemm_bf16_use_pipelined(int on);      // 0: the plain tiled kernel for every K
 void ti_gemm_bf16_row_per_wave(int on);        // 0: few tokens and a weight of few rows take the 16-row kernels too
