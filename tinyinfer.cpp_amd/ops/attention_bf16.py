@@ -6,6 +6,7 @@ the generic kernel (`run` returns False)."""
 from __future__ import annotations
 
 import ctypes
+import functools
 
 import torch
 
@@ -28,12 +29,16 @@ def decode_splits(n_rows: int, kv_heads: int, heads: int, context: int, typical:
     workgroups over the compute units, rounded up: 12 rows of 8 kv heads take 2 runs (192
     workgroups, one round of half the context: 1.67 ms a step) rather than 3 (288: two rounds of
     a third, 1.90 ms)."""
+    return _decode_splits(n_rows, kv_heads, heads, context, typical or context, compute_units())
+
+
+@functools.lru_cache(maxsize=512)          # every layer of a step asks the same question
+def _decode_splits(n_rows: int, kv_heads: int, heads: int, context: int, typical: int, units: int) -> int:
     parts = (heads // kv_heads + 15) // 16
     base = max(1, n_rows * kv_heads * parts)
     blocks = -(-max(1, context) // 16)
     limit = max(1, min(blocks // MIN_BLOCKS_PER_SPLIT, MAX_SPLITS))
-    walk = SPLIT_TOKEN_US * max(1, typical or context)
-    units = compute_units()
+    walk = SPLIT_TOKEN_US * max(1, typical)
     best, best_cost = 1, None
     for s in range(1, limit + 1):
         rounds = -(-base * s // units)
@@ -78,10 +83,10 @@ def run_decode_prepared(ops, ctx, view, qkv, q_w, k_w, eps, inv_freq, rope_table
         part_o = ctx.buf("attn.part_o", (n, heads, S, head_dim), torch.float32)
         part_ml = ctx.buf("attn.part_ml", (n, heads, S, 2), torch.float32)
     rc = lib.ti_attention_decode_prepared_bf16(
-        _ptr(qkv), qkv.shape[1], _ptr(q_w), _ptr(k_w), ctypes.c_float(eps), _ptr(inv_freq), _ptr(rope_table),
+        _ptr(qkv), qkv.shape[1], _ptr(q_w), _ptr(k_w), eps, _ptr(inv_freq), _ptr(rope_table),
         0 if rope_table is None else rope_table.shape[0], _ptr(pool), 1 if write_kv else 0,
         _ptr(table), table.shape[1], _ptr(ctx.positions), _ptr(ctx.slots), _ptr(out), _ptr(part_o), _ptr(part_ml),
-        n, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, S, ops._stream())
+        n, heads, kv_heads, head_dim, P, scale, win, S, ops._stream())
     if rc == 3:
         return False
     ops._check(lib, rc, "attention(decode, prepared)")
@@ -143,7 +148,7 @@ def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) 
             part_ml = ctx.buf("attn.portion_ml", (ctx.M, heads, S, 2), torch.float32)
         rc = lib.ti_attention_prefill_paired_bf16(
             _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.tiles_small), _ptr(ctx.entry_meta), _ptr(out),
-            ctx.n_tiles_small, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, ctx.M, _ptr(part_o),
+            ctx.n_tiles_small, heads, kv_heads, head_dim, P, scale, win, ctx.M, _ptr(part_o),
             _ptr(part_ml), S, int(paired), stream)
         if rc == 3:
             return False
@@ -151,7 +156,7 @@ def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) 
     elif ctx.n_tiles:
         rc = lib.ti_attention_prefill_bf16(
             _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.tiles), _ptr(ctx.entry_meta), _ptr(out),
-            ctx.n_tiles, heads, kv_heads, head_dim, P, ctypes.c_float(scale), win, stream)
+            ctx.n_tiles, heads, kv_heads, head_dim, P, scale, win, stream)
         if rc == 3:
             return False
         ops._check(lib, rc, "attention(prefill)")
@@ -166,7 +171,7 @@ def run(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window) 
             part_ml = ctx.buf("attn.part_ml", (n_dec, heads, S, 2), torch.float32)
         rc = lib.ti_attention_decode_bf16(
             _ptr(q), _ptr(pool), _ptr(table), table.shape[1], _ptr(ctx.positions), _ptr(ctx.slots), _ptr(rows),
-            _ptr(out), _ptr(part_o), _ptr(part_ml), n_dec, heads, kv_heads, head_dim, P, ctypes.c_float(scale),
+            _ptr(out), _ptr(part_o), _ptr(part_ml), n_dec, heads, kv_heads, head_dim, P, scale,
             win, S, stream)
         if rc == 3:
             return False

@@ -180,7 +180,7 @@ class Ops:
             return
         out, ks = pend
         lib = self.lib("gemm_bf16")
-        rc = lib.ti_gemm_bf16_partials_add(_ptr(out), _ptr(self._partials), ks, ctypes.c_long(out.numel()),
+        rc = lib.ti_gemm_bf16_partials_add(_ptr(out), _ptr(self._partials), ks, out.numel(),
                                            self._raw_stream())
         self._check(lib, rc, "linear(bf16): adding the partial sums")
 
@@ -218,14 +218,14 @@ class Ops:
         if pend is not None and rows is None and pend[0].data_ptr() == x.data_ptr() and pend[0].shape == x.shape:
             # the product before left its partial sums: this norm adds them on its way
             rc = lib.ti_rmsnorm_add_partials(_code(out.dtype), _ptr(x), _ptr(self._partials), pend[1], _ptr(w),
-                                             _ptr(out), n, H, ctypes.c_float(eps), self._raw_stream())
+                                             _ptr(out), n, H, eps, self._raw_stream())
             if rc == 0:
                 self._pending = None
                 return
             if rc != 3:
                 self._check(lib, rc, "rmsnorm")
         rc = lib.ti_rmsnorm(_code(out.dtype), _ptr(x), _ptr(w), _ptr(rows), _ptr(out), n, H,
-                            ctypes.c_float(eps), self._stream())
+                            eps, self._stream())
         self._check(lib, rc, "rmsnorm")
 
     def rope_neox(self, x, positions, inv_freq):
@@ -238,7 +238,7 @@ class Ops:
             raise KernelError("rope: inv_freq must be float32 [hd/2], positions int32")
         lib = self.lib("core")
         rc = lib.ti_rope_neox(_ptr(x), _ptr(positions), _ptr(inv_freq), M, heads, hd,
-                              ctypes.c_long(x.stride(0)), self._stream())
+                              x.stride(0), self._stream())
         self._check(lib, rc, "rope")
 
     def rope_table(self, inv_freq, n_pos):
@@ -280,7 +280,7 @@ class Ops:
             _code(q_out.dtype), _ptr(qkv), _ptr(q_w), _ptr(k_w), _ptr(inv_freq), _ptr(rope_table),
             0 if rope_table is None else rope_table.shape[0], _ptr(positions), _ptr(slots),
             _ptr(view.table), view.table.shape[1], _ptr(pool), _ptr(q_out), M, heads, kv_heads, head_dim,
-            pool.shape[3], ctypes.c_float(eps), self._stream())
+            pool.shape[3], eps, self._stream())
         self._check(lib, rc, "qk_norm_rope_kv_write")
 
     def qk_norm_inplace(self, qkv, q_w, k_w, eps, heads, kv_heads, head_dim):
@@ -296,7 +296,7 @@ class Ops:
                 raise KernelError("qk_norm_inplace: norm weights must be float32 [head_dim]")
         lib = self.lib("core")
         rc = lib.ti_qk_norm_inplace(_ptr(qkv), qkv.shape[1], _ptr(q_w), _ptr(k_w), qkv.shape[0], heads, kv_heads,
-                                    head_dim, ctypes.c_float(eps), self._stream())
+                                    head_dim, eps, self._stream())
         self._check(lib, rc, "qk_norm_inplace")
 
     # ---------------------------------------------------------- matrix products
@@ -327,7 +327,7 @@ class Ops:
         if code == BF16 and self.use_fast_gemm and self._linear_bf16(a, w, out, epi, M, N, K, may_defer):
             return
         lib = self.lib("gemm_generic")
-        rc = lib.ti_gemm_generic(code, _ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi,
+        rc = lib.ti_gemm_generic(code, _ptr(a), _ptr(w), _ptr(out), M, N, K, a.stride(0), epi,
                                  self._stream())
         self._check(lib, rc, "linear")
 
@@ -364,7 +364,7 @@ class Ops:
                               f"[pages,2,{kv_heads},P,{head_dim}] of bfloat16")
         lib = self.lib("gemm_bf16")
         rc = lib.ti_gemm_bf16_qkv_prep(
-            _ptr(a), _ptr(w), M, K, ctypes.c_long(a.stride(0)), _ptr(q_w), _ptr(k_w), ctypes.c_float(eps),
+            _ptr(a), _ptr(w), M, K, a.stride(0), _ptr(q_w), _ptr(k_w), eps,
             _ptr(inv_freq), _ptr(rope_table), 0 if rope_table is None else rope_table.shape[0],
             _ptr(positions), _ptr(slots), _ptr(view.table), view.table.shape[1], _ptr(pool), _ptr(q_out),
             heads, kv_heads, head_dim, pool.shape[3], self._stream())
@@ -398,7 +398,7 @@ class Ops:
         if out.shape != (M, N) or out.dtype != want or not out.is_contiguous():
             raise KernelError(f"linear[{epilogue}]: out {tuple(out.shape)} {out.dtype} does not fit [{M},{N}] {want}")
         lib = self.lib("gemm_bf16")
-        rc = lib.ti_gemm_bf16_normed(_ptr(a.x), _ptr(a.weight), ctypes.c_float(a.eps), _ptr(w), _ptr(out),
+        rc = lib.ti_gemm_bf16_normed(_ptr(a.x), _ptr(a.weight), a.eps, _ptr(w), _ptr(out),
                                      M, N, K, EPI[epilogue], self._stream())
         if rc == 3:
             return False
@@ -419,16 +419,15 @@ class Ops:
             # 1: the sums are left for the next norm; 2: the same product, added at once
             defer = 0 if not may_defer else 1 if self.use_deferred_add else 2
             splits = ctypes.c_int(0)
-            rc = lib.ti_gemm_bf16_add_split(_ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi,
-                                          _ptr(ws), ctypes.c_long(self.PARTIALS_BYTES), defer,
-                                          ctypes.byref(splits), stream)
+            rc = lib.ti_gemm_bf16_add_split(_ptr(a), _ptr(w), _ptr(out), M, N, K, a.stride(0), epi, _ptr(ws),
+                                            self.PARTIALS_BYTES, defer, ctypes.byref(splits), stream)
             if rc == 0:
                 if splits.value:
                     self._pending = (out, splits.value)
                 return True
             if rc != 3:
                 self._check(lib, rc, "linear(bf16, split K)")
-        rc = lib.ti_gemm_bf16(_ptr(a), _ptr(w), _ptr(out), M, N, K, ctypes.c_long(a.stride(0)), epi, self._stream())
+        rc = lib.ti_gemm_bf16(_ptr(a), _ptr(w), _ptr(out), M, N, K, a.stride(0), epi, self._stream())
         if rc == 3:          # "shape not served": not an error
             return False
         self._check(lib, rc, "linear(bf16)")
@@ -447,7 +446,7 @@ class Ops:
         lib = self.lib("attention_generic")
         rc = lib.ti_attention_rows(_code(q.dtype), _ptr(q), _ptr(pool), _ptr(table), table.shape[1],
                                    _ptr(positions), _ptr(slots), _ptr(out), M, heads, kv_heads, head_dim,
-                                   pool.shape[3], ctypes.c_float(scale), int(window or 0), self._stream())
+                                   pool.shape[3], scale, int(window or 0), self._stream())
         self._check(lib, rc, "attention")
 
     def attention(self, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window):
