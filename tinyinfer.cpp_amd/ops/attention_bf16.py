@@ -5,7 +5,6 @@ prefill kernel.  Head sizes or page sizes the kernels do not serve are left to
 the generic kernel (`run` returns False)."""
 from __future__ import annotations
 
-import ctypes
 import functools
 
 import torch
