@@ -546,6 +546,53 @@ def test_linear_bf16_mfma_fed_from_memory(ops, M, N, K, ks):
         assert (f64(sw) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
 
 
+@pytest.mark.parametrize("M", [17, 33, 64])
+@pytest.mark.parametrize("epilogue", ["store", "add", "store_act", "swiglu"])
+def test_linear_bf16_large_weight_at_17_to_64_rows(ops, M, epilogue):
+    """17 to 64 rows times a weight of 16 Mi elements: from rows x elements = 280 Mi on the tiled
+    kernels take the product (their tile partly empty), below that the kernels whose workgroups
+    own 16 weight rows.  Both sides of the rule and the rule switched off agree with float64 and
+    with one another up to rounding; the adding epilogue with its sums left to a later kernel too."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    N, K = 8192, 2048
+    g = torch.Generator().manual_seed(M)
+    a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    ref = ref_linear(a.cpu(), w.cpu())
+    tol = 2e-5 * K
+    base = torch.randn(M, N, generator=g)
+    if epilogue == "swiglu":
+        gte, up = ref[:, :N // 2], ref[:, N // 2:]
+        want = gte / (1 + torch.exp(-gte)) * up
+        bound = 0.005 * want.abs().max() + 10 * tol
+    elif epilogue == "add":
+        want, bound = ref + f64(base), tol
+    else:
+        want, bound = ref, tol if epilogue == "store" else 0.005 * ref.abs().max() + tol
+    lib = ops.lib("gemm_bf16")
+    outs = []
+    try:
+        for rule in (280 << 20, 1 << 60, 0):              # as shipped, never, always
+            lib.ti_gemm_bf16_tiled_from(rule)
+            if epilogue == "swiglu":
+                out = torch.empty(M, N // 2, device="cuda", dtype=torch.bfloat16)
+            elif epilogue == "store_act":
+                out = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+            else:
+                out = dev(base.clone())
+            ops.linear(a, w, out, epilogue, may_defer=True)
+            ops.flush()
+            assert (f64(out) - want).abs().max() < bound
+            outs.append(f64(out))
+    finally:
+        lib.ti_gemm_bf16_tiled_from(280 << 20)
+    assert (outs[1] - outs[2]).abs().max() < 2 * bound
+    # 17 rows x 16 Mi lie under the rule, 33 and 64 over it
+    same_as = outs[1] if M == 17 else outs[2]
+    assert torch.equal(outs[0], same_as)
+
+
 @pytest.mark.parametrize("M,N,K", [(17, 16400, 64), (64, 20000, 1024), (40, 16387, 2048), (33, 17000, 192),
                                    (48, 16384, 1088)])
 def test_linear_bf16_wide_weight_at_17_to_64_rows(ops, M, N, K):

@@ -1058,6 +1058,7 @@ static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M,
   const long mid = (long)((M + 127) / 128) * ((N * cols + 63) / 64);
   const bool whole_rounds = big >= 256 && (big % 256 == 0 || big % 256 >= 192);
   int tile = (big >= 1024 || whole_rounds) ? 1 : (mid >= 512 ? 3 : 6);
+  if (M <= 64 && tile == 1) tile = 6;                // few rows times a wide weight: no 256-row tile
   if (g_force_tile) tile = g_force_tile;
   if (tile == 1) return launch_pipelined<256, 128, 4, 2, EPI>(A, W, out, M, N, K, lda, s);
   if constexpr (EPI != TI_EPI_SWIGLU)                // a SwiGLU wavefront needs two column tiles
@@ -1490,6 +1491,20 @@ static void launch_wide_rows(const bf16_t* a, const bf16_t* w, float* out, int M
 #undef TI_GO
 }
 
+// 17..64 rows: the kernels whose workgroups own 16 weight rows pull all token rows in once per 16
+// rows, (1 + M / 16) times the weight's bytes through the caches.  Under a small weight that hides
+// behind the launch; under a large one it is what the product waits for (Qwen3-8B's gate/up at 64
+// rows: 110 us, 1.8 TB/s of weights), and the tiled kernels, which read the token rows once per
+// 64 rows of the weight and take about the same time for 17 rows as for 64, are faster although
+// their tile is partly empty (50 us).  Measured at the widths of Qwen3-0.6B to 8B: the tiled
+// kernels win from about rows x weight elements = 280 Mi on.
+static long g_tiled_from = 280L << 20;           // rows x weight elements from which such steps take the tiled kernels
+extern "C" void ti_gemm_bf16_tiled_from(long rows_times_elems) { g_tiled_from = rows_times_elems; }
+static bool large_weight(int M, int N, int K, int epi) {
+  const long rows = (epi == TI_EPI_SWIGLU) ? 2L * N : (long)N;
+  return M > 16 && M <= 64 && K % PBK == 0 && rows * K * M >= g_tiled_from;
+}
+
 static int g_add_split = 1;        // a hook for measurements: 0: ti_gemm_bf16_add_split serves nothing
 extern "C" void ti_gemm_bf16_add_split_on(int on) { g_add_split = on; }
 
@@ -1532,7 +1547,7 @@ extern "C" int ti_gemm_bf16_add_split(const void* A, const void* W, void* out, i
   TI_REQUIRE(splits != nullptr, "gemm_bf16_add_split: splits must point to an int");
   *splits = 0;
   int KS = 1;
-  const bool small = M <= 64;
+  const bool small = M <= 64 && !(large_weight(M, N, K, epi) && g_use_pipelined);
   if (g_add_split && epi == TI_EPI_ADD_F32 && partial && M > 16 && K % 64 == 0 && lda % 8 == 0 &&
       !((uintptr_t)A & 15) && !((uintptr_t)W & 15) && !((uintptr_t)partial & 15) && (small || g_use_pipelined)) {
     // split K until the launch has about a workgroup per compute unit
@@ -1612,7 +1627,7 @@ extern "C" int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int 
   if (M == 0) return 0;
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
-  const bool skinny = M <= 64;
+  const bool skinny = M <= 64 && !(large_weight(M, N, K, epi) && g_use_pipelined);
   const bool copied = g_skinny_copy && M <= 16 && K % 64 == 0 && K <= 4096;
   if (wide_rows_serves(M, N, K, epi)) {
     launch_wide_rows(a, w, (float*)out, M, N, K, lda, stream);

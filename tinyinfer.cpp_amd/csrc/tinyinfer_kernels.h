@@ -76,6 +76,7 @@ void ti_gemm_bf16_skinny_waves(int waves);    // 4 or 8 wavefronts in the kernel
 void ti_gemm_bf16_qkv_prep_min_rows(int rows); // the fewest rows ti_gemm_bf16_qkv_prep serves (17)
 void ti_gemm_bf16_qkv_prep_rows(int rows);    // 128 / 256: the rows of ti_gemm_bf16_qkv_prep's tile; 0: by the shape
 void ti_gemm_bf16_wide_rows_on(int on);       // 0: 17..64 rows times a weight of 16,384 rows or more take the other kernels
+void ti_gemm_bf16_tiled_from(long rows_times_elems); // 17..64 rows x weight elements from which they take the tiled kernels
 void ti_gemm_bf16_add_split_on(int on);         // 0: ti_gemm_bf16_add_split serves nothing
 void ti_gemm_bf16_use_pipelined(int on);      // 0: the plain tiled kernel for every K
 void ti_gemm_bf16_row_per_wave(int on);        // 0: few tokens and a weight of few rows take the 16-row kernels too
