@@ -104,6 +104,54 @@ def test_greedy_generation_with_graphs_equals_eager(model_folders, dtype):
             fed[r] += 1
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_of_a_repeated_shape_replay_from_graphs(model_folders, dtype):
+    """A prompt that arrives in equal portions beside a decoding request repeats the shape of
+    its step: the second time the shape is captured, from then on replayed.  Every step's
+    logits equal those of an engine that runs eagerly, bit for bit, replay after replay, with
+    eager steps (another shape, and the same one through `step`) in between; and a shape that
+    comes once is never captured."""
+    import tinyinfer_amd as ti
+    d = model_folders("D", "bfloat16", True)
+    e1 = ti.Engine.from_folder(d, dtype, page_size=16, max_tokens=512, max_requests=3, max_seq=256)
+    e2 = ti.Engine.from_folder(d, dtype, page_size=16, max_tokens=512, max_requests=3, max_seq=256)
+    toks = {"x": random_tokens(200, 333, 1), "y": random_tokens(60, 333, 2)}
+    for e in (e1, e2):
+        e.step([ti.StepEntry("y", toks["y"][:9], [8])])
+    fed = {"x": 0, "y": 9}
+    shape = None
+    for i in range(14):
+        entries = [ti.StepEntry("y", [toks["y"][fed["y"]]], [0]),
+                   ti.StepEntry("x", toks["x"][fed["x"]:fed["x"] + 12], [0, 11])]
+        a = e1.step(entries).clone()
+        if i % 5 == 3:
+            b = e2.step(entries).clone()               # the same shape, eagerly, between replays
+        else:
+            b = e2.step_graph(entries).clone()
+        assert torch.equal(a, b), i
+        fed["x"] += 12
+        fed["y"] += 1
+        shape = tuple((len(e.tokens), tuple(e.want)) for e in entries)
+        if i == 6:                                     # another shape, once: eager, not captured
+            odd = [ti.StepEntry("x", toks["x"][fed["x"]:fed["x"] + 5], [4])]
+            assert torch.equal(e1.step(odd), e2.step_graph(odd))
+            fed["x"] += 5
+    assert shape in e2._graphs and len([k for k in e2._graphs if not isinstance(k, int)]) == 1
+    assert not e1._graphs
+    # the captured shape with other requests in it: a new request takes the portion's place
+    for e in (e1, e2):
+        e.release("x")
+    fed["z"] = 0
+    toks["z"] = random_tokens(40, 333, 3)
+    for i in range(3):
+        entries = [ti.StepEntry("y", [toks["y"][fed["y"]]], [0]),
+                   ti.StepEntry("z", toks["z"][fed["z"]:fed["z"] + 12], [0, 11])]
+        assert torch.equal(e1.step(entries), e2.step_graph(entries)), i
+        fed["z"] += 12
+        fed["y"] += 1
+    e2.cache.check()
+
+
 def test_preemption_recomputes_and_changes_nothing(model_folders):
     """With too few pages the youngest request gives way and is fed again later;
     in 32-bit the tokens are the ones a roomy pool gives."""

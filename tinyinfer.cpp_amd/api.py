@@ -44,7 +44,7 @@ def run_requests(engine: Engine, scheduler: Scheduler, sampler: Optional[Sampler
                              (e.n_tokens - 1,) if e.sample else ()) for e in plan.entries]
         decode_only = all(e.n_tokens == 1 for e in plan.entries)
         t0 = time.perf_counter()
-        if use_graph and decode_only:
+        if use_graph:
             logits = engine.step_graph(entries)
         else:
             logits = engine.step(entries)

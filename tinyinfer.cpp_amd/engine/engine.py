@@ -27,6 +27,8 @@ from ..weights.loader import DTYPES
 
 PREFILL_TILE_Q = 128    # query rows per work item of the tiled attention kernels
 PREFILL_TILE_SMALL = 64  # and of the kernel that pairs a tile of many keys with one of few
+STEP_GRAPH_AFTER = 2              # a step's shape is captured when it comes for this many times ...
+MAX_STEP_GRAPHS = 32              # ... and this many such graphs are kept
 PAGE_SCATTER_WINDOW = 512  # free pages are first handed out shuffled within windows of this many (see PagePool)
 
 
@@ -136,7 +138,8 @@ class Engine:
         self._meta_events: List[Optional[torch.cuda.Event]] = []
         self._meta_turn = 0
         self.steps_run = 0
-        self._graphs: Dict[int, "_DecodeGraph"] = {}
+        self._graphs: Dict[object, "_DecodeGraph"] = {}       # batch size, or a step's shape -> its graph
+        self._shapes_seen: Dict[tuple, int] = {}
 
     # ------------------------------------------------------------- construction
     @classmethod
@@ -433,24 +436,41 @@ class Engine:
                 self.cache.commit(e.request, len(e.tokens))
         self.steps_run += 1
 
-    # ------------------------------------------------------------ decode graphs
+    # ------------------------------------------------------------------ graphs
     def step_graph(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
-        """`step` for a batch of single tokens that each want their logits, replayed
-        from a HIP graph captured once per batch size (the reference keys its CUDA
-        graphs the same way: /root/reference/src/inference.cu:267-295).  Anything
-        else runs through `step`.
+        """`step`, replayed from a captured HIP graph where there is one.  A batch of single
+        tokens that each want their logits has a graph per batch size, captured the first time
+        (the reference keys its CUDA graphs the same way: /root/reference/src/inference.cu:267-295).
+        Any other step has a shape: the token count and the wanted places of every entry, in
+        order (a prompt arriving in equal portions beside the same decoding requests repeats
+        its shape step after step); a shape is captured when it comes for the
+        `STEP_GRAPH_AFTER`-th time, the `MAX_STEP_GRAPHS` most recently used are kept, and until
+        then the step runs through `step`.
 
-        What a replay reads is at fixed addresses: the graph has its own metadata
-        buffer (tokens, positions, block-table rows: refreshed by one copy before
-        each replay) and its own workspace; loop bounds are read on the device,
-        and the number of context splits is sized for `max_seq`, not for the
+        What a replay reads is at fixed addresses: the graph has its own metadata buffer
+        (tokens, positions, work lists, block-table rows: refreshed by one copy before each
+        replay) and its own workspace; loop bounds are read on the device, and the numbers of
+        runs the attention cuts contexts into are sized for the longest sequence, not for the
         step.  Sampling stays outside the graph."""
-        if not all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries):
-            return self.step(entries)
-        R = len(entries)
-        rec = self._graphs.get(R)
+        if all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries):
+            key = len(entries)
+        else:
+            key = tuple((len(e.tokens), tuple(e.want)) for e in entries)
+        rec = self._graphs.get(key)
         if rec is None:
-            return self._capture(entries)
+            if not isinstance(key, int):
+                if len(self._shapes_seen) > 4096:
+                    self._shapes_seen.clear()
+                seen = self._shapes_seen[key] = self._shapes_seen.get(key, 0) + 1
+                if seen < STEP_GRAPH_AFTER:
+                    return self.step(entries)
+                del self._shapes_seen[key]
+                shapes = [k for k in self._graphs if not isinstance(k, int)]
+                if len(shapes) >= MAX_STEP_GRAPHS:
+                    del self._graphs[shapes[0]]            # the one unused for longest (see below)
+            return self._capture(entries, key)
+        if not isinstance(key, int):
+            self._graphs[key] = self._graphs.pop(key)       # most recently used last
         saved = self._ws
         self._ws = rec.workspace
         try:
@@ -461,16 +481,22 @@ class Engine:
         self.finish(ctx)
         return rec.logits
 
-    def _capture(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _capture(self, entries: Sequence[StepEntry], key) -> Optional[torch.Tensor]:
         R = len(entries)
         paged = len(self.cache.paged_groups())
+        M = sum(len(e.tokens) for e in entries)
+        n_lists = sum(-(-len(e.tokens) // PREFILL_TILE_Q) + -(-len(e.tokens) // PREFILL_TILE_SMALL) for e in entries)
         rec = _DecodeGraph()
-        rec.meta = torch.empty(8 * R + paged * R * self.table_width + 64, dtype=torch.int32, device=self.device)
+        # what `prepare` lays out: tokens, positions, slots, wanted rows, entries, work lists, tables
+        rec.meta = torch.empty(3 * M + sum(len(e.want) for e in entries) + 4 * R + 2 * n_lists + R
+                               + paged * R * self.table_width + 64, dtype=torch.int32, device=self.device)
         saved = self._ws
         self._ws = rec.workspace
         try:
             ctx = self.prepare(entries, meta_dev=rec.meta)
             ctx.split_context = self.max_seq
+            if ctx.n_tiles:
+                ctx.portion_context = max(ctx.portion_context, self.max_seq // 2)
             # a first run outside the graph: it computes this step's result and makes every
             # workspace buffer the graph will use
             side = torch.cuda.Stream()
@@ -487,12 +513,12 @@ class Engine:
         # capture records, it does not run: the first run above already wrote this step's
         # keys, values and logits, and a replay would write the same again
         self.finish(ctx)
-        self._graphs[R] = rec
+        self._graphs[key] = rec
         return rec.logits
 
 
 class _DecodeGraph:
-    """A captured decode step for one batch size, with the buffers it reads and writes."""
+    """A captured step (one batch size of single tokens, or one shape), with the buffers it reads and writes."""
 
     def __init__(self):
         self.graph = None
