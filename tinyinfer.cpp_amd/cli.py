@@ -22,7 +22,7 @@ USAGE = """usage: {prog} -m model_dir -n max_tokens -p "prompt" [-p "prompt2" ..
   [-t temp] [--top-k K] [--top-p P] [--seed S] [--max-seq N] [--cuda-graph] [--verbose]
   [--dtype bfloat16|float32] [--page-size P] [--chunk N] [--max-batched-tokens N]
   a prompt is a list of token ids ("1,2,3"), or text if the model folder has a tokenizer.json
-  --cuda-graph (alias --graph): replay the decode phase from a captured graph (off by default)
+  --cuda-graph (alias --graph): replay decode steps, and other steps whose shape repeats, from captured graphs (off by default)
 """
 
 
