@@ -152,6 +152,29 @@ def test_steps_of_a_repeated_shape_replay_from_graphs(model_folders, dtype):
     e2.cache.check()
 
 
+def test_only_the_most_recent_step_shapes_keep_their_graphs(model_folders, monkeypatch):
+    """With room for one shape's graph, two shapes in turn push one another out and are captured
+    again; the logits stay those of eager steps."""
+    import tinyinfer_amd as ti
+    from tinyinfer_amd.engine import engine as engine_module
+    monkeypatch.setattr(engine_module, "MAX_STEP_GRAPHS", 1)
+    d = model_folders("D", "bfloat16", True)
+    e1 = ti.Engine.from_folder(d, "bfloat16", page_size=16, max_tokens=512, max_requests=2, max_seq=256)
+    e2 = ti.Engine.from_folder(d, "bfloat16", page_size=16, max_tokens=512, max_requests=2, max_seq=256)
+    toks = random_tokens(240, 333, 9)
+    fed = 0
+    captured = set()
+    for i in range(16):
+        n = (7, 11)[(i // 2) % 2]                      # two steps of one shape, two of the other, ...
+        entries = [ti.StepEntry("x", toks[fed:fed + n], [n - 1])]
+        assert torch.equal(e1.step(entries), e2.step_graph(entries)), i
+        fed += n
+        shapes = [k for k in e2._graphs if not isinstance(k, int)]
+        assert len(shapes) <= 1
+        captured |= set(shapes)
+    assert len(captured) == 2
+
+
 def test_preemption_recomputes_and_changes_nothing(model_folders):
     """With too few pages the youngest request gives way and is fed again later;
     in 32-bit the tokens are the ones a roomy pool gives."""
