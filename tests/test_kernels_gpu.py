@@ -593,6 +593,37 @@ def test_linear_bf16_large_weight_at_17_to_64_rows(ops, M, epilogue):
     assert torch.equal(outs[0], same_as)
 
 
+def test_linear_bf16_large_weight_at_13_to_16_rows(ops):
+    """13 to 16 rows times a weight of 48 Mi elements: over the rule for these row counts (rows x
+    elements of 600 Mi or more), so the tiled kernels take the product and a norm in front becomes
+    a kernel of its own; 12 rows stay with the kernels that take the norm in.  Against float64,
+    and the rule switched off."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    from tinyinfer_amd.ops.kernels import NormedRows
+    N, K = 12288, 4096
+    g = torch.Generator().manual_seed(3)
+    w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    nw = dev(torch.rand(K, generator=g) + 0.5)
+    lib = ops.lib("gemm_bf16")
+    for M in (12, 13, 16):
+        x = dev(torch.randn(M, K, generator=g))
+        h_ref = ref_rmsnorm(x, nw, 1e-6).to(torch.bfloat16)
+        ref = ref_linear(h_ref, w.cpu())
+        outs = []
+        try:
+            for rule in (280 << 20, 1 << 60):
+                lib.ti_gemm_bf16_tiled_from(rule)
+                h = torch.empty(M, K, device="cuda", dtype=torch.bfloat16)
+                out = torch.empty(M, N, device="cuda")
+                ops.linear(NormedRows(x, nw, 1e-6, h), w, out, "store")
+                assert (f64(out) - ref).abs().max() < 0.01 * ref.abs().max() + 2e-5 * K
+                outs.append(out)
+        finally:
+            lib.ti_gemm_bf16_tiled_from(280 << 20)
+        assert torch.equal(outs[0], outs[1]) == (M == 12), M
+
+
 @pytest.mark.parametrize("M,N,K", [(17, 16400, 64), (64, 20000, 1024), (40, 16387, 2048), (33, 17000, 192),
                                    (48, 16384, 1088)])
 def test_linear_bf16_wide_weight_at_17_to_64_rows(ops, M, N, K):

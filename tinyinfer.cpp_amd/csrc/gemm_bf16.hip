@@ -1115,6 +1115,33 @@ static void launch_tiled(const bf16_t* A, const bf16_t* W, void* out, int M, int
   gemm_tiled_kernel<EPI><<<grid, 256, 0, s>>>(A, W, out, M, N, K, lda);
 }
 
+// 1: the pipelined tiled kernel for M > 64 (default); 0: the plain tiled kernel (for comparison)
+static int g_use_pipelined = 1;
+
+// 17..64 rows: the kernels whose workgroups own 16 weight rows pull all token rows in once per 16
+// rows, (1 + M / 16) times the weight's bytes through the caches.  Under a small weight that hides
+// behind the launch; under a large one it is what the product waits for (Qwen3-8B's gate/up at 64
+// rows: 110 us, 1.8 TB/s of weights), and the tiled kernels, which read the token rows once per
+// 64 rows of the weight and take about the same time for 17 rows as for 64, are faster although
+// their tile is partly empty (50 us).  Measured at the widths of Qwen3-0.6B to 8B: the tiled
+// kernels win from about rows x weight elements = 280 Mi on.  13..16 rows: the 16-row kernels
+// multiply without the matrix cores and under a large weight that is what they wait for (8B's
+// gate/up at 16 rows: 72 us with the norm inside, 62 us as norm + tiled product; Qwen3-4B's: 50
+// against 37 us); from rows x weight elements = 600 Mi on these take the tiled kernels too, and
+// the norm a kernel of its own.  (At 9 to 12 rows that was measured as well, and loses.)
+static long g_tiled_from = 280L << 20;           // 17..64 rows x weight elements from which steps take the tiled kernels
+static long g_tiled_from_16 = 600L << 20;        // the same for 13..16 rows
+extern "C" void ti_gemm_bf16_tiled_from(long rows_times_elems) {
+  g_tiled_from = rows_times_elems;
+  g_tiled_from_16 = rows_times_elems >= (280L << 20) && rows_times_elems < (1L << 59) ? rows_times_elems / 280 * 600
+                                                                                     : rows_times_elems;
+}
+static bool large_weight(int M, int N, int K, int epi) {
+  const long rows = (epi == TI_EPI_SWIGLU) ? 2L * N : (long)N;
+  if (M <= 12 || M > 64 || K % PBK != 0) return false;
+  return rows * K * M >= (M <= 16 ? g_tiled_from_16 : g_tiled_from);
+}
+
 // 1 (default): up to GR_MMAX tokens and a weight of fewer than GR_ROWS_BELOW rows take the kernel
 // with a weight row per wavefront; 0: they take the kernels whose workgroups own 16 rows
 #define GR_MMAX 8
@@ -1193,6 +1220,10 @@ extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, c
     ti_set_error("gemm_bf16_normed: M=%d N=%d is left to the kernel with a weight row per wavefront", M, N);
     return 3;
   }
+  if (large_weight(M, N, K, epi) && g_use_pipelined) {
+    ti_set_error("gemm_bf16_normed: M=%d times a weight of %d x %d is left to the tiled kernels", M, N, K);
+    return 3;
+  }
   if (M == 0) return 0;
   const bf16_t* w = (const bf16_t*)W;
   const int grid = (epi == TI_EPI_SWIGLU) ? (N + 7) / 8 : (N + 15) / 16;
@@ -1242,8 +1273,6 @@ static int launch_skinny_copied(const bf16_t* A, const bf16_t* W, void* out, int
               : launch_staged<CopyProducer, EPI, 4, 4>("gemm_bf16", pr, W, out, M, N, K, grid, s);
 }
 
-static int g_use_pipelined = 1;
-// 1: the pipelined tiled kernel for M > 64 (default); 0: the plain tiled kernel (for comparison)
 // ---------------------------------------------------------------------------------------------
 // 17 to 64 rows: 16x16x32 MFMAs fed straight from memory.  A workgroup takes 16 rows of W (16
 // output columns; SwiGLU: 8 gate and 8 up rows) and a range of K; its four wavefronts take the
@@ -1491,20 +1520,6 @@ static void launch_wide_rows(const bf16_t* a, const bf16_t* w, float* out, int M
 #undef TI_GO
 }
 
-// 17..64 rows: the kernels whose workgroups own 16 weight rows pull all token rows in once per 16
-// rows, (1 + M / 16) times the weight's bytes through the caches.  Under a small weight that hides
-// behind the launch; under a large one it is what the product waits for (Qwen3-8B's gate/up at 64
-// rows: 110 us, 1.8 TB/s of weights), and the tiled kernels, which read the token rows once per
-// 64 rows of the weight and take about the same time for 17 rows as for 64, are faster although
-// their tile is partly empty (50 us).  Measured at the widths of Qwen3-0.6B to 8B: the tiled
-// kernels win from about rows x weight elements = 280 Mi on.
-static long g_tiled_from = 280L << 20;           // rows x weight elements from which such steps take the tiled kernels
-extern "C" void ti_gemm_bf16_tiled_from(long rows_times_elems) { g_tiled_from = rows_times_elems; }
-static bool large_weight(int M, int N, int K, int epi) {
-  const long rows = (epi == TI_EPI_SWIGLU) ? 2L * N : (long)N;
-  return M > 16 && M <= 64 && K % PBK == 0 && rows * K * M >= g_tiled_from;
-}
-
 static int g_add_split = 1;        // a hook for measurements: 0: ti_gemm_bf16_add_split serves nothing
 extern "C" void ti_gemm_bf16_add_split_on(int on) { g_add_split = on; }
 
@@ -1628,7 +1643,7 @@ extern "C" int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int 
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
   const bool skinny = M <= 64 && !(large_weight(M, N, K, epi) && g_use_pipelined);
-  const bool copied = g_skinny_copy && M <= 16 && K % 64 == 0 && K <= 4096;
+  const bool copied = g_skinny_copy && M <= 16 && K % 64 == 0 && K <= 4096 && skinny;
   if (wide_rows_serves(M, N, K, epi)) {
     launch_wide_rows(a, w, (float*)out, M, N, K, lda, stream);
     TI_LAUNCH_CHECK();
