@@ -42,7 +42,7 @@ def test_pages_scattered_within_windows_are_a_permutation():
     for i in range(0, 70, 16):
         assert sorted(taken[i:i + 16]) == list(range(i, min(i + 16, 70)))
     assert taken != list(range(70))
-    assert PagePool(70, scatter_window=16)._free == PagePool(70, scatter_window=16)._free   # a fixed order
+    assert PagePool(70, scatter_window=16).free_list() == PagePool(70, scatter_window=16).free_list()   # a fixed order
     with pytest.raises(OutOfPages):
         pool.take()
     pool.give_back(taken[3])
@@ -81,7 +81,7 @@ def test_double_free_and_unknown_requests_are_errors():
     with pytest.raises(CacheError):
         m.release("a")
     with pytest.raises(CacheError):
-        m.pool_give_back = m.groups[0].pool.give_back(0)          # a page that is not held
+        m.groups[0].pool.give_back(0)                             # a page that is not held
     for r in "abcd":
         m.admit(r)
     with pytest.raises(CacheError):
@@ -119,7 +119,7 @@ def test_state_slots_are_cleared_on_admission():
     m = manager(groups=((FULL, 1), (StateNeed((3, 5)), 2)), slots=2)
     s = m.admit("a")
     assert m.slots_to_clear == [s]
-    m.slots_to_clear.clear()
+    m.forget_slots_to_clear()
     m.release("a")
     assert m.admit("b") == s and m.slots_to_clear == [s]      # the slot comes back and is cleared again
     assert [i for i, _ in m.state_groups()] == [1]

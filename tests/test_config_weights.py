@@ -8,8 +8,13 @@ import torch
 import tinyinfer_amd as ti
 from helpers import CONFIGS
 from tinyinfer_amd.config.qwen3 import Qwen3Config
-from tinyinfer_amd.weights import WeightsError, load_weights, write_model_folder, write_safetensors, SafetensorsFile
-from tinyinfer_amd.weights.safetensors_io import SafetensorsError
+from safetensors.torch import load_file, save_file
+from tinyinfer_amd.weights import WeightsError, FileError, load_weights, write_model_folder
+
+
+def stored(d):
+    """{name: tensor} of a folder's model.safetensors, read with the safetensors package."""
+    return load_file(os.path.join(d, "model.safetensors"))
 
 
 def test_config_reads_every_size_from_the_dict():
@@ -91,10 +96,12 @@ def folder(tmp_path, name="A", dtype="bfloat16"):
 
 def test_random_folder_round_trip_and_dtypes(tmp_path):
     d = folder(tmp_path, "B")
-    f = SafetensorsFile(os.path.join(d, "model.safetensors"))
-    assert "lm_head.weight" in f.names()                                  # untied: a head of its own
-    assert f.info("model.layers.0.self_attn.q_proj.weight") == (torch.bfloat16, (192, 96))
-    assert f.info("model.layers.0.self_attn.q_norm.weight") == (torch.float32, (32,))
+    f = stored(d)
+    assert "lm_head.weight" in f                                          # untied: a head of its own
+    q = f["model.layers.0.self_attn.q_proj.weight"]
+    assert (q.dtype, tuple(q.shape)) == (torch.bfloat16, (192, 96))
+    qn = f["model.layers.0.self_attn.q_norm.weight"]
+    assert (qn.dtype, tuple(qn.shape)) == (torch.float32, (32,))
     _, spec = ti.config_and_spec(ti.read_config_json(d))
     m = ti.Model(spec)
     load_weights(m, d, "bfloat16", "cpu")
@@ -102,14 +109,18 @@ def test_random_folder_round_trip_and_dtypes(tmp_path):
     assert att.w_qkv.dtype == torch.bfloat16 and att.w_qkv.shape == (192 + 2 * 64, 96)   # q, k, v fused
     assert att.q_norm_w.dtype == torch.float32                                           # norms stay 32-bit
     assert m.blocks[0].ffn.w_gate_up.shape == (448, 96)
-    assert m.head.weight is not m.embedding.weight
-    q = f.tensor("model.layers.0.self_attn.q_proj.weight")
+    assert m.head.weight.data_ptr() != m.embedding.weight.data_ptr()
     assert torch.equal(att.w_qkv[:192], q)
+    assert torch.equal(att.w_qkv[192:256], f["model.layers.0.self_attn.k_proj.weight"])
+    assert torch.equal(att.w_qkv[256:], f["model.layers.0.self_attn.v_proj.weight"])
+    assert torch.equal(m.blocks[0].ffn.w_gate_up[224:], f["model.layers.0.mlp.up_proj.weight"])
     # same seed, same bits; another seed, other bits
     d2 = str(tmp_path / "again")
-    t2 = write_model_folder(d2, CONFIGS["B"], seed=3)
-    assert torch.equal(t2["model.norm.weight"], f.tensor("model.norm.weight"))
-    t3 = write_model_folder(str(tmp_path / "other"), CONFIGS["B"], seed=4)
+    write_model_folder(d2, CONFIGS["B"], seed=3)
+    t2 = stored(d2)
+    assert torch.equal(t2["model.norm.weight"], f["model.norm.weight"])
+    write_model_folder(str(tmp_path / "other"), CONFIGS["B"], seed=4)
+    t3 = stored(str(tmp_path / "other"))
     assert not torch.equal(t3["model.norm.weight"], t2["model.norm.weight"])
     # norm weights are 1 + N(0, 0.1), matrices N(0, 0.02)
     assert abs(t2["model.norm.weight"].mean().item() - 1.0) < 0.05
@@ -122,22 +133,21 @@ def test_float32_engine_widens_and_tied_head_shares(tmp_path):
     m = ti.Model(spec)
     load_weights(m, d, "float32", "cpu")
     assert m.embedding.weight.dtype == torch.float32
-    assert m.head.weight is m.embedding.weight                           # tied: one tensor
-    f = SafetensorsFile(os.path.join(d, "model.safetensors"))
-    assert "lm_head.weight" not in f.names()
-    assert torch.equal(m.embedding.weight, f.tensor("model.embed_tokens.weight").float())
+    assert m.head.weight.data_ptr() == m.embedding.weight.data_ptr()     # tied: one tensor
+    f = stored(d)
+    assert "lm_head.weight" not in f
+    assert torch.equal(m.embedding.weight, f["model.embed_tokens.weight"].float())
 
 
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     d = folder(tmp_path, "A")
-    f = SafetensorsFile(os.path.join(d, "model.safetensors"))
-    t = {n: f.tensor(n).clone() for n in f.names()}
+    t = stored(d)
     del t["model.layers.1.mlp.up_proj.weight"]
     del t["model.norm.weight"]
     t["model.layers.0.self_attn.q_proj.bias"] = torch.zeros(64)
     t["model.layers.0.self_attn.k_proj.weight"] = t["model.layers.0.self_attn.k_proj.weight"].T.contiguous()
     t["model.layers.1.input_layernorm.weight"] = torch.ones(63)
-    write_safetensors(os.path.join(d, "model.safetensors"), t)
+    save_file(t, os.path.join(d, "model.safetensors"))
     _, spec = ti.config_and_spec(ti.read_config_json(d))
     with pytest.raises(WeightsError) as e:
         load_weights(ti.Model(spec), d, "bfloat16", "cpu")
@@ -153,9 +163,8 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
 
 def test_untied_without_head_and_open_tying(tmp_path):
     d = folder(tmp_path, "B")
-    f = SafetensorsFile(os.path.join(d, "model.safetensors"))
-    t = {n: f.tensor(n).clone() for n in f.names() if n != "lm_head.weight"}
-    write_safetensors(os.path.join(d, "model.safetensors"), t)
+    t = {n: v for n, v in stored(d).items() if n != "lm_head.weight"}
+    save_file(t, os.path.join(d, "model.safetensors"))
     _, spec = ti.config_and_spec(ti.read_config_json(d))
     with pytest.raises(WeightsError) as e:
         load_weights(ti.Model(spec), d, "bfloat16", "cpu")
@@ -166,7 +175,7 @@ def test_untied_without_head_and_open_tying(tmp_path):
     _, spec = ti.config_and_spec(cfg)
     m = ti.Model(spec)
     load_weights(m, d, "bfloat16", "cpu")
-    assert m.head.weight is m.embedding.weight
+    assert m.head.weight.data_ptr() == m.embedding.weight.data_ptr()
 
 
 def test_broken_files_are_refused(tmp_path):
@@ -175,10 +184,10 @@ def test_broken_files_are_refused(tmp_path):
     raw = open(p, "rb").read()
     open(p, "wb").write(raw[:len(raw) // 2])                 # cut short
     _, spec = ti.config_and_spec(ti.read_config_json(d))
-    with pytest.raises(SafetensorsError):
+    with pytest.raises(FileError):
         load_weights(ti.Model(spec), d, "bfloat16", "cpu")
     os.remove(p)
-    with pytest.raises(SafetensorsError):
+    with pytest.raises(FileError):
         load_weights(ti.Model(spec), d, "bfloat16", "cpu")
     with pytest.raises(ti.ConfigError):
         ti.read_config_json(str(tmp_path / "nowhere"))

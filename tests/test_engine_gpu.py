@@ -175,20 +175,15 @@ def test_cuts_agree_bitwise_in_float32(model_folders):
 def test_norm_inside_the_product_changes_no_bit(model_folders):
     """Steps of few tokens run the norm before a projection inside the projection's
     kernel.  With that switched off the same steps give the same bits."""
-    from tinyinfer_amd.ops.kernels import get_ops
     folder = model_folders("A", "bfloat16")
     requests = {r: t for r, t in make_requests(CONFIGS["A"]["vocab_size"]).items() if r in ("a", "b")}
     trace = traces.tail_one_by_one(requests, 32)
-    ops = get_ops()
     results = []
-    try:
-        for fused in (True, False):
-            ops.use_fused_norm = fused
-            engine = build_engine(folder, "bfloat16", traces.max_tokens(trace))
-            assert engine.ops.can_fuse_norm(1, torch.bfloat16) == fused
-            results.append(replay(engine, trace))
-    finally:
-        ops.use_fused_norm = True
+    for fused in (True, False):
+        engine = build_engine(folder, "bfloat16", traces.max_tokens(trace))
+        engine.ops.use_fused_norm = fused            # the switches are the engine's own
+        assert engine.ops.can_fuse_norm(1, torch.bfloat16) == fused
+        results.append(replay(engine, trace))
     for r in requests:
         assert np.array_equal(results[0][r], results[1][r]), r
 
@@ -197,19 +192,14 @@ def test_prepared_decode_attention_changes_only_rounding(model_folders):
     """Steps of single tokens norm, rotate and cache inside the attention kernel.  With that
     switched off the same steps give the same logits up to the rounding of a different order
     of summation (config D: head size 64, one kv head, a window)."""
-    from tinyinfer_amd.ops.kernels import get_ops
     folder = model_folders("D", "bfloat16", True)
     requests = {r: t for r, t in make_requests(CONFIGS["D"]["vocab_size"]).items() if r in ("a", "c")}
     trace = traces.tail_one_by_one(requests, 48)
-    ops = get_ops()
     results = []
-    try:
-        for fused in (True, False):
-            ops.use_fused_qk_decode = fused
-            engine = build_engine(folder, "bfloat16", traces.max_tokens(trace))
-            results.append(replay(engine, trace))
-    finally:
-        ops.use_fused_qk_decode = True
+    for fused in (True, False):
+        engine = build_engine(folder, "bfloat16", traces.max_tokens(trace))
+        engine.ops.use_fused_qk_decode = fused
+        results.append(replay(engine, trace))
     _, tol = plain_logits(folder, make_requests(CONFIGS["D"]["vocab_size"]), "bfloat16")
     for r in requests:
         assert np.abs(results[0][r] - results[1][r]).max() < tol, r
@@ -219,20 +209,15 @@ def test_prepared_decode_attention_changes_only_rounding(model_folders):
 def test_prepared_qkv_product_changes_no_bit(model_folders):
     """Steps of many tokens prepare q and write the cache in the epilogue of the q/k/v product.
     With that switched off the same steps give the same bits (config D, head size 64)."""
-    from tinyinfer_amd.ops.kernels import get_ops
     folder = model_folders("D", "bfloat16", True)
     requests = {"a": random_tokens(300, CONFIGS["D"]["vocab_size"], 5), "b": random_tokens(90, CONFIGS["D"]["vocab_size"], 6)}
     trace = [{"entries": [("a", requests["a"][:200], [0, 199]), ("b", requests["b"][:70], [69])], "end": []},
              {"entries": [("a", requests["a"][200:], list(range(100))), ("b", requests["b"][70:71], [0])], "end": ["a", "b"]}]
-    ops = get_ops()
     results = []
-    try:
-        for fused in (True, False):
-            ops.use_fused_qkv_prefill = fused
-            engine = build_engine(folder, "bfloat16", 512)
-            results.append(replay(engine, trace))
-    finally:
-        ops.use_fused_qkv_prefill = True
+    for fused in (True, False):
+        engine = build_engine(folder, "bfloat16", 512)
+        engine.ops.use_fused_qkv_prefill = fused
+        results.append(replay(engine, trace))
     for r in requests:
         assert np.array_equal(results[0][r], results[1][r]), r
 
@@ -273,7 +258,6 @@ def test_steps_of_17_to_64_tokens_at_real_width(model_folders):
     17, 64 and 33 tokens, one of them beside another request's token, then a step that wants
     nothing: against the plain model; with the sums added at once the bits are the same, and
     with the kernels without MFMA the logits agree within the same bound."""
-    from tinyinfer_amd.ops.kernels import get_ops
     folder = model_folders("E", "bfloat16", True)
     V = CONFIGS["E"]["vocab_size"]
     requests = {"a": random_tokens(154, V, 41), "b": random_tokens(3, V, 42)}
@@ -285,16 +269,13 @@ def test_steps_of_17_to_64_tokens_at_real_width(model_folders):
              {"entries": [("a", a[119:152], [])], "end": []},                   # wants nothing
              {"entries": [("a", a[152:154], [0, 1]), ("b", b[2:3], [0])], "end": ["a", "b"]}]
     rows = {"a": [0, 39, 56, 57, 118, 152, 153], "b": [2]}
-    ops = get_ops()
     results = {}
-    try:
-        for how in ("left to the norm", "added at once", "without MFMA"):
-            ops.use_deferred_add = how == "left to the norm"
-            ops.use_split_k_add = how != "without MFMA"
-            results[how] = replay(build_engine(folder, "bfloat16", 256), trace)
-            assert ops._pending is None
-    finally:
-        ops.use_deferred_add = ops.use_split_k_add = True
+    for how in ("left to the norm", "added at once", "without MFMA"):
+        engine = build_engine(folder, "bfloat16", 256)
+        engine.ops.use_deferred_add = how == "left to the norm"
+        engine.ops.use_split_k_add = how != "without MFMA"
+        results[how] = replay(engine, trace)
+        assert engine.ops._pending is None
     for r in requests:
         got = results["left to the norm"][r]
         err = np.abs(got - want[r][rows[r]]).max()

@@ -62,7 +62,7 @@ def test_config_b_mixed_batch_with_temperature(model_folders):
     engine2 = ti.Engine.from_folder(d, "float32", page_size=16, max_tokens=64, max_requests=1, max_seq=64)
     sched = ti.Scheduler(engine2.cache)
     for i, p in enumerate(prompts):
-        sched._submitted = i
+        sched.set_next_number(i)
         r = sched.add(p, 6, ti.SamplingParams(0.8, 0, 1.0, 123))
         from tinyinfer_amd.api import run_requests
         run_requests(engine2, sched)
@@ -83,7 +83,7 @@ def test_greedy_generation_with_graphs_equals_eager(model_folders, dtype):
         outs[graph] = ti.generate_ids(engine, prompts, max_new_tokens=40, use_graph=graph, chunk_size=16,
                                       max_batched_tokens=24)
         if graph:
-            assert engine._graphs, "no graph was captured"
+            assert engine.graph_keys(), "no graph was captured"
     assert outs[True] == outs[False]
     # logits bit for bit, several replays, eager work between them
     e1 = ti.Engine.from_folder(d, dtype, page_size=16, max_tokens=256, max_requests=2, max_seq=128)
@@ -136,8 +136,8 @@ def test_steps_of_a_repeated_shape_replay_from_graphs(model_folders, dtype):
             odd = [ti.StepEntry("x", toks["x"][fed["x"]:fed["x"] + 5], [4])]
             assert torch.equal(e1.step(odd), e2.step_graph(odd))
             fed["x"] += 5
-    assert shape in e2._graphs and len([k for k in e2._graphs if not isinstance(k, int)]) == 1
-    assert not e1._graphs
+    assert shape in e2.graph_keys() and len([k for k in e2.graph_keys() if not isinstance(k, int)]) == 1
+    assert not e1.graph_keys()
     # the captured shape with other requests in it: a new request takes the portion's place
     for e in (e1, e2):
         e.release("x")
@@ -156,11 +156,9 @@ def test_only_the_most_recent_step_shapes_keep_their_graphs(model_folders, monke
     """With room for one shape's graph, two shapes in turn push one another out and are captured
     again; the logits stay those of eager steps."""
     import tinyinfer_amd as ti
-    from tinyinfer_amd.engine import engine as engine_module
-    monkeypatch.setattr(engine_module, "MAX_STEP_GRAPHS", 1)
     d = model_folders("D", "bfloat16", True)
     e1 = ti.Engine.from_folder(d, "bfloat16", page_size=16, max_tokens=512, max_requests=2, max_seq=256)
-    e2 = ti.Engine.from_folder(d, "bfloat16", page_size=16, max_tokens=512, max_requests=2, max_seq=256)
+    e2 = ti.Engine.from_folder(d, "bfloat16", page_size=16, max_tokens=512, max_requests=2, max_seq=256, max_step_graphs=1)
     toks = random_tokens(240, 333, 9)
     fed = 0
     captured = set()
@@ -169,7 +167,7 @@ def test_only_the_most_recent_step_shapes_keep_their_graphs(model_folders, monke
         entries = [ti.StepEntry("x", toks[fed:fed + n], [n - 1])]
         assert torch.equal(e1.step(entries), e2.step_graph(entries)), i
         fed += n
-        shapes = [k for k in e2._graphs if not isinstance(k, int)]
+        shapes = [k for k in e2.graph_keys() if not isinstance(k, int)]
         assert len(shapes) <= 1
         captured |= set(shapes)
     assert len(captured) == 2

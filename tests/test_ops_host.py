@@ -1,7 +1,7 @@
-"""What the kernels' Python side decides on the host.  The argument types that Python gives the kernel
-libraries come from the declarations in tinyinfer_kernels.h: pointers are passed as plain ints,
-which ctypes would cut to 32 bits for a function without declared types.  And the number of runs the
-decode attention cuts a context into."""
+"""What the kernels' host side decides.  The argument types that Python gives the kernel libraries
+(tests that call one kernel) come from the declarations in tinyinfer_kernels.h: pointers are passed as
+plain ints, which ctypes would cut to 32 bits for a function without declared types.  And the number of
+runs the decode attention cuts a context into."""
 import ctypes
 import os
 import re
@@ -16,17 +16,17 @@ def header_text():
         return f.read()
 
 
-def test_every_function_python_calls_is_declared():
+def test_every_kernel_the_host_library_calls_is_declared():
+    """ops.cpp resolves kernels by name (`KERNEL("lib", ti_fn)`) with the type of the header's declaration:
+    a name the header does not declare would not compile.  Here: every such name is in the header, and the
+    library it is looked up in is one the build knows."""
     declared = kernels.header_signatures(header_text())
-    ops_dir = os.path.dirname(kernels.__file__)
-    called = set()
-    for name in os.listdir(ops_dir):
-        if name.endswith(".py"):
-            with open(os.path.join(ops_dir, name)) as f:
-                called |= set(re.findall(r"lib\.(ti_\w+)\(", f.read()))
-    called.discard("ti_last_error")
-    assert called, "no calls found: the pattern of this test is out of date"
-    assert not called - set(declared), f"called but not declared in the header: {sorted(called - set(declared))}"
+    with open(os.path.join(os.path.dirname(build.HERE), "ops", "ops.cpp")) as f:
+        used = re.findall(r'KERNEL\("(\w+)",\s*(ti_\w+)\)', f.read())
+    assert len(used) > 15, "the pattern of this test is out of date"
+    for lib, fn in used:
+        assert fn in declared, fn
+        assert lib in build.SOURCES, lib
 
 
 def test_declarations_are_read_as_written():
@@ -39,7 +39,9 @@ def test_declarations_are_read_as_written():
                     ctypes.c_int, ctypes.c_float, ctypes.c_void_p]
     restype, args = sig["ti_gemm_bf16"]
     assert args[6] is ctypes.c_long and args[-1] is ctypes.c_void_p and len(args) == 9
-    assert sig["ti_gemm_bf16_force_tile"] == (None, [ctypes.c_int])
+    with open(os.path.join(build.HERE, "tinyinfer_kernels_tuning.h")) as f:
+        assert kernels.header_signatures(f.read())["ti_gemm_bf16_force_tile"] == (None, [ctypes.c_int])
+    assert sig["ti_fill_random"][1][6] is ctypes.c_ulong
     # what the call sites pass for such arguments is accepted
     assert ctypes.c_void_p.from_param(None) is None
     ctypes.c_void_p.from_param(ctypes.byref(ctypes.c_int(0)))

@@ -1,12 +1,13 @@
 """tinyinfer for AMD MI355X: a small, whole inference engine for the Qwen3 dense
-decoder.  Configuration, weights, parts, cache and scheduler are plain Python;
-everything that touches a token's numbers is a hand-written HIP kernel."""
+decoder.  Configuration, weights, parts, cache manager, step function, scheduler
+and sampler are a C++ library (include/inference.h) over hand-written HIP kernels
+(csrc/); this package binds it, and lets parts and architectures be defined in
+Python beside the built-in ones."""
 from .config.base import ConfigError, read_config_json
 from .config.qwen3 import Qwen3Config
 from .registry import register_architecture, registered_architectures, config_and_spec
 from .parts.registry import register_part, build_part
 from . import parts as _parts          # noqa: F401  registers the built-in parts
-from . import models as _models        # noqa: F401  registers the built-in architecture
 from .models import Model, ModelSpec, LayerSpec, PartSpec
 from .engine import Engine, StepEntry
 from .engine.scheduler import Scheduler, Request

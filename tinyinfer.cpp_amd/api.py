@@ -6,16 +6,18 @@
 
 `generate` drives the scheduler, the step function and the device sampler: the
 loop of /root/reference/src/main.cpp:210-297 with admission, portions and
-preemption added.  Options carry the reference's names and meanings
-(`max_new_tokens` = -n, `temperature` = -t, `top_k`, `top_p`, `seed`, `max_seq`).
+preemption added (`run_requests`, engine/scheduler.cpp).  Options carry the
+reference's names and meanings (`max_new_tokens` = -n, `temperature` = -t,
+`top_k`, `top_p`, `seed`, `max_seq`).
 """
 from __future__ import annotations
 
-import time
-from dataclasses import dataclass, field
+import json
+from dataclasses import dataclass
 from typing import List, Optional, Sequence
 
-from .engine.engine import Engine, StepEntry
+from . import native
+from .engine.engine import Engine
 from .engine.scheduler import Request, Scheduler
 from .sampling.sampler import Sampler, SamplingParams
 
@@ -32,46 +34,30 @@ class GenerationStats:
 
 def run_requests(engine: Engine, scheduler: Scheduler, sampler: Optional[Sampler] = None,
                  stats: Optional[GenerationStats] = None, on_token=None, use_graph: bool = False) -> None:
-    """Run until the scheduler has no work.  `on_token(request, token)` is called
-    for every generated token."""
-    import torch
-    sampler = sampler or Sampler(engine.ops, engine.device)
-    stats = stats if stats is not None else GenerationStats()
-    while scheduler.has_work():
-        plan = scheduler.plan()
-        stats.preemptions += len(plan.preempted)
-        entries = [StepEntry(e.request.key, e.request.tokens[e.start:e.start + e.n_tokens],
-                             (e.n_tokens - 1,) if e.sample else ()) for e in plan.entries]
-        decode_only = all(e.n_tokens == 1 for e in plan.entries)
-        t0 = time.perf_counter()
-        if use_graph:
-            logits = engine.step_graph(entries)
-        else:
-            logits = engine.step(entries)
-        sampled = {}
-        asked = [e.request for e in plan.entries if e.sample]
-        if asked:
-            toks = sampler.sample(logits, [r.params for r in asked], [r.number for r in asked],
-                                  [len(r.generated) for r in asked])
-            sampled = {r.number: t for r, t in zip(asked, toks)}
-        else:
-            torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) * 1e3
-        n_tok = sum(e.n_tokens for e in plan.entries)
-        if decode_only:
-            stats.decode_ms += dt
-            stats.decode_tokens += n_tok
-        else:
-            stats.prefill_ms += dt
-            stats.prefill_tokens += n_tok
-        stats.steps += 1
-        before = {r.number: len(r.generated) for r in asked}
-        for req in scheduler.commit(plan, sampled):
-            engine.release(req.key)
-        if on_token:
-            for r in asked:
-                if len(r.generated) > before[r.number]:
-                    on_token(r, r.generated[-1])
+    """Run until the scheduler has no work.  `on_token(request, token)` is called for every
+    generated token.  When a step fails, every request the scheduler still holds is given back
+    to the cache before the error is raised."""
+    native.ensure_kernels(["sampling"])
+    callback = native.ON_TOKEN(lambda number, token: on_token(scheduler._requests[number], token)) if on_token else \
+        ctypes_null(native.ON_TOKEN)
+    try:
+        out = native.text("ti_run_requests", engine._ptr, scheduler._ptr, sampler._ptr if sampler else None,
+                          int(use_graph), callback)
+    finally:
+        native.forget_contexts()
+    if stats is not None:
+        d = json.loads(out)
+        stats.prefill_ms += d["prefill_ms"]
+        stats.prefill_tokens += d["prefill_tokens"]
+        stats.decode_ms += d["decode_ms"]
+        stats.decode_tokens += d["decode_tokens"]
+        stats.steps += d["steps"]
+        stats.preemptions += d["preemptions"]
+
+
+def ctypes_null(kind):
+    import ctypes
+    return ctypes.cast(None, kind)
 
 
 def generate_ids(engine: Engine, prompts: Sequence[Sequence[int]], max_new_tokens: int = 128,
@@ -90,15 +76,22 @@ def generate_ids(engine: Engine, prompts: Sequence[Sequence[int]], max_new_token
 
 
 class LLM:
-    """A model folder made ready for generation."""
+    """A model folder made ready for generation (or, with `random_seed`, a config.json alone with
+    random weights drawn on the device)."""
 
     def __init__(self, model_dir: str, dtype: str = "bfloat16", max_seq: int = 2048, max_requests: int = 16,
                  page_size: int = 16, max_tokens: Optional[int] = None, chunk_size: int = 512,
-                 max_batched_tokens: int = 2048, use_graph: bool = False):
-        if max_tokens is None:
+                 max_batched_tokens: int = 2048, use_graph: bool = False, num_pages: Optional[int] = None,
+                 random_seed: Optional[int] = None):
+        if max_tokens is None and num_pages is None:
             max_tokens = max_seq * max_requests
-        self.engine = Engine.from_folder(model_dir, dtype, page_size=page_size, max_tokens=max_tokens,
-                                         max_requests=max_requests, max_seq=max_seq)
+        options = dict(page_size=page_size, max_tokens=max_tokens, num_pages=num_pages, max_requests=max_requests,
+                       max_seq=max_seq)
+        if random_seed is None:
+            self.engine = Engine.from_folder(model_dir, dtype, **options)
+        else:
+            from .config.base import read_config_json
+            self.engine = Engine.from_config(read_config_json(model_dir), random_seed, dtype, **options)
         self.chunk_size = chunk_size
         self.max_batched_tokens = max_batched_tokens
         self.use_graph = use_graph

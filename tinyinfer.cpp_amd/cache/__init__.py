@@ -1,2 +1,1 @@
 from .manager import CacheManager, CacheError, OutOfPages, PagePool, PagedGroup
-from .storage import CacheStorage

@@ -3,8 +3,10 @@
 
     tinyinfer -m MODEL_DIR -n max_tokens -p "prompt" [-p "prompt2" ...] [-f prompts.txt]
               [-t temp] [--top-k K] [--top-p P] [--seed S] [--max-seq N] [--cuda-graph] [--verbose]
+              [--dtype D] [--page-size P] [--num-pages N] [--chunk N] [--max-batched-tokens N] [--random-weights]
 
--m is a model folder (config.json and safetensors) instead of a GGUF file.  A
+-m is a model folder (config.json and safetensors) instead of a GGUF file; with
+--random-weights a config.json alone is enough, and the weights are drawn on the device from --seed.  A
 prompt is a list of token ids ("1,2,3" or "1 2 3"); if the folder holds a
 `tokenizer.json`, any other prompt is text and is tokenized with it, and outputs
 are printed as text too.  `-f` reads one prompt per non-empty line.  Results go
@@ -20,7 +22,10 @@ from typing import List, Optional
 
 USAGE = """usage: {prog} -m model_dir -n max_tokens -p "prompt" [-p "prompt2" ...] [-f prompts.txt]
   [-t temp] [--top-k K] [--top-p P] [--seed S] [--max-seq N] [--cuda-graph] [--verbose]
-  [--dtype bfloat16|float32] [--page-size P] [--chunk N] [--max-batched-tokens N]
+  [--dtype bfloat16|float32] [--page-size P] [--num-pages N] [--chunk N] [--max-batched-tokens N]
+  [--random-weights]
+  --random-weights: -m needs a config.json only; the weights are drawn on the device from --seed
+  --num-pages: pages in the cache pool (default: enough for --max-seq tokens of every prompt)
   a prompt is a list of token ids ("1,2,3"), or text if the model folder has a tokenizer.json
   --cuda-graph (alias --graph): replay decode steps, and other steps whose shape repeats, from captured graphs (off by default)
 """
@@ -58,6 +63,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     n_predict, temp, top_k, top_p, seed, max_seq = 128, 0.0, 0, 1.0, 42, 2048
     graph = verbose = chat = False
     dtype, page_size, chunk, budget = "bfloat16", 16, 512, 2048
+    num_pages, random_weights = None, False
 
     def usage() -> int:
         sys.stderr.write(USAGE.format(prog=os.path.basename(prog)))
@@ -101,6 +107,10 @@ def main(argv: Optional[List[str]] = None) -> int:
                 dtype = args[i + 1]; i += 2
             elif a == "--page-size" and has:
                 page_size = int(args[i + 1]); i += 2
+            elif a == "--num-pages" and has:
+                num_pages = int(args[i + 1]); i += 2
+            elif a == "--random-weights":
+                random_weights = True; i += 1
             elif a == "--chunk" and has:
                 chunk = int(args[i + 1]); i += 2
             elif a == "--max-batched-tokens" and has:
@@ -138,12 +148,13 @@ def main(argv: Optional[List[str]] = None) -> int:
         ids.append(t)
 
     import tinyinfer_amd as ti
-    from tinyinfer_amd.weights import WeightsError
+    from tinyinfer_amd.weights import WeightsError, FileError
     try:
         n_req = max(1, min(len(ids), 64))
         llm = ti.LLM(model, dtype=dtype, max_seq=max_seq, max_requests=n_req, page_size=page_size,
-                     chunk_size=chunk, max_batched_tokens=budget, use_graph=graph)
-    except (ti.ConfigError, WeightsError, FileNotFoundError) as e:
+                     chunk_size=chunk, max_batched_tokens=budget, use_graph=graph, num_pages=num_pages,
+                     random_seed=seed if random_weights else None)
+    except (ti.ConfigError, WeightsError, FileError, FileNotFoundError) as e:
         sys.stderr.write(f"main: {e}\n")
         return 1
     if verbose:

@@ -24,6 +24,7 @@
 // /root/reference/src/cuda/attention.cu:107-198.)
 #include "common.h"
 #include "tinyinfer_kernels.h"
+#include "tinyinfer_kernels_tuning.h"
 #include "qk_prep.h"
 
 TI_ERROR_API

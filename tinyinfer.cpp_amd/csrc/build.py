@@ -30,7 +30,7 @@ FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-shared",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-mllvm", "-amdgpu-kernarg-preload-count=16",
          "-Wno-unused-command-line-argument"]
-HEADERS = ["common.h", "qk_prep.h", "tinyinfer_kernels.h"]
+HEADERS = ["common.h", "qk_prep.h", "tinyinfer_kernels.h", "tinyinfer_kernels_tuning.h"]
 # flags of single libraries.  The attention kernels rescale their MFMA accumulators with
 # vector instructions; kept in the accumulation registers they would be copied out and back
 # on every turn of the loop, so their MFMAs are told to work on ordinary vector registers.
@@ -47,6 +47,17 @@ SOURCES: Dict[str, str] = {
     "gemm_bf16": "gemm_bf16.hip",
     "attention_bf16": "attention_bf16.hip",
 }
+
+
+# the host library (configuration, weights, parts, cache manager, step function, scheduler, sampler
+# and the C interface the Python package binds): C++17, no device code
+PKG = os.path.dirname(HERE)
+HOST_SOURCES = ["config/json.cpp", "config/config.cpp", "ops/ops.cpp", "parts/parts.cpp", "weights/weights.cpp",
+                "models/model.cpp", "cache/cache_manager.cpp", "engine/engine.cpp", "engine/scheduler.cpp",
+                "sampling/sampler.cpp", "engine/c_api.cpp"]
+HOST_HEADERS = ["include/inference.h", "weights/weights.h", "csrc/tinyinfer_kernels.h"]
+HOST_FLAGS = ["-std=c++17", "-O2", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-Wall", "-Wno-unused-function"]
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 
 class BuildError(RuntimeError):
@@ -182,8 +193,110 @@ def ensure(names: Iterable[str], force: bool = False) -> Dict[str, str]:
     return paths
 
 
+def _host_digest() -> str:
+    h = hashlib.sha256()
+    for f in HOST_SOURCES + HOST_HEADERS:
+        with open(os.path.join(PKG, f), "rb") as fh:
+            h.update(fh.read())
+    h.update(" ".join(HOST_FLAGS).encode())
+    return h.hexdigest()[:12]
+
+
+def host_lib_name() -> str:
+    return f"libtinyinfer.{_host_digest()}.so"
+
+
+def find_host():
+    for d in _lib_dirs():
+        p = os.path.join(d, host_lib_name())
+        if os.path.isfile(p):
+            return p
+    return None
+
+
+def ensure_host(force: bool = False) -> str:
+    """Path of the host library, compiled (its files several at a time) if it is not there."""
+    p = None if force else find_host()
+    if p:
+        return p
+    cxx = shutil.which("g++") or shutil.which("c++") or os.path.join(ROCM, "llvm", "bin", "clang++")
+    if not cxx or not os.path.isfile(cxx):
+        raise BuildError("no C++ compiler found (g++, c++, or ROCm's clang++): the host library cannot be compiled")
+    out_dir = _writable_dir()
+    final = os.path.join(out_dir, host_lib_name())
+    work = tempfile.mkdtemp(prefix="tinyinfer_host_")
+    t0 = time.time()
+    _say(f"compiling the host library ({len(HOST_SOURCES)} files) ...")
+    errors: List[str] = []
+    objects = []
+
+    def one(src):
+        obj = os.path.join(work, src.replace("/", "_") + ".o")
+        objects.append(obj)
+        proc = subprocess.run([cxx] + HOST_FLAGS + ["-I" + os.path.join(ROCM, "include"), "-c", os.path.join(PKG, src), "-o", obj],
+                              stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode != 0:
+            errors.append(f"{src}:\n{proc.stdout}")
+
+    done = threading.Event()
+
+    def heartbeat():
+        while not done.wait(10.0):
+            _say(f"still compiling the host library ({time.time() - t0:.0f} s) ...")
+
+    threading.Thread(target=heartbeat, daemon=True).start()
+    threads = [threading.Thread(target=one, args=(s,)) for s in HOST_SOURCES]
+    limit = max(1, min(8, os.cpu_count() or 1))
+    for i in range(0, len(threads), limit):
+        for t in threads[i:i + limit]:
+            t.start()
+        for t in threads[i:i + limit]:
+            t.join()
+    try:
+        if errors:
+            raise BuildError("the host library does not compile:\n" + "\n".join(errors))
+        part = final + f".{os.getpid()}.part"
+        proc = subprocess.run([cxx, "-shared", "-o", part] + objects + ["-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-ldl",
+                                                                          "-lpthread", "-Wl,-rpath," + os.path.join(ROCM, "lib")],
+                              stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode != 0:
+            raise BuildError(f"the host library does not link:\n{proc.stdout}")
+        os.replace(part, final)
+    finally:
+        done.set()
+        shutil.rmtree(work, ignore_errors=True)
+    for f in os.listdir(out_dir):
+        if f.startswith("libtinyinfer.") and f.endswith(".so") and f != os.path.basename(final):
+            try:
+                os.remove(os.path.join(out_dir, f))
+            except OSError:
+                pass
+    _say(f"compiled the host library in {time.time() - t0:.1f} s")
+    return final
+
+
+def write_manifest() -> None:
+    """kernels.manifest beside the libraries: `name file` a line, for programs that use the host library
+    without this package (it looks the kernel libraries up there)."""
+    for d in _lib_dirs():
+        lines = []
+        for n in SOURCES:
+            p = os.path.join(d, lib_name(n))
+            if os.path.isfile(p):
+                lines.append(f"{n} {os.path.basename(p)}")
+        if lines:
+            try:
+                with open(os.path.join(d, "kernels.manifest"), "w") as f:
+                    f.write("\n".join(lines) + "\n")
+            except OSError:
+                pass
+
+
 def build_all(force: bool = True) -> Dict[str, str]:
-    return ensure([n for n, s in SOURCES.items() if os.path.isfile(os.path.join(HERE, s))], force=force)
+    paths = ensure([n for n, s in SOURCES.items() if os.path.isfile(os.path.join(HERE, s))], force=force)
+    paths["host"] = ensure_host(force=force)
+    write_manifest()
+    return paths
 
 
 if __name__ == "__main__":

@@ -381,3 +381,63 @@ extern "C" int ti_qk_norm_inplace(float* qkv, int row_width, const float* q_w, c
   TI_LAUNCH_CHECK();
   return 0;
 }
+
+// ----------------------------------------------------------------------- fills
+// Zero `words` four-byte words (a kernel, not a memset node: a caller may be capturing a graph).
+__global__ void fill_zero_kernel(uint32_t* __restrict__ p, long words) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += (long)gridDim.x * blockDim.x) p[i] = 0u;
+}
+
+extern "C" int ti_fill_zero(void* p, long bytes, hipStream_t stream) {
+  TI_REQUIRE(bytes >= 0 && bytes % 4 == 0 && ((uintptr_t)p & 3) == 0, "fill_zero: %ld bytes at %p are not whole words",
+             bytes, p);
+  if (bytes == 0) return 0;
+  const long words = bytes / 4;
+  const unsigned blocks = (unsigned)((words + 255) / 256 < 4096 ? (words + 255) / 256 : 4096);
+  fill_zero_kernel<<<blocks, 256, 0, stream>>>((uint32_t*)p, words);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// Random weights on the device.  Element i of a tensor is a pure function of (seed, i): two
+// 24-bit uniforms from splitmix64's output function, then Box-Muller for a normal.  The host's
+// generator (the one that writes model folders) is the same function.
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+// kind 0: normal(a, b); 1: uniform [a, b); 2: constant a
+template <typename T>
+__global__ void fill_random_kernel(T* __restrict__ p, long n, int kind, float a, float b, uint64_t seed) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const uint64_t z = mix64(mix64(seed) ^ (uint64_t)i);
+    const float u1 = ((float)((z >> 40) & 0xffffffu) + 1.0f) * (1.0f / 16777216.0f);   // (0, 1]
+    const float u2 = (float)((z >> 16) & 0xffffffu) * (1.0f / 16777216.0f);            // [0, 1)
+    float v;
+    if (kind == 0) v = a + b * (sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2));
+    else if (kind == 1) v = a + (b - a) * u2;
+    else v = a;
+    st<T>(p + i, v);
+  }
+}
+__global__ void fill_random_int_kernel(int* __restrict__ p, long n, int lo, int hi, uint64_t seed) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const uint64_t z = mix64(mix64(seed) ^ (uint64_t)i);
+    p[i] = lo + (int)((z >> 11) % (uint64_t)(hi > lo ? hi - lo : 1));
+  }
+}
+
+extern "C" int ti_fill_random(int dtype, void* p, long n, int kind, float a, float b, unsigned long seed,
+                              hipStream_t stream) {
+  TI_REQUIRE(n >= 0 && kind >= 0 && kind <= 2, "fill_random: bad count %ld or kind %d", n, kind);
+  TI_REQUIRE(dtype == TI_F32 || dtype == TI_BF16 || dtype == 2, "fill_random: unknown dtype %d", dtype);
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
+  if (dtype == TI_F32) fill_random_kernel<float><<<blocks, 256, 0, stream>>>((float*)p, n, kind, a, b, seed);
+  else if (dtype == TI_BF16) fill_random_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)p, n, kind, a, b, seed);
+  else fill_random_int_kernel<<<blocks, 256, 0, stream>>>((int*)p, n, (int)a, (int)b, seed);
+  TI_LAUNCH_CHECK();
+  return 0;
+}

@@ -18,6 +18,7 @@
 // per row of A for M <= 32.)
 #include "common.h"
 #include "tinyinfer_kernels.h"
+#include "tinyinfer_kernels_tuning.h"
 #include "qk_prep.h"
 
 TI_ERROR_API

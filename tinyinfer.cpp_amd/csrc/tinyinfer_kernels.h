@@ -43,6 +43,11 @@ int ti_qk_norm_rope_kv_write(int dtype, const float* qkv, const float* q_w, cons
 // the per-head norm alone, in place
 int ti_qk_norm_inplace(float* qkv, int row_width, const float* q_w, const float* k_w, int M, int n_head, int n_kv, int hd,
                        float eps, hipStream_t stream);
+// zero `bytes` bytes (whole four-byte words) with a kernel
+int ti_fill_zero(void* p, long bytes, hipStream_t stream);
+// random values, element i a pure function of (seed, i).  dtype 0 / 1: kind 0 normal(a, b), 1 uniform
+// [a, b), 2 constant a; dtype 2 (int32): uniform integers in [a, b)
+int ti_fill_random(int dtype, void* p, long n, int kind, float a, float b, unsigned long seed, hipStream_t stream);
 
 // ---- libti_gemm_generic: out (op)= A W^T for any sizes, float32 or bfloat16, fixed summation order
 int ti_gemm_generic(int dtype, const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
@@ -70,18 +75,6 @@ int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K, long lda, 
                           float eps, const float* inv_freq, const float* rope_table, int table_len, const int* pos,
                           const int* slot, const int* table, int table_stride, void* pool, void* q_out, int n_head,
                           int n_kv, int hd, int page_size, hipStream_t stream);
-// switches for measurements and tests (0 restores the choice by shape)
-void ti_gemm_bf16_force_tile(int which);      // 1: 256 x 128, 3: 128 x 64, 6: 64 x 64
-void ti_gemm_bf16_skinny_waves(int waves);    // 4 or 8 wavefronts in the kernel for M <= 64
-void ti_gemm_bf16_qkv_prep_min_rows(int rows); // the fewest rows ti_gemm_bf16_qkv_prep serves (17)
-void ti_gemm_bf16_qkv_prep_rows(int rows);    // 128 / 256: the rows of ti_gemm_bf16_qkv_prep's tile; 0: by the shape
-void ti_gemm_bf16_wide_rows_on(int on);       // 0: 17..64 rows times a weight of 16,384 rows or more take the other kernels
-void ti_gemm_bf16_tiled_from(long rows_times_elems); // 17..64 rows x weight elements from which they take the tiled kernels
-void ti_gemm_bf16_add_split_on(int on);         // 0: ti_gemm_bf16_add_split serves nothing
-void ti_gemm_bf16_use_pipelined(int on);      // 0: the plain tiled kernel for every K
-void ti_gemm_bf16_row_per_wave(int on);        // 0: few tokens and a weight of few rows take the 16-row kernels too
-void ti_gemm_bf16_skinny_copy(int on);        // 0: up to 16 tokens, fragments of the token rows straight from memory
-void ti_gemm_bf16_skinny_deep(int on);        // 0: four chunks of K in flight per wavefront also for a long K
 
 // ---- libti_attention_generic: paged causal attention of every row, any head size in steps of 16
 int ti_attention_rows(int dtype, const void* q, const void* pool, const int* table, int table_stride, const int* pos,
@@ -119,9 +112,6 @@ int ti_attention_prefill_paired_bf16(const void* q, const void* pool, const int*
                                      const int* tiles, const int* entries, void* out, int n_tiles, int n_head,
                                      int n_kv, int hd, int page_size, float scale, int window, int n_rows,
                                      float* part_o, float* part_ml, int n_splits, int paired, hipStream_t stream);
-void ti_attention_decode_shared_query(int on);   // 0: every wavefront of a decode workgroup prepares the query itself
-void ti_attention_prefill_groups(int groups);  // 1 or 2 groups of wavefronts per workgroup, 0: by the launch
-void ti_attention_prefill_use_lds(int on);     // 0: the kernel without LDS for every head size
 
 // ---- libti_sampling
 // out[r] = lowest index of the largest logit; scratch: 2 * 64 * n_rows four-byte words (two stages:

@@ -1,1 +1,3 @@
-from .engine import Engine, StepEntry, StepContext, EngineError, required_libraries
+from .engine import Engine, StepEntry, EngineError
+from .context import StepContext
+from ..ops.kernels import required_libraries

@@ -1,3 +1,2 @@
 from ..spec import ModelSpec, LayerSpec, PartSpec, TensorNeed, PagedKVNeed, StateNeed
 from .model import Model
-from . import qwen3  # noqa: F401  (registers the architecture)

@@ -1,12 +1,16 @@
 """A model put together from a `ModelSpec`: parts built through the part
-registry, cache needs gathered into groups, the run order kept as a list."""
+registry, handed to the host library, which gathers their cache needs into
+groups and keeps the run order (models/model.cpp)."""
 from __future__ import annotations
 
+import ctypes
+import json
 from typing import Dict, List, Tuple
 
-from ..spec import ModelSpec, TensorNeed
-from ..parts.registry import build_part, _PARTS
-from ..parts.base import join
+from .. import native
+from ..parts.base import join, part_handle
+from ..parts.registry import _PARTS, build_part
+from ..spec import ModelSpec, TensorNeed, cache_need_from_dict
 
 
 class Model:
@@ -36,9 +40,33 @@ class Model:
         for i in self.run_order:
             if not 0 <= i < len(self.blocks):
                 raise ValueError(f"schedule names layer {i}, but there are {len(self.blocks)}")
-        self._group_cache()
+        meta = {"architecture": spec.architecture, "vocab_size": spec.vocab_size, "hidden_size": spec.hidden_size,
+                "schedule": spec.schedule, "eos_token_ids": list(spec.eos_token_ids),
+                "max_position_embeddings": spec.max_position_embeddings,
+                "cache_from": [ls.cache_from for ls in spec.layers]}
+        handles = (ctypes.c_void_p * max(1, len(self.blocks)))(*[part_handle(b).ptr for b in self.blocks])
+        try:
+            self._ptr = native.pointer("ti_model_create", json.dumps(meta).encode(), part_handle(self.embedding).ptr,
+                                       len(self.blocks), handles, part_handle(self.final_norm).ptr,
+                                       part_handle(self.head).ptr)
+        except native.ConfigError as e:
+            raise ValueError(str(e)) from None
+        # groups of cache layers with the same need, and per run: id(part) -> (group, cache layer)
+        groups = json.loads(native.text("ti_model_cache_groups", self._ptr))
+        self.cache_groups: List[Tuple[object, int]] = [(cache_need_from_dict(g["need"]), g["layers"]) for g in groups]
+        by_identity = {part_handle(p).identity(): p for p in self.parts()}
+        self.bindings: List[Dict[int, Tuple[int, int]]] = [
+            {id(by_identity[ident]): (g, l) for ident, g, l in run}
+            for run in json.loads(native.text("ti_model_bindings", self._ptr))]
+        self.dtype = None
 
-    # ------------------------------------------------------------------ parts
+    def __del__(self):
+        try:
+            if native._lib is not None and getattr(self, "_ptr", None):
+                native._lib.ti_model_release(self._ptr)
+        except Exception:  # noqa: BLE001
+            pass
+
     def parts(self):
         yield from self.embedding.walk()
         for b in self.blocks:
@@ -47,69 +75,5 @@ class Model:
         yield from self.head.walk()
 
     def tensors(self) -> Dict[str, TensorNeed]:
-        """Every checkpoint tensor the model asks for, in a fixed order.  A name
-        asked for twice (a tied head) must be asked for with one shape; it is
-        optional only if every asker says so."""
-        out: Dict[str, TensorNeed] = {}
-        for p in self.parts():
-            for name, need in p.tensors().items():
-                if name in out:
-                    old = out[name]
-                    if old.shape != need.shape or old.role != need.role:
-                        raise ValueError(f"tensor '{name}' is asked for as {old.shape}/{old.role} "
-                                         f"and as {need.shape}/{need.role}")
-                    if old.optional and not need.optional:
-                        out[name] = need
-                else:
-                    out[name] = need
-        return out
-
-    # ------------------------------------------------------------------ cache
-    def _group_cache(self):
-        """Give every run of a layer that keeps a cache a cache layer of its own,
-        and gather cache layers with the same need into groups (one page id
-        addresses a token's slot in every cache layer of its group).
-
-        A layer named twice in the run order computes different keys and values
-        each time, so each run has its own cache layer.  A layer with
-        `cache_from = j` keeps none: it reads what the latest earlier run of
-        layer j wrote (the first run of j if none came earlier).
-
-        `self.bindings[r][id(part)] = (group, cache_layer)` for run r.
-        """
-        index: Dict[object, int] = {}
-        counts: List[int] = []
-        layers = self.spec.layers
-        self.bindings: List[Dict[int, Tuple[int, int]]] = [dict() for _ in self.run_order]
-        runs_of: Dict[int, List[int]] = {}
-        for r, i in enumerate(self.run_order):
-            runs_of.setdefault(i, []).append(r)
-            if layers[i].cache_from is not None:
-                continue
-            for part in self.blocks[i].walk():
-                need = part.cache_need()
-                if need is None:
-                    continue
-                if need not in index:
-                    index[need] = len(counts)
-                    counts.append(0)
-                g = index[need]
-                self.bindings[r][id(part)] = (g, counts[g])
-                counts[g] += 1
-        for r, i in enumerate(self.run_order):
-            j = layers[i].cache_from
-            if j is None:
-                continue
-            if j not in runs_of or layers[j].cache_from is not None:
-                raise ValueError(f"layer {i} reads the cache of layer {j}, which keeps none")
-            earlier = [q for q in runs_of[j] if q < r]
-            src = earlier[-1] if earlier else runs_of[j][0]
-            theirs = [b for b in self.bindings[src].values()]
-            mine = [p for p in self.blocks[i].walk() if p.cache_need() is not None]
-            if len(theirs) != len(mine):
-                raise ValueError(f"layer {i} cannot read the cache of layer {j}: "
-                                 "they keep different numbers of caches")
-            for part, b in zip(mine, theirs):
-                self.bindings[r][id(part)] = b
-        needs = sorted(index, key=lambda n: index[n])
-        self.cache_groups: List[Tuple[object, int]] = [(n, counts[index[n]]) for n in needs]
+        """Every checkpoint tensor the model asks for, in a fixed order."""
+        return {n: TensorNeed.from_dict(v) for n, v in json.loads(native.text("ti_model_tensors", self._ptr)).items()}

@@ -2,4 +2,5 @@
 built-in kinds."""
 from .registry import register_part, build_part, registered_parts
 from .base import Part
-from . import norm, rotary, attention, ffn, embedding, block  # noqa: F401  (registration)
+from . import builtin  # noqa: F401  (registration)
+from .builtin import NativePart

@@ -1,7 +1,8 @@
 """Registry of parts by family and kind.
 
 Families: "embedding", "norm", "pos", "mixer", "ffn", "block", "head".
-A `PartSpec(kind, params)` is built by looking its kind up in its family.
+A `PartSpec(kind, params)` is built by looking its kind up in its family: among
+the kinds registered from Python first, then among the host library's own.
 """
 from __future__ import annotations
 

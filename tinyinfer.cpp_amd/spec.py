@@ -4,7 +4,8 @@ Nothing here computes.  An architecture's builder turns its typed configuration
 into a `ModelSpec`; the weight loader, the cache manager and the engine read
 only the spec, so an architecture with other parts in some layers, a layer that
 runs twice, or a layer that reads another layer's cache is a different list,
-not different code.
+not different code.  The host library has the same records (include/inference.h);
+a spec crosses as JSON.
 """
 from __future__ import annotations
 
@@ -20,15 +21,31 @@ class PartSpec:
     params: Dict[str, Any] = field(default_factory=dict)
     name: str = ""
 
+    def to_dict(self) -> dict:
+        return {"kind": self.kind, "params": _plain(self.params), "name": self.name}
+
+    @classmethod
+    def from_dict(cls, d) -> "PartSpec":
+        params = {k: (cls.from_dict(v) if isinstance(v, dict) and "kind" in v and "params" in v else v)
+                  for k, v in (d.get("params") or {}).items()}
+        return cls(d["kind"], params, d.get("name") or "")
+
+
+def _plain(v):
+    if isinstance(v, PartSpec):
+        return v.to_dict()
+    if isinstance(v, dict):
+        return {k: _plain(x) for k, x in v.items()}
+    if isinstance(v, (list, tuple)):
+        return [_plain(x) for x in v]
+    return v
+
 
 @dataclass
 class LayerSpec:
-    """One layer: a block arrangement over named parts.
-
-    `prefix` starts the names of the layer's tensors in the checkpoint.
-    `cache_from` names another layer (by index into `ModelSpec.layers`) whose
-    cache this layer's mixer reads instead of keeping one of its own.
-    """
+    """One layer: a block arrangement over named parts.  `prefix` starts the names of the
+    layer's tensors in the checkpoint.  `cache_from` names another layer (by index into
+    `ModelSpec.layers`) whose cache this layer's mixer reads instead of keeping one of its own."""
     prefix: str
     block: PartSpec
     parts: Dict[str, PartSpec]
@@ -52,6 +69,15 @@ class ModelSpec:
     def run_order(self) -> List[int]:
         return list(range(len(self.layers))) if self.schedule is None else list(self.schedule)
 
+    @classmethod
+    def from_dict(cls, d) -> "ModelSpec":
+        layers = [LayerSpec(l["prefix"], PartSpec.from_dict(l["block"]),
+                            {k: PartSpec.from_dict(v) for k, v in l["parts"].items()}, l.get("cache_from"))
+                  for l in d["layers"]]
+        return cls(d["architecture"], d["vocab_size"], d["hidden_size"], PartSpec.from_dict(d["embedding"]), layers,
+                   PartSpec.from_dict(d["final_norm"]), PartSpec.from_dict(d["lm_head"]), d.get("schedule"),
+                   tuple(d.get("eos_token_ids") or ()), d.get("max_position_embeddings"))
+
 
 # ----------------------------------------------------------------- tensor needs
 @dataclass(frozen=True)
@@ -61,13 +87,21 @@ class TensorNeed:
     role: "matrix"  — a matrix product operand, held in the engine's compute dtype
           "vector"  — a small vector used in 32-bit arithmetic, held in float32
           "table"   — an integer table, held in int32
-    init: how the random-weights mode fills it: ("normal", mean, std)
+    init: how the random-weights mode fills it: ("normal", mean, std), ("uniform", lo, hi), ("constant", v, 0)
     optional: absent from the checkpoint is allowed (the part copes)
     """
     shape: Tuple[int, ...]
     role: str = "matrix"
     init: Tuple[str, float, float] = ("normal", 0.0, 0.02)
     optional: bool = False
+
+    def to_dict(self) -> dict:
+        return {"shape": list(self.shape), "role": self.role, "init": self.init[0], "a": float(self.init[1]),
+                "b": float(self.init[2]), "optional": self.optional}
+
+    @classmethod
+    def from_dict(cls, d) -> "TensorNeed":
+        return cls(tuple(d["shape"]), d["role"], (d["init"], d["a"], d["b"]), d["optional"])
 
 
 # -------------------------------------------------------------------- cache needs
@@ -79,8 +113,22 @@ class PagedKVNeed:
     head_dim: int
     window: Optional[int] = None
 
+    def to_dict(self) -> dict:
+        return {"kind": "paged_kv", "kv_heads": self.kv_heads, "head_dim": self.head_dim, "window": self.window}
+
 
 @dataclass(frozen=True)
 class StateNeed:
     """Per-request state of fixed size (float32), zeroed when a request is admitted."""
     shape: Tuple[int, ...]
+
+    def to_dict(self) -> dict:
+        return {"kind": "state", "shape": list(self.shape)}
+
+
+def cache_need_from_dict(d):
+    if d is None:
+        return None
+    if d["kind"] == "state":
+        return StateNeed(tuple(d["shape"]))
+    return PagedKVNeed(d["kv_heads"], d["head_dim"], d.get("window"))
