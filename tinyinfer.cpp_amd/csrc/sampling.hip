@@ -10,6 +10,8 @@
 // which the descending cumulative mass reaches top_p, each by 32 steps of
 // bisection over the order-preserving integer image of the floats; every sum is
 // reduced in a fixed order, so the result is reproducible.
+#include <mutex>
+
 #include "common.h"
 #include "tinyinfer_kernels.h"
 
@@ -265,6 +267,48 @@ extern "C" int ti_argmax(const float* logits, int* out, void* scratch, int n_row
   } else {
     argmax_kernel<<<n_rows, SNT, 0, stream>>>(logits, out, V);
   }
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// The same greedy choice for callers that cannot allocate (code under HIP graph capture, tight
+// serving loops, harnesses that forbid hipMalloc): the two-stage kernels above, with their partial
+// results in a file-scope device array instead of a workspace argument.  Each GPU holds its own
+// copy of the array (128 KiB) until the process ends; its address on a device is asked for once,
+// with that device current, and kept.  Nothing in the array has to start at zero: the first stage
+// writes every slot of the rows it is given before the second stage reads them.  Every call on a
+// GPU shares that GPU's array, so calls that overlap on one GPU (two streams, two threads) race.
+#define ARGMAX_STATIC_MAX_ROWS 256
+static __device__ __align__(256) unsigned int scratch[2 * ARG_PARTS * ARGMAX_STATIC_MAX_ROWS];
+#define ARGMAX_STATIC_MAX_DEVICES 64
+static void* g_scratch_ptr[ARGMAX_STATIC_MAX_DEVICES];     // per device: where `scratch` lies there
+static std::mutex g_scratch_mutex;
+
+extern "C" int ti_argmax_static(const float* logits, int* out, int n_rows, int V, hipStream_t stream) {
+  TI_REQUIRE(n_rows >= 0 && V > 0, "argmax_static: bad sizes rows=%d V=%d", n_rows, V);
+  TI_REQUIRE(n_rows <= ARGMAX_STATIC_MAX_ROWS,
+             "argmax_static: %d rows are more than the %d its fixed scratch array serves (use ti_argmax with a workspace)",
+             n_rows, ARGMAX_STATIC_MAX_ROWS);
+  if (n_rows == 0) return 0;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  TI_REQUIRE(e == hipSuccess && dev >= 0 && dev < ARGMAX_STATIC_MAX_DEVICES, "argmax_static: no current device (%s)",
+             hipGetErrorString(e));
+  void* ptr;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      TI_REQUIRE(e == hipSuccess && p, "argmax_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      g_scratch_ptr[dev] = p;
+    }
+    ptr = g_scratch_ptr[dev];
+  }
+  float* pv = (float*)ptr;
+  int* pi = (int*)ptr + (size_t)n_rows * ARG_PARTS;
+  argmax_part_kernel<<<dim3(n_rows, ARG_PARTS), 256, 0, stream>>>(logits, pv, pi, V);
+  argmax_final_kernel<<<n_rows, 64, 0, stream>>>(pv, pi, out);
   TI_LAUNCH_CHECK();
   return 0;
 }

@@ -117,6 +117,13 @@ int ti_attention_prefill_paired_bf16(const void* q, const void* pool, const int*
 // out[r] = lowest index of the largest logit; scratch: 2 * 64 * n_rows four-byte words (two stages:
 // 64 workgroups per row, then one) or null (one workgroup reads a whole row)
 int ti_argmax(const float* logits, int* out, void* scratch, int n_rows, int V, hipStream_t stream);
+// ti_argmax for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+// harnesses that forbid hipMalloc): the same two-stage kernels with their partial results in a
+// device array of the library itself (128 KiB on each GPU it runs on, kept until the process ends)
+// instead of a workspace argument.  At most 256 rows, else an error.  It calls no hipMalloc, hipFree or
+// allocating routine; calls that overlap on one GPU share the array and race.  The reference has no
+// counterpart (its argmax needs no scratch: /root/reference/src/cuda/sample.cu:13-54).
+int ti_argmax_static(const float* logits, int* out, int n_rows, int V, hipStream_t stream);
 // temperature, top-k (0: all), top-p and one uniform number per row
 int ti_sample(const float* logits, const float* temp, const int* top_k, const float* top_p, const float* uni, int* out,
               int n_rows, int V, hipStream_t stream);
