@@ -1,30 +1,45 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model 0.6b|8b|32b] [--context N] [--prefill-tokens N]
 
 The default run has the layer sizes of Qwen3-0.6B with random weights in
 bfloat16: a batch of 8 requests, each holding 2,048 cached tokens (filled by
-real prefill steps), decoded for K steps through the serving path (scheduler's
-step function from a captured graph, greedy sampling on the device, the sampled
+real prefill steps), decoded for K steps through the serving path (the step
+function from a captured graph, greedy sampling on the device, the sampled
 token fed back).  One JSON line goes to stdout: `value` is decoded tokens a
 second at batch 8; `points` has batch 1 and 64; `prefill` a 2,048-token prompt in
 one step; `roofline` the decode step's bytes (every weight once, the cache of
-the live requests) over its time against 8 TB/s.
+the live requests) over its time against 8 TB/s.  Beside the fractions of the
+published peaks stand fractions of what this GPU delivers to a kernel that only
+reads memory, and to matrix-core instructions on registers (csrc/measure.hip),
+as the reference times its own kernels against the clock
+(/root/reference/src/selftest.cpp:392-428).
+
+`--model 8b` and `--model 32b` run the same with the sizes of Qwen3-8B and
+Qwen3-32B.  `--kernel-times` adds a table of the decode step's calls, timed with
+events (a line of its own on stderr).
 """
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import sys
 import time
 
-CONFIG = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=28, hidden_size=1024,
-              num_attention_heads=16, num_key_value_heads=8, head_dim=128, intermediate_size=3072,
-              vocab_size=151936, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
-              attention_bias=False, hidden_act="silu", max_position_embeddings=40960)
-CONTEXT = 2048            # cached tokens each decoding request holds
-MAX_SEQ = 4096            # context length a request may reach
-PREFILL_TOKENS = 2048
+BASE = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", head_dim=128, vocab_size=151936,
+            rope_theta=1000000.0, rms_norm_eps=1e-6, attention_bias=False, hidden_act="silu",
+            max_position_embeddings=40960)
+MODELS = {
+    "0.6b": dict(BASE, num_hidden_layers=28, hidden_size=1024, num_attention_heads=16, num_key_value_heads=8,
+                 intermediate_size=3072, tie_word_embeddings=True),
+    "8b": dict(BASE, num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+               intermediate_size=12288, tie_word_embeddings=False),
+    "32b": dict(BASE, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,
+                intermediate_size=25600, tie_word_embeddings=False),
+}
+NAMES = {"0.6b": "Qwen3-0.6B", "8b": "Qwen3-8B", "32b": "Qwen3-32B"}
+MAX_SEQ = 4096            # context length a request may reach (more if --context asks for it)
 PAGE = 16
 PEAK_HBM = 8.0e12         # bytes/s, MI355X
 PEAK_BF16 = 2.5e15        # dense bf16 MFMA flop/s, MI355X
@@ -42,6 +57,8 @@ def model_numbers(c):
     layer_params = (nq + 2 * nk) * H + H * nq + 3 * H * F
     norm_params = 2 * H + 2 * c["head_dim"]
     head_params = V * H
+    # a decode step reads every layer, the head's matrix (the embedding itself when tied) and one
+    # embedding row per token
     weight_bytes = L * (layer_params * 2 + norm_params * 4) + head_params * 2 + H * 4
     kv_bytes_per_token = 2 * nk * L * 2
     return dict(layer_params=layer_params, head_params=head_params, weight_bytes=weight_bytes,
@@ -56,30 +73,67 @@ def prefill_flops(c, T):
     return gemm + attn
 
 
-def fill(engine, rids, context, rng):
+def measured_peaks():
+    """(bytes/s of a kernel that only reads memory, flop/s of bfloat16 MFMAs on registers), the best of a few runs."""
+    import torch
+    from tinyinfer_amd import native
+    from tinyinfer_amd.csrc import build
+    native.ensure_kernels(["measure"])
+    lib = ctypes.CDLL(build.find("measure"))
+    lib.ti_measure_read.argtypes = [ctypes.c_void_p, ctypes.c_long, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+    lib.ti_measure_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    n = 4 << 30
+    buf = torch.empty(n, dtype=torch.uint8, device="cuda")
+    buf.fill_(1)
+    sink = torch.zeros(1 << 16, dtype=torch.int32, device="cuda")
+
+    def best(fn, reps=6):
+        t = []
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            assert fn() == 0
+            b.record()
+            b.synchronize()
+            t.append(a.elapsed_time(b) * 1e-3)
+        return min(t[1:])
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    read = n / best(lambda: lib.ti_measure_read(buf.data_ptr(), n, sink.data_ptr(), units * 16, None))
+    blocks, iters = units * 8, 4000
+    mfma = blocks * 4 * iters * 4 * 32768 / best(lambda: lib.ti_measure_mfma(blocks, iters, sink.data_ptr(), None))
+    del buf
+    torch.cuda.empty_cache()
+    return read, mfma
+
+
+def fill(engine, rids, context, rng, chunk=4096):
     """Give each request `context` cached tokens by real prefill steps."""
     import torch
     from tinyinfer_amd.engine import StepEntry
     V = engine.model.vocab_size
     for rid in rids:
-        toks = rng.integers(0, V, size=context).tolist()
-        engine.step([StepEntry(rid, toks, ())])
+        left = context
+        while left > 0:
+            n = min(left, chunk)
+            engine.step([StepEntry(rid, rng.integers(0, V, size=n).tolist(), ())])
+            left -= n
     torch.cuda.synchronize()
 
 
-def measure_decode(engine, sampler, batch, steps, warmup, rng, tag):
-    """tokens/s and ms/step of `steps` decode steps at `batch`, every request at CONTEXT tokens."""
+def measure_decode(engine, sampler, batch, steps, warmup, context, rng, tag, kernel_times=False):
+    """tokens/s and ms/step of `steps` decode steps at `batch`, every request at `context` tokens."""
     import torch
     from tinyinfer_amd.engine import StepEntry
     from tinyinfer_amd.sampling import SamplingParams
     rids = [f"{tag}{i}" for i in range(batch)]
-    fill(engine, rids, CONTEXT, rng)
+    fill(engine, rids, context, rng)
     greedy = [SamplingParams()] * batch
     nums = list(range(batch))
     last = rng.integers(0, engine.model.vocab_size, size=batch).tolist()
 
-    def one_step(tokens):
-        logits = engine.step_graph([StepEntry(r, [t], (0,)) for r, t in zip(rids, tokens)])
+    def one_step(tokens, graph=True):
+        entries = [StepEntry(r, [t], (0,)) for r, t in zip(rids, tokens)]
+        logits = engine.step_graph(entries) if graph else engine.step(entries)
         return sampler.sample(logits, greedy, nums, nums)            # reads the ids back: a full sync
 
     for _ in range(warmup):
@@ -90,21 +144,29 @@ def measure_decode(engine, sampler, batch, steps, warmup, rng, tag):
         last = one_step(last)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    table = None
+    if kernel_times:
+        one_step(last, graph=False)
+        engine.ops.timing(True)
+        for _ in range(4):
+            last = one_step(last, graph=False)
+        table = [dict(r, us=r["us"] / 4, calls=r["calls"] // 4) for r in engine.ops.timing_report()]
+        engine.ops.timing(False)
     for r in rids:
         engine.release(r)
-    return batch * steps / dt, dt / steps * 1e3
+    return batch * steps / dt, dt / steps * 1e3, table
 
 
-def measure_prefill(engine, rng, reps=5):
+def measure_prefill(engine, rng, tokens, reps=5):
     import torch
     from tinyinfer_amd.engine import StepEntry
     V = engine.model.vocab_size
     times = []
     for i in range(reps + 2):
-        toks = rng.integers(0, V, size=PREFILL_TOKENS).tolist()
+        toks = rng.integers(0, V, size=tokens).tolist()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        logits = engine.step([StepEntry("prefill", toks, (PREFILL_TOKENS - 1,))])
+        logits = engine.step([StepEntry("prefill", toks, (tokens - 1,))])
         logits[0, :8].cpu()
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
@@ -113,16 +175,17 @@ def measure_prefill(engine, rng, reps=5):
     return times[len(times) // 2]
 
 
-def measure_mixed(engine, batch, portion, cached, rng, reps=8):
-    """ms of a step that holds one decoded token of each of `batch` requests (CONTEXT tokens
-    each) beside `portion` tokens of a prompt of which `cached` tokens are in the cache already:
-    what the scheduler runs while a prompt arrives in portions.  Not a captured graph."""
+def measure_mixed(engine, batch, portion, cached, context, rng, reps=8):
+    """ms of a step that holds one decoded token of each of `batch` requests (`context` tokens each)
+    beside `portion` tokens of a prompt of which `cached` tokens are in the cache already: what the
+    scheduler runs while a prompt arrives in portions.  Not a captured graph.  Also the ms after
+    which the host has handed the whole step to the GPU."""
     import torch
     from tinyinfer_amd.engine import StepEntry
     V = engine.model.vocab_size
     rids = [f"x{i}" for i in range(batch)]
-    fill(engine, rids, CONTEXT, rng)
-    times = []
+    fill(engine, rids, context, rng)
+    times, host = [], []
     for i in range(reps + 3):
         if cached:
             engine.step([StepEntry("long", rng.integers(0, V, size=cached).tolist(), ())])
@@ -131,14 +194,24 @@ def measure_mixed(engine, batch, portion, cached, rng, reps=8):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         logits = engine.step(entries)
+        t1 = time.perf_counter()
         logits[0, :8].cpu()
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
+        host.append(t1 - t0)
         engine.release("long")
     for r in rids:
         engine.release(r)
-    times = sorted(times[3:])
-    return times[len(times) // 2] * 1e3
+    times, host = sorted(times[3:]), sorted(host[3:])
+    return times[len(times) // 2] * 1e3, host[len(host) // 2] * 1e3
+
+
+def print_table(table, title):
+    say(title)
+    total = sum(r["us"] for r in table)
+    for r in sorted(table, key=lambda r: -r["us"]):
+        say(f"  {r['us']:9.1f} us  {r['calls']:4d} calls  {r['us'] / max(1, r['calls']):7.2f} us each  {r['name']}")
+    say(f"  {total:9.1f} us  in all (events around every call; a graph replay leaves out the gaps between kernels)")
 
 
 def main() -> int:
@@ -146,9 +219,14 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--model", choices=sorted(MODELS), default="0.6b", help="whose layer sizes the model has")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=2048, help="cached tokens each decoding request holds")
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
+    ap.add_argument("--no-peaks", action="store_true", help="skip measuring the GPU's read bandwidth and MFMA rate")
+    ap.add_argument("--kernel-times", action="store_true", help="a table of the decode step's calls, timed with events")
     ap.add_argument("--only", choices=["all", "decode", "prefill", "mixed"], default="all",
                     help="measure one phase only (for profiles): the other's fields are null; "
                          "mixed: a step of --batch decoded tokens beside --portion tokens of a prompt, a line of its own")
@@ -165,61 +243,78 @@ def main() -> int:
     from tinyinfer_amd.engine import Engine
     from tinyinfer_amd.sampling import Sampler
 
-    cfg = dict(CONFIG)
+    cfg = dict(MODELS[args.model])
     layers_full = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     rng = np.random.default_rng(0)
+    context, prefill_tokens = args.context, args.prefill_tokens
+    max_seq = max(MAX_SEQ, context + args.warmup + args.steps + 64, prefill_tokens, args.cached + args.portion)
     biggest = max(args.batch, 1 if (args.no_points or args.only != "all") else 64)
-    say("building the model (random weights on the device) ...")
+    peaks = None
+    if not args.no_peaks and args.only != "mixed":
+        say("what the GPU delivers: a kernel that only reads, MFMAs on registers ...")
+        peaks = measured_peaks()
+        say(f"  read {peaks[0] / 1e9:.0f} GB/s, bf16 MFMA {peaks[1] / 1e12:.0f} TFLOP/s")
+    say(f"building the model ({NAMES[args.model]} sizes, random weights on the device) ...")
     engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", page_size=PAGE,
-                                max_tokens=biggest * (CONTEXT + 512) + PREFILL_TOKENS + args.cached + args.portion,
-                                max_requests=biggest + 1,
-                                max_seq=MAX_SEQ)
+                                max_tokens=biggest * (context + 512) + prefill_tokens + args.cached + args.portion,
+                                max_requests=biggest + 1, max_seq=max_seq)
     sampler = Sampler(engine.ops, engine.device)
     nums = model_numbers(cfg)
 
     if args.only == "mixed":
         say(f"a step of {args.batch} decoded tokens beside a portion of {args.portion} (after {args.cached} cached) ...")
-        ms = measure_mixed(engine, args.batch, args.portion, args.cached, rng)
-        print(json.dumps({"mixed": {"ms_per_step": round(ms, 3), "tokens": args.batch + args.portion,
+        ms, host_ms = measure_mixed(engine, args.batch, args.portion, args.cached, context, rng)
+        print(json.dumps({"mixed": {"ms_per_step": round(ms, 3), "host_ms": round(host_ms, 3), "tokens": args.batch + args.portion,
                                     "decoded": args.batch, "portion": args.portion, "cached": args.cached,
-                                    "decode_context": CONTEXT}}), flush=True)
+                                    "decode_context": context, "model": NAMES[args.model]}}), flush=True)
         return 0
     p_s = tps = ms = None
     if args.only != "decode":
-        say(f"prefill of {PREFILL_TOKENS} tokens ...")
-        p_s = measure_prefill(engine, rng)
+        say(f"prefill of {prefill_tokens} tokens ...")
+        p_s = measure_prefill(engine, rng, prefill_tokens)
     if args.only != "prefill":
         say(f"decode at batch {args.batch} ...")
-        tps, ms = measure_decode(engine, sampler, args.batch, args.steps, args.warmup, rng, "m")
+        tps, ms, table = measure_decode(engine, sampler, args.batch, args.steps, args.warmup, context, rng, "m",
+                                        args.kernel_times)
+        if table:
+            print_table(table, f"a decode step at batch {args.batch}, call by call (not from the graph):")
     points = {}
     if not args.no_points and args.only == "all":
         for b, k in ((1, args.steps), (64, max(16, args.steps // 4))):
             say(f"decode at batch {b} ...")
-            points[f"decode_b{b}"] = round(measure_decode(engine, sampler, b, k, max(4, args.warmup // 2), rng, f"p{b}_")[0], 1)
+            points[f"decode_b{b}"] = round(measure_decode(engine, sampler, b, k, max(4, args.warmup // 2), context, rng,
+                                                          f"p{b}_")[0], 1)
 
-    ctx_mean = CONTEXT + args.warmup + args.steps / 2.0
+    ctx_mean = context + args.warmup + args.steps / 2.0
     step_bytes = nums["weight_bytes"] + args.batch * ctx_mean * nums["kv_bytes_per_token"]
     achieved = step_bytes / (ms * 1e-3) if ms else None
+    roofline = prefill = None
+    if achieved is not None:
+        roofline = {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+                    "frac": round(achieved / PEAK_HBM, 4)}
+        if peaks:
+            roofline.update(measured_read=round(peaks[0] / 1e9, 1), frac_of_measured=round(achieved / peaks[0], 4))
+    if p_s is not None:
+        flops = prefill_flops(cfg, prefill_tokens)
+        prefill = {"value": round(prefill_tokens / p_s, 1), "tokens": prefill_tokens, "ms": round(p_s * 1e3, 3),
+                   "frac": round(flops / p_s / PEAK_BF16, 4)}
+        if peaks:
+            prefill.update(measured_mfma_tflops=round(peaks[1] / 1e12, 1), frac_of_measured=round(flops / p_s / peaks[1], 4))
     out = {
-        "metric": f"decode tok/s @ batch {args.batch} (Qwen3-0.6B sizes, 2,048 cached tokens per request)",
+        "metric": f"decode tok/s @ batch {args.batch} ({NAMES[args.model]} sizes, {context:,} cached tokens per request)",
         "value": None if tps is None else round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": None if ms is None else round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic (uniform random token ids, random weights N(0, 0.02))",
-        "config": {"model": "Qwen3-0.6B sizes", "layers": cfg["num_hidden_layers"], "layers_in_config": layers_full,
+        "config": {"model": f"{NAMES[args.model]} sizes", "layers": cfg["num_hidden_layers"], "layers_in_config": layers_full,
                    "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
-                   "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"], "tied_head": True,
-                   "global_batch": args.batch, "cached_tokens": CONTEXT, "seq_len": MAX_SEQ, "page_size": PAGE,
-                   "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU", "decode_graph": True},
-        "prefill": None if p_s is None else
-        {"value": round(PREFILL_TOKENS / p_s, 1), "tokens": PREFILL_TOKENS, "ms": round(p_s * 1e3, 3),
-         "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / p_s / PEAK_BF16, 4)},
-        "roofline": None if achieved is None else
-        {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
-         "frac": round(achieved / PEAK_HBM, 4)},
-        "points": points,
+                   "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
+                   "tied_head": bool(cfg["tie_word_embeddings"]),
+                   "global_batch": args.batch, "cached_tokens": context, "seq_len": max_seq, "page_size": PAGE,
+                   "prefill_tokens": prefill_tokens, "parallelism": "single GPU", "decode_graph": True},
+        "prefill": prefill, "roofline": roofline, "points": points,
     }
     print(json.dumps(out), flush=True)
     return 0

@@ -390,6 +390,24 @@ def test_sample_limits_reduce_to_argmax(ops):
     assert run_sample(ops, logits, 1.0, 0, 1e-6, u) == want          # top-p -> 0
 
 
+def test_sample_keeps_every_logit_equal_to_the_kth(ops):
+    """Equal logits at the cut: top-k keeps every logit that is no smaller than the k-th largest, so the kept
+    set may hold more than k (the reference's nth_element picks among equals arbitrarily and keeps exactly k:
+    /root/reference/src/main.cpp:47-53; which of the equals it keeps is not defined, so parity is unpinned
+    there).  With logits [1, 3, 2, 2, 2, 0] and k = 2 the kept set is {1, 2, 3, 4}: weights e^1 : 1 : 1 : 1 at
+    T = 1, and a uniform number near the end of [0, 1) draws index 4, which a cut to exactly two would never do."""
+    row = torch.tensor([[1.0, 3.0, 2.0, 2.0, 2.0, 0.0]])
+    e = math.e
+    edges = [e / (e + 3), (e + 1) / (e + 3), (e + 2) / (e + 3)]
+    u = [0.01, edges[0] - 0.01, edges[0] + 0.01, edges[1] + 0.01, edges[2] + 0.01, 0.999]
+    got = run_sample(ops, row.repeat(len(u), 1), 1.0, 2, 1.0, u)
+    assert got == [1, 1, 2, 3, 4, 4]
+    # and the plain sampler says the same
+    from plain.qwen3_plain import sample_distribution, draw
+    p = sample_distribution(row[0].double().numpy(), 1.0, 2, 1.0)
+    assert [draw(p, x) for x in u] == got
+
+
 def test_sample_matches_inverse_cdf(ops):
     """The draw is the inverse CDF of softmax(l/T) over the index order at u."""
     from plain.qwen3_plain import sample_distribution

@@ -38,11 +38,24 @@ def run_requests(engine: Engine, scheduler: Scheduler, sampler: Optional[Sampler
     generated token.  When a step fails, every request the scheduler still holds is given back
     to the cache before the error is raised."""
     native.ensure_kernels(["sampling"])
-    callback = native.ON_TOKEN(lambda number, token: on_token(scheduler._requests[number], token)) if on_token else \
-        ctypes_null(native.ON_TOKEN)
+    raised = []
+
+    def relay(number, token):
+        try:
+            on_token(scheduler._requests[number], token)
+            return 0
+        except BaseException as e:  # noqa: BLE001  (it must not unwind through the library: the run is stopped there)
+            raised.append(e)
+            return 1
+
+    callback = native.ON_TOKEN(relay) if on_token else ctypes_null(native.ON_TOKEN)
     try:
         out = native.text("ti_run_requests", engine._ptr, scheduler._ptr, sampler._ptr if sampler else None,
                           int(use_graph), callback)
+    except native.EngineError:
+        if raised:
+            raise raised[0] from None
+        raise
     finally:
         native.forget_contexts()
     if stats is not None:

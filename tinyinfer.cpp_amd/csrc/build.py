@@ -46,6 +46,7 @@ SOURCES: Dict[str, str] = {
     "sampling": "sampling.hip",
     "gemm_bf16": "gemm_bf16.hip",
     "attention_bf16": "attention_bf16.hip",
+    "measure": "measure.hip",
 }
 
 

@@ -128,6 +128,14 @@ int ti_argmax_static(const float* logits, int* out, int n_rows, int V, hipStream
 int ti_sample(const float* logits, const float* temp, const int* top_k, const float* top_p, const float* uni, int* out,
               int n_rows, int V, hipStream_t stream);
 
+
+// ---- libti_measure: what the GPU delivers, for the bench tool's fractions
+// reads `bytes` bytes (a multiple of 16) once with `blocks` workgroups of 256 threads; sink: `blocks` words
+int ti_measure_read(const void* p, long bytes, void* sink, int blocks, hipStream_t stream);
+// `blocks` workgroups of four wavefronts, each wavefront `iters` rounds of four 32x32x16 bfloat16 MFMAs on
+// registers: blocks * 4 * iters * 4 * 32,768 flops
+int ti_measure_mfma(int blocks, int iters, void* sink, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

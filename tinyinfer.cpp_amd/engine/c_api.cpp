@@ -895,13 +895,16 @@ int ti_scheduler_request(void* scheduler, int64_t number, const char** out) {
   return give(out, request_json(*it->second).dump());
   TI_END
 }
-int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph, void (*on_token)(int64_t, int),
+int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph, int (*on_token)(int64_t, int),
                     const char** out_stats) {
   TI_BEGIN
   SchedulerHandle& h = *static_cast<SchedulerHandle*>(scheduler);
   GenerationStats st;
   std::function<void(const Request&, int)> cb;
-  if (on_token) cb = [on_token](const Request& r, int tok) { on_token(r.number, tok); };
+  if (on_token)
+    cb = [on_token](const Request& r, int tok) {
+      if (on_token(r.number, tok) != 0) throw EngineError("the token callback stopped the run");
+    };
   run_requests(*static_cast<Engine*>(engine), *h.s, static_cast<Sampler*>(sampler), &st, cb, use_graph != 0);
   Json j = Json::object();
   j.set("prefill_ms", st.prefill_ms);
@@ -1068,6 +1071,8 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     ops.sample(arg(0), fptr(1), iptr(2), fptr(3), fptr(4), arg(5).ptr<int>());
   } else if (op == "flush") {
     ops.flush();
+  } else if (op == "timing") {
+    ops.timing(num(0) != 0);
   } else if (op == "pending") {
     answer(ops.pending_splits());
   } else if (op == "can_fuse_norm") {
@@ -1089,6 +1094,19 @@ int ti_portion_launch(int n_tiles_small, int heads, int portion_context, int win
   const int s = Ops::portion_launch(n_tiles_small, heads, portion_context, window, units, &p);
   if (paired) *paired = p ? 1 : 0;
   return s;
+}
+int ti_ops_timing_report(void* ops_, const char** out) {
+  TI_BEGIN
+  Json a = Json::array();
+  for (const auto& t : static_cast<Ops*>(ops_)->timing_report()) {
+    Json j = Json::object();
+    j.set("name", t.name);
+    j.set("calls", t.calls);
+    j.set("us", t.us);
+    a.push(j);
+  }
+  return give(out, a.dump());
+  TI_END
 }
 int ti_decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units) {
   return Ops::decode_splits(n_rows, kv_heads, heads, context, typical, units);

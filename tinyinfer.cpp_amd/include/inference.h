@@ -297,6 +297,12 @@ class Ops {
   // the norm that would have added them).  Every launch through this object does it first.
   void flush();
   int pending_splits() const { return pending_.out ? pending_.splits : 0; }   // 0: no sums are waiting
+  // Per-call timing with events (the reference's selftest times its kernels the same way:
+  // /root/reference/src/selftest.cpp:404-424): while on, every call records an event before and
+  // after what it launches; the report waits for them and gives (name with sizes, calls, microseconds).
+  void timing(bool on);
+  struct Timed { std::string name; int calls = 0; double us = 0; };
+  std::vector<Timed> timing_report();
 
   // switches for tests and measurements: each leaves the results the same up to the order of sums
   struct Switches {
@@ -315,6 +321,9 @@ class Ops {
   DeviceBuffer partials_;
   DeviceBuffer argmax_scratch_;
   struct { void* out = nullptr; int64_t count = 0; int splits = 0; } pending_;
+  struct Timing;
+  friend struct TimedScope;
+  std::unique_ptr<Timing> timing_;
 };
 
 // Activation rows handed from a norm to its consumer: computed (`t`), or, when the consumer
@@ -919,8 +928,9 @@ int ti_scheduler_abort(void* scheduler, int64_t number);
 int ti_scheduler_set_next_number(void* scheduler, int64_t number);
 int ti_scheduler_state(void* scheduler, const char** out_json);
 int ti_scheduler_request(void* scheduler, int64_t number, const char** out_json);
+// on_token returns 0; anything else stops the run (the requests still held are given back, and the call fails)
 int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph,
-                    void (*on_token)(int64_t number, int token), const char** out_stats_json);
+                    int (*on_token)(int64_t number, int token), const char** out_stats_json);
 
 // the kernels through an Ops object (what the kernel tests and foreign parts call)
 int ti_ops_create(void* stream, void** out);
@@ -928,6 +938,7 @@ void ti_ops_release(void* ops);
 int ti_ops_switch(void* ops, const char* name, int value, int* old);
 int ti_ops_call(void* ops, const char* op, const ti_tensor* t, int n_t, const double* scalars, int n_scalars,
                 const char* text, ti_tensor* result);
+int ti_ops_timing_report(void* ops, const char** out_json);     // [{"name", "calls", "us"}] since timing was switched on
 int ti_decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units);
 int ti_portion_launch(int n_tiles_small, int heads, int portion_context, int window, int units, int* paired);
 }

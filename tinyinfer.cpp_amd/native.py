@@ -77,7 +77,7 @@ _ERRORS = {"ConfigError": ConfigError, "CacheError": CacheError, "OutOfPages": O
 FOREIGN_CALL = ctypes.CFUNCTYPE(c_int, c_u64, c_char_p, c_void_p, P(ti_tensor), c_int, c_char_p, P(ti_tensor))
 ALLOC = ctypes.CFUNCTYPE(c_void_p, c_void_p, c_size_t)
 RELEASE = ctypes.CFUNCTYPE(None, c_void_p, c_void_p)
-ON_TOKEN = ctypes.CFUNCTYPE(None, c_i64, c_int)
+ON_TOKEN = ctypes.CFUNCTYPE(c_int, c_i64, c_int)
 
 _OUT_TEXT = P(c_char_p)
 _OUT_PTR = P(c_void_p)
@@ -150,6 +150,7 @@ _SIGNATURES = {
     "ti_run_requests": [c_void_p, c_void_p, c_void_p, c_int, ON_TOKEN, _OUT_TEXT],
     "ti_ops_create": [c_void_p, _OUT_PTR],
     "ti_ops_switch": [c_void_p, c_char_p, c_int, P(c_int)],
+    "ti_ops_timing_report": [c_void_p, _OUT_TEXT],
     "ti_ops_call": [c_void_p, c_char_p, _TT, c_int, P(c_double), c_int, c_char_p, _TT],
 }
 _VOID = {"ti_part_release": [c_void_p], "ti_ctx_release": [c_void_p], "ti_model_release": [c_void_p],

@@ -191,6 +191,15 @@ class Ops:
         """The number of partial sums a product left for the next norm (None: none are waiting)."""
         return self._call("pending", libs=["core"]) or None
 
+    def timing(self, on: bool) -> None:
+        """Switch per-call timing with events on or off (see `Ops::timing`)."""
+        self._call("timing", [], [int(bool(on))], libs=["core"])
+
+    def timing_report(self):
+        """[{"name", "calls", "us"}] of the calls since timing was switched on (or last reported)."""
+        import json
+        return json.loads(native.text("ti_ops_timing_report", self._ptr))
+
     def flush(self):
         """Partial sums that a product left for the next norm are added now (same bits).  Every launch
         through this object does it first; code that reads such a residual with torch calls it itself."""

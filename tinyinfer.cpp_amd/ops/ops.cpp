@@ -268,8 +268,80 @@ bool kernel_library_available(const std::string& name) {
 static const int64_t PARTIALS_BYTES = 4 << 20;
 static const int NORMED_MAX_ROWS = 16;
 
+struct Ops::Timing {
+  struct Rec { std::string name; hipEvent_t a, b; };
+  std::vector<Rec> recs;
+  int depth = 0;
+};
 Ops::Ops(void* stream) : stream_(stream) {}
-Ops::~Ops() {}
+Ops::~Ops() {
+  if (timing_)
+    for (auto& r : timing_->recs) {
+      (void)hipEventDestroy(r.a);
+      (void)hipEventDestroy(r.b);
+    }
+}
+
+void Ops::timing(bool on) {
+  flush();
+  if (on && !timing_) timing_.reset(new Timing());
+  if (!on && timing_) {
+    timing_report();
+    timing_.reset();
+  }
+}
+
+std::vector<Ops::Timed> Ops::timing_report() {
+  std::vector<Timed> out;
+  if (!timing_) return out;
+  hip_check(hipStreamSynchronize((hipStream_t)stream_), "hipStreamSynchronize");
+  std::map<std::string, size_t> index;
+  for (auto& r : timing_->recs) {
+    float ms = 0.f;
+    (void)hipEventElapsedTime(&ms, r.a, r.b);
+    auto it = index.find(r.name);
+    if (it == index.end()) {
+      it = index.emplace(r.name, out.size()).first;
+      out.push_back({r.name, 0, 0.0});
+    }
+    out[it->second].calls += 1;
+    out[it->second].us += ms * 1e3;
+    (void)hipEventDestroy(r.a);
+    (void)hipEventDestroy(r.b);
+  }
+  timing_->recs.clear();
+  return out;
+}
+
+// Events around what one call launches, when timing is on (the outermost call only).
+struct TimedScope {
+  Ops& ops;
+  bool active = false;
+  size_t index = 0;
+  template <class F> TimedScope(Ops& o, F&& name) : ops(o) {
+    if (!ops.timing_) return;
+    if (ops.timing_->depth++ > 0) return;
+    if (ops.pending_.out) ops.flush();          // the sums of the call before are not this call's time
+    Ops::Timing::Rec r;
+    r.name = name();
+    if (hipEventCreate(&r.a) != hipSuccess || hipEventCreate(&r.b) != hipSuccess) return;
+    (void)hipEventRecord(r.a, (hipStream_t)ops.stream_);
+    index = ops.timing_->recs.size();
+    ops.timing_->recs.push_back(r);
+    active = true;
+  }
+  ~TimedScope() {
+    if (!ops.timing_) return;
+    --ops.timing_->depth;
+    if (active) (void)hipEventRecord(ops.timing_->recs[index].b, (hipStream_t)ops.stream_);
+  }
+};
+static std::string dims(const Tensor& t) {
+  std::string s;
+  for (int i = 0; i < t.ndim; ++i) s += (i ? "x" : "") + std::to_string(t.shape[i]);
+  return s;
+}
+#define TIMED(expr) TimedScope timed_scope_(*this, [&]() -> std::string { return expr; })
 
 int Ops::compute_units() {
   if (!units_) {
@@ -304,6 +376,7 @@ const Tensor& Rows::materialize(Ops& ops) const {
 }
 
 void Ops::embed(const Tensor& table, const int* tokens, int64_t M, const Tensor& x) {
+  TIMED("embed " + dims(x));
   require(table.ndim == 2 && x.ndim == 2, "embed: table and x must be matrices");
   const int64_t V = table.shape[0], H = table.shape[1];
   require(x.shape[0] == M && x.shape[1] == H && x.dtype == DType::F32,
@@ -315,6 +388,7 @@ void Ops::embed(const Tensor& table, const int* tokens, int64_t M, const Tensor&
 }
 
 void Ops::rmsnorm(const Tensor& x, const Tensor& w, float eps, const Tensor& out, const int* rows, int64_t n_rows) {
+  TIMED(std::string(pending_.out ? "rmsnorm+partials " : "rmsnorm ") + std::to_string(rows ? n_rows : x.shape[0]) + "x" + std::to_string(x.shape[1]));
   require(x.ndim == 2, "rmsnorm: x must be a matrix");
   const int64_t H = x.shape[1];
   const int64_t n = rows ? n_rows : x.shape[0];
@@ -341,6 +415,7 @@ void Ops::rmsnorm(const Tensor& x, const Tensor& w, float eps, const Tensor& out
 }
 
 void Ops::rope_neox(const Tensor& x, const int* positions, const Tensor& inv_freq) {
+  TIMED("rope_neox " + dims(x));
   require(x.ndim == 3 && x.dtype == DType::F32 && x.stride[2] == 1 && x.stride[1] == x.shape[2],
           "rope: x must be float32 [M, heads, hd] with contiguous heads");
   const int64_t M = x.shape[0], heads = x.shape[1], hd = x.shape[2];
@@ -371,6 +446,7 @@ static void check_pool(const char* what, const Tensor& pool, int kv_heads, int h
 void Ops::qk_norm_rope_kv_write(const Tensor& qkv, const float* q_w, const float* k_w, float eps, const Rotation& rot,
                                 const int* positions, const int* slots, const CacheView& view, const Tensor& pool,
                                 const Tensor& q_out, int heads, int kv_heads, int head_dim) {
+  TIMED("qk_norm_rope_kv_write " + dims(qkv));
   const int64_t M = qkv.shape[0];
   const int64_t width = (int64_t)(heads + 2 * kv_heads) * head_dim;
   require(qkv.ndim == 2 && qkv.shape[1] == width && qkv.dtype == DType::F32 && qkv.contiguous(),
@@ -392,6 +468,7 @@ void Ops::qk_norm_rope_kv_write(const Tensor& qkv, const float* q_w, const float
 
 void Ops::qk_norm_inplace(const Tensor& qkv, const float* q_w, const float* k_w, float eps, int heads, int kv_heads,
                           int head_dim) {
+  TIMED("qk_norm_inplace " + dims(qkv));
   require(qkv.ndim == 2 && qkv.dtype == DType::F32 && qkv.contiguous() &&
               qkv.shape[1] >= (int64_t)(heads + kv_heads) * head_dim,
           "qk_norm_inplace: qkv " + qkv.describe() + " does not hold " + std::to_string(heads) + " + " +
@@ -408,6 +485,8 @@ bool Ops::can_fuse_norm(int64_t n_rows, DType dtype) const {
 }
 
 bool Ops::linear_with_norm(const Rows& a, const Tensor& w, const Tensor& out, Epilogue epi) {
+  static const char* EPI_NAMES[] = {"store", "add", "store_act", "swiglu"};
+  TIMED(std::string("norm+linear.") + EPI_NAMES[epi] + " " + dims(a.t) + " * " + dims(w));
   const int64_t M = a.t.shape[0], K = a.t.shape[1];
   if (!can_fuse_norm(M, a.t.dtype) || w.dtype != DType::BF16) return false;
   const int64_t rows = w.shape[0];
@@ -437,6 +516,8 @@ void Ops::linear(const Rows& a, const Tensor& w, const Tensor& out, Epilogue epi
 }
 
 void Ops::linear(const Tensor& a, const Tensor& w, const Tensor& out, Epilogue epi, bool may_defer) {
+  static const char* EPI_NAMES[] = {"store", "add", "store_act", "swiglu"};
+  TIMED(std::string("linear.") + EPI_NAMES[epi] + " " + dims(a) + " * " + dims(w));
   require(a.ndim == 2 && w.ndim == 2, "linear: a and w must be matrices");
   const int64_t M = a.shape[0], K = a.shape[1], rows = w.shape[0];
   const int64_t N = epi == SwiGLU ? rows / 2 : rows;
@@ -485,6 +566,7 @@ void Ops::linear(const Tensor& a, const Tensor& w, const Tensor& out, Epilogue e
 bool Ops::qkv_prepared(const Rows& a, const Tensor& w, const float* q_w, const float* k_w, float eps, const Rotation& rot,
                        const int* positions, const int* slots, const CacheView& view, const Tensor& pool,
                        const Tensor& q_out, int heads, int kv_heads, int head_dim) {
+  TIMED("qkv_prepared " + dims(a.t) + " * " + dims(w));
   if (!(use.fused_qkv_prefill && use.fast_gemm) || a.lazy) return false;
   if (a.t.dtype != DType::BF16 || w.dtype != DType::BF16 || q_out.dtype != DType::BF16) return false;
   if (!kernel_library_available("gemm_bf16")) return false;
@@ -512,6 +594,7 @@ bool Ops::qkv_prepared(const Rows& a, const Tensor& w, const float* q_w, const f
 // ---------------------------------------------------------------------------------- attention
 void Ops::attention_rows(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
                          const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window) {
+  TIMED("attention_rows " + dims(q));
   const int64_t M = q.shape[0];
   require(q.ndim == 2 && q.shape[1] == (int64_t)heads * head_dim && out.ndim == 2 && out.shape[0] == M &&
               out.shape[1] == q.shape[1] && q.dtype == pool.dtype && out.dtype == q.dtype,
@@ -583,6 +666,7 @@ bool Ops::attention_from_projections(const AttentionWork& work, Workspace& ws, c
                                      const float* q_w, const float* k_w, float eps, const Rotation& rot,
                                      const Tensor& pool, bool write_kv, const Tensor& out, int heads, int kv_heads,
                                      int head_dim, float scale, int window) {
+  TIMED("attention.decode_prepared rows=" + std::to_string(work.M) + " context<=" + std::to_string(work.max_context));
   if (!(use.fused_qk_decode && use.fast_attention && work.decode_only && pool.dtype == DType::BF16)) return false;
   if (!kernel_library_available("attention_bf16")) return false;
   const int64_t M = qkv.shape[0];
@@ -615,6 +699,7 @@ bool Ops::attention_from_projections(const AttentionWork& work, Workspace& ws, c
 
 void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& view, const Tensor& q, const Tensor& pool,
                     const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window) {
+  TIMED("attention rows=" + std::to_string(work.M) + (work.decode_only ? " decode" : " tiles=" + std::to_string(work.n_tiles) + " single=" + std::to_string(work.n_decode_rows)) + " context<=" + std::to_string(work.max_context));
   bool done = false;
   if (q.dtype == DType::BF16 && use.fast_attention && kernel_library_available("attention_bf16")) {
     check_pool("attention", pool, kv_heads, head_dim, DType::BF16);
@@ -676,6 +761,7 @@ void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& v
 
 // ----------------------------------------------------------------------------------- sampling
 void Ops::argmax(const Tensor& logits, int* out) {
+  TIMED("argmax " + dims(logits));
   require(logits.ndim == 2 && logits.dtype == DType::F32 && logits.contiguous(),
           "argmax: logits must be contiguous float32 [n, V]");
   const int64_t n = logits.shape[0];
@@ -691,6 +777,7 @@ void Ops::argmax(const Tensor& logits, int* out) {
 
 void Ops::sample(const Tensor& logits, const float* temperature, const int* top_k, const float* top_p,
                  const float* uniform, int* out) {
+  TIMED("sample " + dims(logits));
   require(logits.ndim == 2 && logits.dtype == DType::F32 && logits.contiguous(),
           "sample: logits must be contiguous float32 [n, V]");
   int rc = KERNEL("sampling", ti_sample)((const float*)logits.data, temperature, top_k, top_p, uniform, out,
