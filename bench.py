@@ -274,6 +274,12 @@ def main() -> int:
     if args.only != "decode":
         say(f"prefill of {prefill_tokens} tokens ...")
         p_s = measure_prefill(engine, rng, prefill_tokens)
+        if args.kernel_times:
+            engine.ops.timing(True)
+            measure_prefill(engine, rng, prefill_tokens, reps=2)
+            table = [dict(r, us=r["us"] / 4, calls=r["calls"] // 4) for r in engine.ops.timing_report()]
+            engine.ops.timing(False)
+            print_table(table, f"a prefill step of {prefill_tokens} tokens, call by call:")
     if args.only != "prefill":
         say(f"decode at batch {args.batch} ...")
         tps, ms, table = measure_decode(engine, sampler, args.batch, args.steps, args.warmup, context, rng, "m",

@@ -61,3 +61,17 @@ extern "C" int ti_measure_mfma(int blocks, int iters, void* sink, hipStream_t st
   TI_LAUNCH_CHECK();
   return 0;
 }
+
+// every workgroup reads one word every `stride` bytes of [p, p + bytes): address translations and nothing else
+__global__ void __launch_bounds__(64) touch_kernel(const char* __restrict__ p, long bytes, long stride, unsigned* __restrict__ sink) {
+  unsigned acc = 0;
+  for (long off = (long)threadIdx.x * stride; off < bytes; off += 64 * stride) acc += *(const unsigned*)(p + off);
+  if (acc == 0x9e3779b9u) sink[blockIdx.x] = acc;
+}
+
+extern "C" int ti_measure_touch(const void* p, long bytes, long stride, void* sink, int blocks, hipStream_t stream) {
+  TI_REQUIRE(bytes > 0 && stride >= 4 && stride % 4 == 0 && blocks > 0, "measure_touch: bad sizes");
+  touch_kernel<<<blocks, 64, 0, stream>>>((const char*)p, bytes, stride, (unsigned*)sink);
+  TI_LAUNCH_CHECK();
+  return 0;
+}

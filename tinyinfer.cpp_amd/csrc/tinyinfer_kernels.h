@@ -135,6 +135,8 @@ int ti_measure_read(const void* p, long bytes, void* sink, int blocks, hipStream
 // `blocks` workgroups of four wavefronts, each wavefront `iters` rounds of four 32x32x16 bfloat16 MFMAs on
 // registers: blocks * 4 * iters * 4 * 32,768 flops
 int ti_measure_mfma(int blocks, int iters, void* sink, hipStream_t stream);
+// `blocks` workgroups of one wavefront each read one word every `stride` bytes of [p, p + bytes)
+int ti_measure_touch(const void* p, long bytes, long stride, void* sink, int blocks, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -949,7 +949,10 @@ int ti_ops_switch(void* ops_, const char* name_, int value, int* old) {
   else if (name == "deferred_add") flag(ops.use.deferred_add);
   else if (name == "paired_prefill") flag(ops.use.paired_prefill);
   else if (name == "portion_splits") flag(ops.use.portion_splits);
-  else if (name == "force_paired_tiles") {
+  else if (name == "force_decode_splits") {
+    if (old) *old = ops.use.force_decode_splits;
+    if (value >= 0) ops.use.force_decode_splits = value;
+  } else if (name == "force_paired_tiles") {
     if (old) *old = ops.use.force_paired_tiles;
     if (value >= -1) ops.use.force_paired_tiles = value;
   } else {

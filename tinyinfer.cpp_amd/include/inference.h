@@ -309,6 +309,7 @@ class Ops {
     bool fast_gemm = true, fast_attention = true, fused_norm = true, fused_qk_decode = true, fused_qkv_prefill = true;
     bool split_k_add = true, deferred_add = true, paired_prefill = true, portion_splits = true;
     int force_paired_tiles = -1;    // 1 / 0: that kernel with / without pairs, whatever the launch
+    int force_decode_splits = 0;    // > 0: the decode attention cuts every context into this many runs
   } use;
   static int decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units);
   // runs of keys for the prefill kernel with 64-row tiles, and whether it pairs a heavy with a light tile

@@ -131,6 +131,10 @@ class Ops:
             return bool(old.value)
         if name == "_pending":
             return type(self)._pending.fget(self)
+        if name == "force_decode_splits":
+            old = ctypes.c_int()
+            native.call("ti_ops_switch", self._ptr, b"force_decode_splits", -1, ctypes.byref(old))
+            return old.value
         if name == "force_paired_tiles":
             old = ctypes.c_int()
             native.call("ti_ops_switch", self._ptr, b"force_paired_tiles", -2, ctypes.byref(old))
@@ -140,6 +144,8 @@ class Ops:
     def __setattr__(self, name, value):
         if name in _SWITCHES:
             native.call("ti_ops_switch", self._ptr, _SWITCHES[name].encode(), int(bool(value)), None)
+        elif name == "force_decode_splits":
+            native.call("ti_ops_switch", self._ptr, b"force_decode_splits", int(value or 0), None)
         elif name == "force_paired_tiles":
             native.call("ti_ops_switch", self._ptr, b"force_paired_tiles", -1 if value is None else int(bool(value)), None)
         else:

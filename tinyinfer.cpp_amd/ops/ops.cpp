@@ -682,7 +682,8 @@ bool Ops::attention_from_projections(const AttentionWork& work, Workspace& ws, c
   if ((head_dim != 64 && head_dim != 128) || P % 16 != 0 || heads / kv_heads > 16) return false;
   const int n = (int)work.M;
   const int context = window == 0 ? work.split_context : std::min(work.split_context, window + 16);
-  const int S = decode_splits(n, kv_heads, heads, context, std::min(context, typical_context(work)), compute_units());
+  int S = decode_splits(n, kv_heads, heads, context, std::min(context, typical_context(work)), compute_units());
+  if (use.force_decode_splits > 0) S = std::min(use.force_decode_splits, std::max(1, (context + 15) / 16));
   float *part_o = nullptr, *part_ml = nullptr;
   if (S > 1) {
     part_o = (float*)ws.get("attn.part_o", (size_t)n * heads * S * head_dim * 4);
