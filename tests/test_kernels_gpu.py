@@ -56,6 +56,26 @@ def test_rmsnorm_reference_vector(ops):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H", [4100, 5120, 8192, 8196, 17000])
+def test_rmsnorm_wide_rows(ops, dtype, H):
+    """Rows wider than 4,096 take a workgroup per row: whole, gathered, with one element that dominates."""
+    g = torch.Generator().manual_seed(H)
+    x = torch.randn(7, H, generator=g) * 2
+    x[3, H - 1] = 300.0
+    w = 1 + 0.1 * torch.randn(H, generator=g)
+    rows = torch.tensor([6, 3, 3, 0], dtype=torch.int32)
+    out = torch.empty(7, H, device="cuda", dtype=DT[dtype])
+    ops.rmsnorm(dev(x), dev(w), 1e-6, out)
+    ref = ref_rmsnorm(x, w, 1e-6)
+    # bfloat16 keeps 8 bits: half a unit in the last place is 2^-9 of the value (the dominant element is ~60)
+    allowed = 1e-5 * (1 + ref.abs()) if dtype == "float32" else 2.0 ** -8 * ref.abs() + 1e-3
+    assert bool(((f64(out) - ref).abs() <= allowed).all())
+    some = torch.empty(4, H, device="cuda", dtype=DT[dtype])
+    ops.rmsnorm(dev(x), dev(w), 1e-6, some, dev(rows))
+    assert torch.equal(some, out[rows.long()])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_rmsnorm_gather_odd_width(ops, dtype):
     g = torch.Generator().manual_seed(3)
     x = torch.randn(11, 100, generator=g) * 3
@@ -564,6 +584,108 @@ def test_linear_bf16_mfma_fed_from_memory(ops, M, N, K, ks):
         assert (f64(sw) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
 
 
+@pytest.mark.parametrize("M,N,K,ks", [(1, 16, 64, 1), (8, 1024, 5120, 3), (16, 50, 2048, 2), (5, 40, 1088, 1), (13, 7, 4160, 5),
+                                      (3, 130, 3072, 2), (16, 260, 8192, 4), (2, 48, 25600, 6)])
+def test_linear_bf16_token_rows_in_pieces(ops, M, N, K, ks):
+    """The kernel for up to 16 rows that takes the token rows through LDS in pieces of 1,024 columns while the
+    next piece's weights are on their way, alone through its test entry point: every epilogue, a K of one
+    piece, of several and of several and a part, columns that do not fill a tile, K split over workgroups
+    (also into more workgroups than some have pieces for), strided rows; against float64.  A row's bits do
+    not depend on the rows beside it, and with K in one workgroup they are the bits of the kernels that take
+    all of K into LDS at once."""
+    import ctypes
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    lib = ops.lib("gemm_bf16")
+    g = torch.Generator().manual_seed(M * 7 + N + K + ks)
+    wide = (torch.rand(M, K + 24, generator=g) * 2 - 1).to(torch.bfloat16)
+    a = dev(wide)[:, 8:8 + K]
+    w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    ref = ref_linear(wide[:, 8:8 + K], w.cpu())
+    tol = 2e-5 * K
+    split_counts = sorted({1, ks, min(ks + 3, -(-K // 1024))})
+    partial = torch.empty(max(split_counts) * M * N, device="cuda")
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def run(rows, out, epi, splits=1):
+        assert splits * rows.shape[0] * out.shape[1] <= partial.numel()
+        rc = lib.ti_gemm_bf16_pieces_any(ptr(rows), ptr(w), ptr(out), rows.shape[0], out.shape[1], K,
+                                         ctypes.c_long(rows.stride(0)), epi, ptr(partial), splits, None)
+        assert rc == 0, lib.ti_last_error()
+    out = torch.full((M + 1, N), 7.0, device="cuda")
+    run(a, out[:M], 0)
+    assert (f64(out[:M]) - ref).abs().max() < tol
+    assert bool((out[M] == 7.0).all())
+    one = torch.empty(1, N, device="cuda")
+    run(a[M - 1:M], one, 0)
+    assert torch.equal(one[0], out[M - 1])
+    # the kernels that hold all of K at once: the same order of summation
+    lib.ti_gemm_bf16_pieces_on(0)
+    lib.ti_gemm_bf16_row_per_wave(0)
+    lib.ti_gemm_bf16_skinny_waves(4)
+    try:
+        old = torch.empty(M, N, device="cuda")
+        rc = lib.ti_gemm_bf16(ptr(a), ptr(w), ptr(old), M, N, K, ctypes.c_long(a.stride(0)), 0, None)
+        assert rc == 0, lib.ti_last_error()
+        assert torch.equal(old, out[:M])
+    finally:
+        lib.ti_gemm_bf16_pieces_on(1)
+        lib.ti_gemm_bf16_row_per_wave(1)
+        lib.ti_gemm_bf16_skinny_waves(0)
+    base = torch.randn(M, N, generator=g)
+    for splits in split_counts:
+        acc = dev(base.clone())
+        run(a, acc, 1, splits)
+        assert (f64(acc) - (ref + f64(base))).abs().max() < tol, splits
+    act = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+    run(a, act, 2)
+    assert (f64(act) - ref).abs().max() < 0.005 * ref.abs().max() + tol
+    if N % 2 == 0:
+        F = N // 2
+        sw = torch.empty(M, F, device="cuda", dtype=torch.bfloat16)
+        run(a, sw, 3)
+        gte, up = ref[:, :F], ref[:, F:]
+        want = gte / (1 + torch.exp(-gte)) * up
+        assert (f64(sw) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
+
+
+@pytest.mark.parametrize("M", [1, 8, 16])
+def test_linear_bf16_long_k_split_for_few_rows(ops, M):
+    """Up to 16 rows added into a residual through a weight with a long K and few rows (the shape of a
+    large model's down projection): K goes to several workgroups; their sums are left to the next norm,
+    or added at once, with the same bits; a row's bits do not depend on the rows beside it."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    N, K = 2064, 17408
+    g = torch.Generator().manual_seed(M)
+    a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    base = torch.randn(M, N, generator=g)
+    ref = ref_linear(a.cpu(), w.cpu()) + f64(base)
+    x = dev(base.clone())
+    ops.linear(a, w, x, "add", may_defer=True)
+    assert ops._pending is not None and ops._pending > 1
+    ops.flush()
+    assert (f64(x) - ref).abs().max() < 2e-5 * K
+    at_once = dev(base.clone())
+    ops.linear(a, w, at_once, "add")
+    assert ops._pending is None
+    assert torch.equal(at_once, x)
+    one = dev(base[M - 1:M].clone())
+    ops.linear(a[M - 1:M], w, one, "add")
+    assert torch.equal(one[0], x[M - 1])
+    # and the norm that reads such a residual adds the sums on its way
+    nw = dev(torch.rand(N, generator=g) + 0.5)
+    y = dev(base.clone())
+    ops.linear(a, w, y, "add", may_defer=True)
+    h = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+    ops.rmsnorm(y, nw, 1e-6, h)
+    assert ops._pending is None and torch.equal(y, x)
+    h2 = torch.empty_like(h)
+    ops.rmsnorm(x, nw, 1e-6, h2)
+    assert torch.equal(h, h2)
+
+
 @pytest.mark.parametrize("M", [17, 33, 64])
 @pytest.mark.parametrize("epilogue", ["store", "add", "store_act", "swiglu"])
 def test_linear_bf16_large_weight_at_17_to_64_rows(ops, M, epilogue):
@@ -612,14 +734,15 @@ def test_linear_bf16_large_weight_at_17_to_64_rows(ops, M, epilogue):
 
 
 def test_linear_bf16_large_weight_at_13_to_16_rows(ops):
-    """13 to 16 rows times a weight of 48 Mi elements: over the rule for these row counts (rows x
-    elements of 600 Mi or more), so the tiled kernels take the product and a norm in front becomes
-    a kernel of its own; 12 rows stay with the kernels that take the norm in.  Against float64,
-    and the rule switched off."""
+    """13 to 16 rows times a weight of 48 Mi elements with a short K (one piece of the kernel that
+    takes the token rows in pieces, which serves a longer K at these row counts): over the rule for
+    these row counts (rows x elements of 600 Mi or more), so the tiled kernels take the product and
+    a norm in front becomes a kernel of its own; 12 rows stay with the kernels that take the norm
+    in.  Against float64, and the rule switched off."""
     if not ops.use_fast_gemm:
         pytest.skip("bfloat16 MFMA kernels are switched off")
     from tinyinfer_amd.ops.kernels import NormedRows
-    N, K = 12288, 4096
+    N, K = 49152, 1024
     g = torch.Generator().manual_seed(3)
     w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
     nw = dev(torch.rand(K, generator=g) + 0.5)
@@ -732,7 +855,8 @@ def test_partial_sums_left_to_the_next_norm(ops, M, N, K):
         ops.use_split_k_add = True
 
 
-@pytest.mark.parametrize("rows,H,KS", [(5, 2304, 3), (3, 1028, 5), (9, 64, 1), (2, 1024, 4), (70, 1536, 2)])
+@pytest.mark.parametrize("rows,H,KS", [(5, 2304, 3), (3, 1028, 5), (9, 64, 1), (2, 1024, 4), (70, 1536, 2),
+                                       (8, 5120, 4), (3, 4100, 2), (2, 8192, 3), (5, 9220, 2), (1, 20480, 1)])
 def test_rmsnorm_that_adds_partial_sums(ops, rows, H, KS):
     """The norm that first adds KS partial sums to its rows, alone, at widths and counts that the
     products of the engine do not produce: the rows afterwards are x + p0 + ... in that order

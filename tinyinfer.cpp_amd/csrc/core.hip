@@ -66,9 +66,11 @@ rmsnorm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w, co
   if (r >= n_rows) return;
   const float* src = x + (size_t)(rows ? rows[r] : r) * H;
   float ss = 0.f;
+#pragma unroll 8
   for (int k = lane * 4; k < H; k += 256) ss = rms_accumulate(ss, *reinterpret_cast<const float4*>(src + k));
   const float scale = rms_scale(ss, H, eps);
   T* dst = out + (size_t)r * H;
+#pragma unroll 4
   for (int k = lane * 4; k < H; k += 256) {
     const float4 v = *reinterpret_cast<const float4*>(src + k);
     const float4 g = *reinterpret_cast<const float4*>(w + k);
@@ -79,11 +81,98 @@ rmsnorm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w, co
   }
 }
 
+// Rows wider than RMS_WIDE_FROM: a workgroup per row, thread t the 16-byte pieces t, t + 256, ...,
+// eight of them asked for at a time (a wavefront per row would walk such a row in twenty round trips
+// to memory).  ADD: x[r] += partial[0][r] + ... + partial[KS - 1][r] first, in that order, written
+// back (see rmsnorm_add_partials_kernel).  The sum of squares: each thread over its pieces in
+// ascending order, then block_sum.  Both with and without ADD: the same bits for the same x.
+#define RMS_WIDE_FROM 4096
+template <typename T, bool ADD>
+__global__ void __launch_bounds__(256)
+rmsnorm_wide_kernel(float* __restrict__ x, const float* __restrict__ partial, int KS, const float* __restrict__ w,
+                    const int* __restrict__ rows, T* __restrict__ out, int n_rows, int H, float eps) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  float* src = x + (size_t)(rows ? rows[r] : r) * H;
+  const size_t count = (size_t)n_rows * H;
+  const float* prow = partial + (size_t)r * H;
+  T* dst = out + (size_t)r * H;
+  float4 v[8];
+  auto fetch = [&](int base) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int k = base + threadIdx.x * 4 + i * 1024;
+      v[i] = *reinterpret_cast<const float4*>(src + (k < H ? k : 0));
+    }
+    if (ADD) {
+      for (int s = 0; s < KS; ++s) {
+        float4 q[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int k = base + threadIdx.x * 4 + i * 1024;
+          q[i] = *reinterpret_cast<const float4*>(prow + s * count + (k < H ? k : 0));
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          v[i].x += q[i].x;
+          v[i].y += q[i].y;
+          v[i].z += q[i].z;
+          v[i].w += q[i].w;
+        }
+      }
+    }
+  };
+  auto scaled = [&](int k, float4 val, float scale) {
+    const float4 g = *reinterpret_cast<const float4*>(w + k);
+    st<T>(dst + k, val.x * scale * g.x);
+    st<T>(dst + k + 1, val.y * scale * g.y);
+    st<T>(dst + k + 2, val.z * scale * g.z);
+    st<T>(dst + k + 3, val.w * scale * g.w);
+  };
+  float ss = 0.f;
+  for (int base = 0; base < H; base += 8192) {
+    fetch(base);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int k = base + threadIdx.x * 4 + i * 1024;
+      if (k < H) {
+        if (ADD) *reinterpret_cast<float4*>(src + k) = v[i];
+        ss = rms_accumulate(ss, v[i]);
+      }
+    }
+  }
+  ss = block_sum<256>(ss, red);
+  const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+  if (H <= 8192) {   // the row is still in registers
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int k = threadIdx.x * 4 + i * 1024;
+      if (k < H) scaled(k, v[i], scale);
+    }
+    return;
+  }
+  for (int base = 0; base < H; base += 8192) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int k = base + threadIdx.x * 4 + i * 1024;
+      if (k < H) scaled(k, *reinterpret_cast<const float4*>(src + k), scale);     // this thread's own store above
+    }
+  }
+}
+
 extern "C" int ti_rmsnorm(int out_dtype, const float* x, const float* w, const int* rows, void* out,
                           int n_rows, int H, float eps, hipStream_t stream) {
   TI_REQUIRE(n_rows >= 0 && H > 0, "rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
   TI_REQUIRE(out_dtype == TI_F32 || out_dtype == TI_BF16, "rmsnorm: unknown dtype %d", out_dtype);
   if (n_rows == 0) return 0;
+  if (H % 4 == 0 && H > RMS_WIDE_FROM && (((uintptr_t)x | (uintptr_t)w) & 15) == 0) {
+    if (out_dtype == TI_F32)
+      rmsnorm_wide_kernel<float, false><<<n_rows, 256, 0, stream>>>((float*)x, nullptr, 0, w, rows, (float*)out, n_rows, H, eps);
+    else
+      rmsnorm_wide_kernel<bf16_t, false><<<n_rows, 256, 0, stream>>>((float*)x, nullptr, 0, w, rows, (bf16_t*)out, n_rows, H, eps);
+    TI_LAUNCH_CHECK();
+    return 0;
+  }
   if (H % 4 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0) {
     const int grid = (n_rows + 3) / 4;
     if (out_dtype == TI_F32)
@@ -175,6 +264,7 @@ rmsnorm_add_partials_kernel(float* __restrict__ x, const float* __restrict__ par
     }
     return;
   }
+#pragma unroll 4
   for (int k = lane * 4; k < H; k += 256) {
     const float4 v = summed(k);
     *reinterpret_cast<float4*>(src + k) = v;
@@ -188,6 +278,10 @@ rmsnorm_add_partials_kernel(float* __restrict__ x, const float* __restrict__ par
 template <typename T>
 static void launch_rmsnorm_add_partials(float* x, const float* partial, int KS, const float* w, T* out, int n_rows,
                                         int H, float eps, hipStream_t stream) {
+  if (H > RMS_WIDE_FROM) {
+    rmsnorm_wide_kernel<T, true><<<n_rows, 256, 0, stream>>>(x, partial, KS, w, nullptr, out, n_rows, H, eps);
+    return;
+  }
   const int grid = (n_rows + 3) / 4;
 #define TI_GO(KS_T, PIECES) \
   rmsnorm_add_partials_kernel<T, KS_T, PIECES><<<grid, 256, 0, stream>>>(x, partial, KS, w, out, n_rows, H, eps)

@@ -16,6 +16,7 @@
 // never depends on M within one kernel.  (The reference's two products are
 // /root/reference/src/cuda/gemm.cu:37-85 and 152-261; it reads the weights once
 // per row of A for M <= 32.)
+#include <algorithm>
 #include "common.h"
 #include "tinyinfer_kernels.h"
 #include "tinyinfer_kernels_tuning.h"
@@ -364,6 +365,162 @@ gemm_skinny_staged_kernel(Producer producer, const bf16_t* __restrict__ W, void*
     if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = sum;
     if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] = prev + sum;
     if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(sum);
+  }
+}
+
+// ================================== few tokens, any K: the token rows in pieces, loads never at rest
+// out (op)= A W^T for M <= 16, K a multiple of 64.  As in the kernels above a workgroup of four
+// wavefronts owns 16 weight rows, wavefront w takes the 64-wide chunks w, w + 4, ... of K, and the
+// four sums meet in LDS in the order 0..3: with one workgroup per 16 rows the bits are those of
+// the kernels above.  Two things differ.
+//  * The token rows go through LDS in pieces of SP_PIECE columns, two buffers in turn: any K fits,
+//    and any M <= 16 leaves room for two workgroups or more on a compute unit.
+//  * While a piece is multiplied, the weights and the token rows of the next one are already on
+//    their way: a wavefront always has 8 to 16 KB of weights in flight, where the kernels above
+//    ask for a batch, wait for all of it, multiply, and only then ask again.  On weights of tens
+//    to hundreds of megabytes that is the difference between ~3.5 and ~5.5 TB/s.
+// grid (ceil(N / 16), KS) (SwiGLU: ceil(F / 8)).  KS > 1 (adding epilogue only): workgroup
+// (., s) takes the pieces s, s + KS, ... and leaves its sums in partial [KS][M][N]; they are
+// added to the residual in the order 0..KS-1 by whoever reads it next.
+#define SP_PIECE 1024              // 16 chunks: four per wavefront, one batch of loads
+#define SP_LD (SP_PIECE + 8)       // LDS row stride in bfloat16
+// AV: 16-byte pieces of the token rows per thread and piece (M <= 2 AV)
+template <int EPI, int AV, bool SPLIT>
+__global__ void __launch_bounds__(256)
+gemm_skinny_pieces_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict__ W, void* __restrict__ out_,
+                          float* __restrict__ partial, int M, int N, int K) {
+  constexpr bool SW = (EPI == TI_EPI_SWIGLU);
+  extern __shared__ __attribute__((aligned(16))) unsigned char dyn_smem[];
+  bf16_t* sA = reinterpret_cast<bf16_t*>(dyn_smem);          // [2][M][SP_LD]
+  __shared__ float red[4][16][17];
+  constexpr int NT = 256;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 15, j = lane >> 4;
+  const int tile = blockIdx.x;               // 16 rows (SwiGLU: 8 gate and 8 up rows)
+  int wrow;
+  if (SW) {
+    const int n = tile * 8 + (r & 7);
+    wrow = (r < 8 ? 0 : N) + (n < N ? n : N - 1);
+  } else {
+    const int n = tile * 16 + r;
+    wrow = n < N ? n : N - 1;
+  }
+  const bf16_t* wp = W + (size_t)wrow * K + j * 16;
+  const int chunks = K / 64;
+  const int n_pieces = (K + SP_PIECE - 1) / SP_PIECE;
+  const int KS = SPLIT ? gridDim.y : 1, split = SPLIT ? blockIdx.y : 0;
+
+  const int tok = threadIdx.x >> 4, row = threadIdx.x & 15;
+  float prev = 0.f;
+  if (EPI == TI_EPI_ADD_F32 && !SPLIT) {   // threads without an output element read a valid one: no branch
+    const int n = tile * 16 + row;
+    prev = ((const float*)out_)[(size_t)(tok < M ? tok : 0) * N + (n < N ? n : N - 1)];
+  }
+
+  // piece p: thread t copies the 16-byte pieces t, t + NT, ... of [M][SP_PIECE / 8]
+  uint4 av[AV];
+  auto ask_rows = [&](int p) {
+#pragma unroll
+    for (int b = 0; b < AV; ++b) {
+      const int v = threadIdx.x + NT * b;
+      const int m = v / (SP_PIECE / 8), k = p * SP_PIECE + (v % (SP_PIECE / 8)) * 8;
+      const bool ok = m < M && k < K;
+      av[b] = ld16(A + (ok ? (size_t)m * lda + k : 0));
+    }
+  };
+  auto keep_rows = [&](int buf) {
+#pragma unroll
+    for (int b = 0; b < AV; ++b) {
+      const int v = threadIdx.x + NT * b;
+      const int m = v / (SP_PIECE / 8);
+      if (m < M) *reinterpret_cast<uint4*>(sA + ((size_t)buf * M + m) * SP_LD + (v % (SP_PIECE / 8)) * 8) = av[b];
+    }
+  };
+  // a chunk beyond the last reads chunk 0 and counts for nothing: no branch between the loads
+  auto ask_weights = [&](int p, Frag (&w0)[4], Frag (&w1)[4]) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = p * (SP_PIECE / 64) + wave + 4 * u;
+      const size_t at = (size_t)(c < chunks ? c : 0) * 64;
+      w0[u].u = ld16(wp + at);
+      w1[u].u = ld16(wp + at + 8);
+    }
+  };
+  floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  auto multiply = [&](int p, int buf, Frag (&w0)[4], Frag (&w1)[4]) {
+    const bf16_t* ap = sA + ((size_t)buf * M + (r < M ? r : 0)) * SP_LD + j * 16;
+    Frag a0[4], a1[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      a0[u].u = *reinterpret_cast<const uint4*>(ap + (wave + 4 * u) * 64);
+      a1[u].u = *reinterpret_cast<const uint4*>(ap + (wave + 4 * u) * 64 + 8);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (p * (SP_PIECE / 64) + wave + 4 * u >= chunks) w0[u].u = w1[u].u = zero;
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u].v, a0[u].v, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, a1[u].v, acc, 0, 0, 0);
+    }
+  };
+  // one turn: piece p is multiplied out of `buf` and (w0, w1) while piece p + KS arrives in the
+  // other buffer and (n0, n1).  Loads return in the order they were asked for: the rows of the
+  // next piece are asked for before its weights, so that keeping them waits for nothing else.
+  auto turn = [&](int p, int buf, Frag (&w0)[4], Frag (&w1)[4], Frag (&n0)[4], Frag (&n1)[4]) {
+    const bool more = p + KS < n_pieces;
+    if (more) {
+      ask_rows(p + KS);
+      __builtin_amdgcn_sched_barrier(0);
+      ask_weights(p + KS, n0, n1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    multiply(p, buf, w0, w1);
+    if (more) keep_rows(buf ^ 1);
+    __syncthreads();
+  };
+  Frag wa0[4], wa1[4], wb0[4], wb1[4];
+  int p = split;
+  if (p < n_pieces) {
+    ask_rows(p);
+    __builtin_amdgcn_sched_barrier(0);
+    ask_weights(p, wa0, wa1);
+    __builtin_amdgcn_sched_barrier(0);
+    keep_rows(0);
+  }
+  __syncthreads();
+  while (p < n_pieces) {
+    turn(p, 0, wa0, wa1, wb0, wb1);
+    p += KS;
+    if (p >= n_pieces) break;
+    turn(p, 1, wb0, wb1, wa0, wa1);
+    p += KS;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) red[wave][r][4 * j + i] = acc[i];
+  __syncthreads();
+  if (tok >= M) return;
+  if (SW) {
+    if (row >= 8) return;
+    const int n = tile * 8 + row;
+    if (n >= N) return;
+    float gt = 0.f, up = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      gt += red[w][tok][row];
+      up += red[w][tok][row + 8];
+    }
+    ((bf16_t*)out_)[(size_t)tok * N + n] = f2bf(silu_mul(gt, up));
+  } else {
+    const int n = tile * 16 + row;
+    if (n >= N) return;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) sum += red[w][tok][row];
+    const size_t o = (size_t)tok * N + n;
+    if (SPLIT) partial[(size_t)split * M * N + o] = sum;
+    else if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = sum;
+    else if (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] = prev + sum;
+    else if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(sum);
   }
 }
 
@@ -1521,6 +1678,56 @@ static void launch_wide_rows(const bf16_t* a, const bf16_t* w, float* out, int M
 #undef TI_GO
 }
 
+template <int EPI, int AV, bool SPLIT>
+static int launch_pieces_av(const bf16_t* a, long lda, const bf16_t* w, void* out, float* partial, int M, int N, int K,
+                            int KS, hipStream_t s) {
+  const size_t lds = (size_t)2 * M * SP_LD * 2;
+  auto kern = gemm_skinny_pieces_kernel<EPI, AV, SPLIT>;
+  static size_t allowed = 48 * 1024;
+  if (lds > allowed) {
+    TI_REQUIRE(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess,
+               "gemm_bf16: LDS size refused");
+    allowed = lds;
+  }
+  const int tile = (EPI == TI_EPI_SWIGLU) ? 8 : 16;
+  kern<<<dim3((N + tile - 1) / tile, KS), 256, lds, s>>>(a, lda, w, out, partial, M, N, K);
+  return 0;
+}
+template <int EPI, bool SPLIT>
+static int launch_pieces(const bf16_t* a, long lda, const bf16_t* w, void* out, float* partial, int M, int N, int K, int KS,
+                         hipStream_t s) {
+  if (M <= 2) return launch_pieces_av<EPI, 1, SPLIT>(a, lda, w, out, partial, M, N, K, KS, s);
+  if (M <= 4) return launch_pieces_av<EPI, 2, SPLIT>(a, lda, w, out, partial, M, N, K, KS, s);
+  if (M <= 8) return launch_pieces_av<EPI, 4, SPLIT>(a, lda, w, out, partial, M, N, K, KS, s);
+  return launch_pieces_av<EPI, 8, SPLIT>(a, lda, w, out, partial, M, N, K, KS, s);
+}
+
+// 1 (default): up to 16 rows times a weight whose K is a multiple of 64 and at least two pieces long
+// take the kernel with the token rows in pieces; 0: the kernels above it (for comparison)
+static int g_pieces = 1;
+extern "C" void ti_gemm_bf16_pieces_on(int on) { g_pieces = on; }
+static bool pieces_serves(int M, int N, int K, int epi) {
+  if (!g_pieces || M > 16 || K % 64 != 0 || K < 2 * SP_PIECE) return false;
+  if (epi < TI_EPI_STORE_F32 || epi > TI_EPI_SWIGLU) return false;
+  // few tokens times a weight of few rows: a row per wavefront wins (and fills the compute units)
+  if (row_per_wave_serves(M, N, K, epi)) return false;
+  // where the kernels with the norm in front take eight wavefronts, this one would give other bits
+  const int grid = (epi == TI_EPI_SWIGLU) ? (N + 7) / 8 : (N + 15) / 16;
+  return skinny_waves_for(grid, K) == 4;
+}
+// Into how many workgroups the pieces of K go when the product adds into the residual: a long K under
+// few rows of weight leaves a launch of few workgroups that each walk a long way (Qwen3-32B's down
+// projection: 320 workgroups, 25 pieces each, 3.1 TB/s; split four ways 4.8 TB/s).  By the weight's
+// shape alone, so that a row's bits do not depend on the rows beside it.
+static int pieces_splits(int N, int K, long partial_bytes) {
+  const int n_pieces = (K + SP_PIECE - 1) / SP_PIECE;
+  if (n_pieces < 16) return 1;
+  const int grid = (N + 15) / 16;
+  int ks = std::min(n_pieces / 4, (4 * compute_units() + grid - 1) / grid);
+  while (ks > 1 && (long)ks * 16 * N * 4 > partial_bytes) --ks;
+  return ks < 1 ? 1 : ks;
+}
+
 static int g_add_split = 1;        // a hook for measurements: 0: ti_gemm_bf16_add_split serves nothing
 extern "C" void ti_gemm_bf16_add_split_on(int on) { g_add_split = on; }
 
@@ -1552,6 +1759,7 @@ extern "C" int ti_gemm_bf16_partials_add(float* out, const float* partial, int K
 // gemm_mblocks_kernel (measured against the kernels without MFMA at 64 rows: 1024 x 3072 19.7 ->
 // 9.7 us with the addition of the partial sums as a kernel of its own, ~6 us without).  More rows:
 // the pipelined kernel with 64 x 64 tiles, storing (136 rows: 18.5 -> ~8 us).
+// Up to 16 rows: the kernel with the token rows in pieces, where pieces_splits says so.
 // defer = 0: the partial sums are added to `out` here, and only what gains even so is served.
 // defer = 1: they are left in `partial`, *splits gets their number, and the caller sees to the
 // addition (ti_gemm_bf16_partials_add, or a kernel that reads the residual next and adds them on
@@ -1562,6 +1770,24 @@ extern "C" int ti_gemm_bf16_add_split(const void* A, const void* W, void* out, i
   TI_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K, "gemm_bf16_add_split: bad sizes M=%d N=%d K=%d lda=%ld", M, N, K, lda);
   TI_REQUIRE(splits != nullptr, "gemm_bf16_add_split: splits must point to an int");
   *splits = 0;
+  if (M <= 16 && M > 0 && g_add_split && epi == TI_EPI_ADD_F32 && partial && lda % 8 == 0 && !((uintptr_t)A & 15) &&
+      !((uintptr_t)W & 15) && !((uintptr_t)partial & 15) && pieces_serves(M, N, K, epi)) {
+    const int ks = pieces_splits(N, K, partial_bytes);
+    if (ks > 1) {
+      int rc_ = launch_pieces<TI_EPI_ADD_F32, true>((const bf16_t*)A, lda, (const bf16_t*)W, out, (float*)partial, M, N, K, ks,
+                                                    stream);
+      if (rc_) return rc_;
+      if (defer == 1) {
+        *splits = ks;
+      } else {
+        const size_t count = (size_t)M * N;
+        gemm_partials_add_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>((float*)out, (const float*)partial,
+                                                                                    ks, count);
+      }
+      TI_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   int KS = 1;
   const bool small = M <= 64 && !(large_weight(M, N, K, epi) && g_use_pipelined);
   if (g_add_split && epi == TI_EPI_ADD_F32 && partial && M > 16 && K % 64 == 0 && lda % 8 == 0 &&
@@ -1569,7 +1795,7 @@ extern "C" int ti_gemm_bf16_add_split(const void* A, const void* W, void* out, i
     // split K until the launch has about a workgroup per compute unit
     const long tiles = small ? (N + 15) / 16 : (long)((M + 63) / 64) * ((N + 63) / 64);
     const int nb = K / 64;
-    while (KS < 8 && tiles * KS * 2 <= 256 && nb / (KS * 2) >= 4) KS *= 2;
+    while (KS < 8 && tiles * KS * 2 <= compute_units() && nb / (KS * 2) >= 4) KS *= 2;
     if ((long)KS * M * N * 4 > partial_bytes) KS = 1;
     // with the addition as a kernel of its own, only large products gain
     if (!defer && small && !((long)M * K >= 128 * 1024 || (K >= 3072 && (long)M * K >= 96 * 1024))) KS = 1;
@@ -1593,6 +1819,39 @@ extern "C" int ti_gemm_bf16_add_split(const void* A, const void* W, void* out, i
     gemm_partials_add_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>((float*)out, (const float*)partial,
                                                                                 KS, count);
   }
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// the kernel with the token rows in pieces alone, for tests and measurements: any epilogue, 1..16
+// rows, K a multiple of 64 split ks ways (1: not split; partial sums are added here)
+extern "C" int ti_gemm_bf16_pieces_any(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
+                                       void* partial, int ks, hipStream_t stream) {
+  TI_REQUIRE(M > 0 && M <= 16 && N > 0 && K > 0 && K % 64 == 0 && lda >= K && lda % 8 == 0 && ks >= 1 &&
+                 ks <= (K + SP_PIECE - 1) / SP_PIECE,
+             "gemm_bf16_pieces_any: bad sizes M=%d N=%d K=%d lda=%ld ks=%d", M, N, K, lda, ks);
+  TI_REQUIRE(ks == 1 || (epi == TI_EPI_ADD_F32 && partial), "gemm_bf16_pieces_any: a split K needs the adding epilogue");
+  const bf16_t* a = (const bf16_t*)A;
+  const bf16_t* w = (const bf16_t*)W;
+  int rc = 0;
+  switch (epi) {
+    case TI_EPI_STORE_F32: rc = launch_pieces<TI_EPI_STORE_F32, false>(a, lda, w, out, nullptr, M, N, K, 1, stream); break;
+    case TI_EPI_STORE_ACT: rc = launch_pieces<TI_EPI_STORE_ACT, false>(a, lda, w, out, nullptr, M, N, K, 1, stream); break;
+    case TI_EPI_SWIGLU: rc = launch_pieces<TI_EPI_SWIGLU, false>(a, lda, w, out, nullptr, M, N, K, 1, stream); break;
+    case TI_EPI_ADD_F32:
+      if (ks == 1) {
+        rc = launch_pieces<TI_EPI_ADD_F32, false>(a, lda, w, out, nullptr, M, N, K, 1, stream);
+      } else {
+        rc = launch_pieces<TI_EPI_ADD_F32, true>(a, lda, w, out, (float*)partial, M, N, K, ks, stream);
+        const size_t count = (size_t)M * N;
+        gemm_partials_add_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>((float*)out, (const float*)partial,
+                                                                                    ks, count);
+      }
+      break;
+    default:
+      TI_REQUIRE(false, "gemm_bf16_pieces_any: unknown epilogue %d", epi);
+  }
+  if (rc) return rc;
   TI_LAUNCH_CHECK();
   return 0;
 }
@@ -1645,6 +1904,18 @@ extern "C" int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int 
   const bf16_t* w = (const bf16_t*)W;
   const bool skinny = M <= 64 && !(large_weight(M, N, K, epi) && g_use_pipelined);
   const bool copied = g_skinny_copy && M <= 16 && K % 64 == 0 && K <= 4096 && skinny;
+  if (pieces_serves(M, N, K, epi)) {
+    int rc_ = 0;
+    switch (epi) {
+      case TI_EPI_STORE_F32: rc_ = launch_pieces<TI_EPI_STORE_F32, false>(a, lda, w, out, nullptr, M, N, K, 1, stream); break;
+      case TI_EPI_ADD_F32: rc_ = launch_pieces<TI_EPI_ADD_F32, false>(a, lda, w, out, nullptr, M, N, K, 1, stream); break;
+      case TI_EPI_STORE_ACT: rc_ = launch_pieces<TI_EPI_STORE_ACT, false>(a, lda, w, out, nullptr, M, N, K, 1, stream); break;
+      default: rc_ = launch_pieces<TI_EPI_SWIGLU, false>(a, lda, w, out, nullptr, M, N, K, 1, stream); break;
+    }
+    if (rc_) return rc_;
+    TI_LAUNCH_CHECK();
+    return 0;
+  }
   if (wide_rows_serves(M, N, K, epi)) {
     launch_wide_rows(a, w, (float*)out, M, N, K, lda, stream);
     TI_LAUNCH_CHECK();

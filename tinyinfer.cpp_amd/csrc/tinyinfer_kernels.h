@@ -67,6 +67,10 @@ int ti_gemm_bf16_partials_add(float* out, const float* partial, int KS, long cou
 // the kernel of ti_gemm_bf16_add_split alone, for tests: any epilogue, 1..64 rows, K split ks ways
 int ti_gemm_bf16_mblocks_any(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
                              void* partial, int ks, hipStream_t stream);
+// the kernel for up to 16 rows that takes the token rows through LDS in pieces, alone, for tests: any
+// epilogue, K a multiple of 64 split ks ways (adding epilogue only; partial f32 [ks][M][N])
+int ti_gemm_bf16_pieces_any(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
+                            void* partial, int ks, hipStream_t stream);
 // out (op)= rmsnorm(x; nw, eps) W^T for M <= 16, K a multiple of 64
 int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, const void* W, void* out, int M, int N, int K, int epi,
                         hipStream_t stream);

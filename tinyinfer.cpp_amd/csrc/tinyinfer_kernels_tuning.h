@@ -15,6 +15,7 @@ void ti_gemm_bf16_add_split_on(int on);         // 0: ti_gemm_bf16_add_split ser
 void ti_gemm_bf16_use_pipelined(int on);      // 0: the plain tiled kernel for every K
 void ti_gemm_bf16_row_per_wave(int on);        // 0: few tokens and a weight of few rows take the 16-row kernels too
 void ti_gemm_bf16_skinny_copy(int on);        // 0: up to 16 tokens, fragments of the token rows straight from memory
+void ti_gemm_bf16_pieces_on(int on);          // 0: up to 16 rows never take the kernel with the token rows in pieces
 void ti_gemm_bf16_skinny_deep(int on);        // 0: four chunks of K in flight per wavefront also for a long K
 void ti_attention_decode_shared_query(int on);   // 0: every wavefront of a decode workgroup prepares the query itself
 void ti_attention_prefill_groups(int groups);  // 1 or 2 groups of wavefronts per workgroup, 0: by the launch

@@ -533,7 +533,7 @@ void Ops::linear(const Tensor& a, const Tensor& w, const Tensor& out, Epilogue e
   const long lda = (long)a.stride[0];
   if (a.dtype == DType::BF16 && use.fast_gemm && kernel_library_available("gemm_bf16") && K % 8 == 0 && lda % 8 == 0 &&
       ((uintptr_t)a.data % 16) == 0 && ((uintptr_t)w.data % 16) == 0) {
-    if (M > 16 && epi == Add && use.split_k_add) {
+    if (epi == Add && use.split_k_add) {
       // a product of few tiles: K split over workgroups; their sums go through a workspace
       void* stream = launch_stream();
       if (!partials_.data()) partials_ = DeviceBuffer(PARTIALS_BYTES);
