@@ -1363,6 +1363,8 @@ static int skinny_waves_for(int grid, int K) {
   return g_skinny_waves ? g_skinny_waves : ((grid <= 128 && K >= 1024) ? 8 : 4);
 }
 
+static bool pieces_serves(int M, int N, int K, int epi);
+#define NORMED_WEIGHT_BELOW (64L << 20)   // weight elements from which the norm stays a kernel of its own
 // out = rmsnorm(x; nw, eps) W^T for M <= 16 (see gemm_skinny_staged_kernel).  Returns 3 for
 // sizes it does not serve (M > 16, K not a multiple of 64 or above 4096).
 extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, const void* W, void* out,
@@ -1380,6 +1382,13 @@ extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, c
   }
   if (large_weight(M, N, K, epi) && g_use_pipelined) {
     ti_set_error("gemm_bf16_normed: M=%d times a weight of %d x %d is left to the tiled kernels", M, N, K);
+    return 3;
+  }
+  // Every workgroup here norms all M rows for itself, which pulls as many bytes through the caches as
+  // its share of the weight has.  Under a large weight the kernel that keeps loads in flight gains more
+  // than the norm's own launch costs (Qwen3-8B's gate/up at 8 rows: 46 us here, 38 + 5 us there).
+  if ((long)(epi == TI_EPI_SWIGLU ? 2 : 1) * N * K >= NORMED_WEIGHT_BELOW && pieces_serves(M, N, K, epi)) {
+    ti_set_error("gemm_bf16_normed: a weight of %d x %d is left to the norm's kernel and the product's", N, K);
     return 3;
   }
   if (M == 0) return 0;

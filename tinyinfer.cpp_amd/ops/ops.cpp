@@ -489,6 +489,8 @@ bool Ops::linear_with_norm(const Rows& a, const Tensor& w, const Tensor& out, Ep
   TIMED(std::string("norm+linear.") + EPI_NAMES[epi] + " " + dims(a.t) + " * " + dims(w));
   const int64_t M = a.t.shape[0], K = a.t.shape[1];
   if (!can_fuse_norm(M, a.t.dtype) || w.dtype != DType::BF16) return false;
+  // the rows wait for partial sums: the norm's own kernel adds them on its way
+  if (pending_.out && pending_.out == a.x.data) return false;
   const int64_t rows = w.shape[0];
   const int64_t N = epi == SwiGLU ? rows / 2 : rows;
   require(w.ndim == 2 && w.shape[1] == K && w.contiguous() && !(epi == SwiGLU && rows % 2),
