@@ -197,7 +197,7 @@ extern "C" int ti_rmsnorm(int out_dtype, const float* x, const float* w, const i
 // rmsnorm_wave_kernel over the new x.  A wavefront per row, four rows a workgroup.
 // KS_T: the number of partial sums if known when compiled (their loads then do not wait for one
 // another), 0: KS.  PIECES: 16-byte pieces of a row a lane keeps in registers between the sum and
-// the scaling (rows up to 1024 PIECES wide), 0: it reads them again.
+// the scaling (rows up to 256 PIECES floats wide; wider rows take the kernels below).
 template <typename T, int KS_T, int PIECES>
 __global__ void __launch_bounds__(256)
 rmsnorm_add_partials_kernel(float* __restrict__ x, const float* __restrict__ partial, int KS,
@@ -208,27 +208,17 @@ rmsnorm_add_partials_kernel(float* __restrict__ x, const float* __restrict__ par
   const size_t count = (size_t)n_rows * H;
   const float* prow = partial + (size_t)r * H;
   if (KS_T) KS = KS_T;
-  auto summed = [&](int k) {
+  auto summed = [&](int k) {   // KS_T partial sums, all asked for at once
     float4 v = *reinterpret_cast<const float4*>(src + k);
-    if (KS_T) {
-      float4 p[KS_T ? KS_T : 1];
+    float4 p[KS_T ? KS_T : 1];
 #pragma unroll
-      for (int s = 0; s < KS_T; ++s) p[s] = *reinterpret_cast<const float4*>(prow + s * count + k);
+    for (int s = 0; s < KS_T; ++s) p[s] = *reinterpret_cast<const float4*>(prow + s * count + k);
 #pragma unroll
-      for (int s = 0; s < KS_T; ++s) {
-        v.x += p[s].x;
-        v.y += p[s].y;
-        v.z += p[s].z;
-        v.w += p[s].w;
-      }
-    } else {
-      for (int s = 0; s < KS; ++s) {
-        const float4 p = *reinterpret_cast<const float4*>(prow + s * count + k);
-        v.x += p.x;
-        v.y += p.y;
-        v.z += p.z;
-        v.w += p.w;
-      }
+    for (int s = 0; s < KS_T; ++s) {
+      v.x += p[s].x;
+      v.y += p[s].y;
+      v.z += p[s].z;
+      v.w += p[s].w;
     }
     return v;
   };
@@ -241,12 +231,37 @@ rmsnorm_add_partials_kernel(float* __restrict__ x, const float* __restrict__ par
     st<T>(dst + k + 3, v.w * scale * g.w);
   };
   float ss = 0.f;
-  if (PIECES) {
-    float4 v[PIECES ? PIECES : 1];
+  {
+    float4 v[PIECES];
+    if (KS_T) {
 #pragma unroll
-    for (int i = 0; i < PIECES; ++i) {
-      const int k = lane * 4 + i * 256;
-      if (k < H) v[i] = summed(k);
+      for (int i = 0; i < PIECES; ++i) {
+        const int k = lane * 4 + i * 256;
+        if (k < H) v[i] = summed(k);
+      }
+    } else {
+      // the row, then one partial sum after the other, each asked for as a whole: 1 + KS round trips
+      // to memory, not one per piece
+#pragma unroll
+      for (int i = 0; i < PIECES; ++i) {
+        const int k = lane * 4 + i * 256;
+        v[i] = *reinterpret_cast<const float4*>(src + (k < H ? k : 0));
+      }
+      for (int s = 0; s < KS; ++s) {
+        float4 q[PIECES];
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+          const int k = lane * 4 + i * 256;
+          q[i] = *reinterpret_cast<const float4*>(prow + s * count + (k < H ? k : 0));
+        }
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+          v[i].x += q[i].x;
+          v[i].y += q[i].y;
+          v[i].z += q[i].z;
+          v[i].w += q[i].w;
+        }
+      }
     }
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
@@ -262,17 +277,80 @@ rmsnorm_add_partials_kernel(float* __restrict__ x, const float* __restrict__ par
       const int k = lane * 4 + i * 256;
       if (k < H) scaled(k, v[i], scale);
     }
-    return;
   }
-#pragma unroll 4
-  for (int k = lane * 4; k < H; k += 256) {
-    const float4 v = summed(k);
-    *reinterpret_cast<float4*>(src + k) = v;
-    ss = rms_accumulate(ss, v);
+}
+
+// The same for rows of 1,025 to 4,096 floats: a workgroup per row, so that four times as many loads
+// are on their way as with a wavefront per row (64 rows of 4,096 with 8 partial sums: 26 -> ~7 us).
+// Thread t adds up the 16-byte pieces t, t + 256, ... (the partial sums four at a time), writes them
+// back and leaves them in LDS; wavefront 0 takes the sum of squares from there in the order of
+// rmsnorm_wave_kernel (lane l the pieces l, l + 64, ...), so the bits are that kernel's.
+template <typename T>
+__global__ void __launch_bounds__(256)
+rmsnorm_add_partials_row_kernel(float* __restrict__ x, const float* __restrict__ partial, int KS,
+                                const float* __restrict__ w, T* __restrict__ out, int n_rows, int H, float eps) {
+  __shared__ __attribute__((aligned(16))) float row[4096];
+  __shared__ float s_scale;
+  const int r = blockIdx.x, lane = threadIdx.x & 63;
+  float* src = x + (size_t)r * H;
+  const size_t count = (size_t)n_rows * H;
+  const float* prow = partial + (size_t)r * H;
+  float4 v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int k = threadIdx.x * 4 + i * 1024;
+    v[i] = *reinterpret_cast<const float4*>(src + (k < H ? k : 0));
   }
-  const float scale = rms_scale(ss, H, eps);
-  for (int k = lane * 4; k < H; k += 256)
-    scaled(k, *reinterpret_cast<const float4*>(src + k), scale);     // this lane's own store above
+  for (int s0 = 0; s0 < KS; s0 += 4) {
+    float4 q[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int k = threadIdx.x * 4 + i * 1024;
+        q[j][i] = *reinterpret_cast<const float4*>(prow + (size_t)(s0 + j < KS ? s0 + j : s0) * count + (k < H ? k : 0));
+      }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (s0 + j < KS) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[i].x += q[j][i].x;
+          v[i].y += q[j][i].y;
+          v[i].z += q[j][i].z;
+          v[i].w += q[j][i].w;
+        }
+      }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int k = threadIdx.x * 4 + i * 1024;
+    if (k < H) {
+      *reinterpret_cast<float4*>(src + k) = v[i];
+      *reinterpret_cast<float4*>(row + k) = v[i];
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    float ss = 0.f;
+    for (int k = lane * 4; k < H; k += 256) ss = rms_accumulate(ss, *reinterpret_cast<const float4*>(row + k));
+    const float scale = rms_scale(ss, H, eps);
+    if (lane == 0) s_scale = scale;
+  }
+  __syncthreads();
+  const float scale = s_scale;
+  T* dst = out + (size_t)r * H;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int k = threadIdx.x * 4 + i * 1024;
+    if (k < H) {
+      const float4 g = *reinterpret_cast<const float4*>(w + k);
+      st<T>(dst + k, v[i].x * scale * g.x);
+      st<T>(dst + k + 1, v[i].y * scale * g.y);
+      st<T>(dst + k + 2, v[i].z * scale * g.z);
+      st<T>(dst + k + 3, v[i].w * scale * g.w);
+    }
+  }
 }
 
 template <typename T>
@@ -288,8 +366,8 @@ static void launch_rmsnorm_add_partials(float* x, const float* partial, int KS, 
   if (H <= 1024 && KS == 4) TI_GO(4, 4);
   else if (H <= 1024 && KS == 2) TI_GO(2, 4);
   else if (H <= 1024 && KS == 8) TI_GO(8, 4);
-  else if (H <= 2048) TI_GO(0, 8);
-  else TI_GO(0, 0);
+  else if (H <= 1024) TI_GO(0, 4);
+  else rmsnorm_add_partials_row_kernel<T><<<n_rows, 256, 0, stream>>>(x, partial, KS, w, out, n_rows, H, eps);
 #undef TI_GO
 }
 

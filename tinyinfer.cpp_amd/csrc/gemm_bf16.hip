@@ -1804,8 +1804,14 @@ extern "C" int ti_gemm_bf16_add_split(const void* A, const void* W, void* out, i
     // split K until the launch has about a workgroup per compute unit
     const long tiles = small ? (N + 15) / 16 : (long)((M + 63) / 64) * ((N + 63) / 64);
     const int nb = K / 64;
+    // (a large weight is waited for from memory: then about four workgroups per unit, so that enough
+    // of it is on its way at any time)
+    // as long as the partial sums stay a small part of what the weight has in bytes
+    const bool streamed = !small && (long)N * K >= (8L << 20);
     while (KS < 8 && tiles * KS * 2 <= compute_units() && nb / (KS * 2) >= 4) KS *= 2;
-    if ((long)KS * M * N * 4 > partial_bytes) KS = 1;
+    if (streamed)
+      while (KS < 8 && tiles * KS * 2 <= 4L * compute_units() && nb / (KS * 2) >= 4 && (long)KS * 2 * M * 16 <= K) KS *= 2;
+    while (KS > 1 && (long)KS * M * N * 4 > partial_bytes) KS /= 2;
     // with the addition as a kernel of its own, only large products gain
     if (!defer && small && !((long)M * K >= 128 * 1024 || (K >= 3072 && (long)M * K >= 96 * 1024))) KS = 1;
     if (!defer && !small && KS < 4) KS = 1;

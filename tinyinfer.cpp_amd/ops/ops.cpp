@@ -265,7 +265,7 @@ bool kernel_library_available(const std::string& name) {
 }
 
 // ---------------------------------------------------------------------------------------- Ops
-static const int64_t PARTIALS_BYTES = 4 << 20;
+static const int64_t PARTIALS_BYTES = 32 << 20;
 static const int NORMED_MAX_ROWS = 16;
 
 struct Ops::Timing {
