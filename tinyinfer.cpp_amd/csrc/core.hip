@@ -81,44 +81,53 @@ rmsnorm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w, co
   }
 }
 
-// Rows wider than RMS_WIDE_FROM: a workgroup per row, thread t the 16-byte pieces t, t + 256, ...,
-// eight of them asked for at a time (a wavefront per row would walk such a row in twenty round trips
-// to memory).  ADD: x[r] += partial[0][r] + ... + partial[KS - 1][r] first, in that order, written
-// back (see rmsnorm_add_partials_kernel).  The sum of squares: each thread over its pieces in
-// ascending order, then block_sum.  Both with and without ADD: the same bits for the same x.
+// Rows wider than RMS_WIDE_FROM: a workgroup of 1,024 threads per row, thread t the 16-byte pieces
+// t, t + 1024, ... (a wavefront per row would walk such a row in twenty round trips to memory).
+// ADD: x[r] += partial[0][r] + ... + partial[KS - 1][r] first, in that order, written back (see
+// rmsnorm_add_partials_kernel); the partial sums are asked for four at a time.  The sum of squares:
+// each thread over its pieces in ascending order, then block_sum.  With and without ADD: the same
+// bits for the same x.
 #define RMS_WIDE_FROM 4096
+#define RMS_WIDE_THREADS 1024
 template <typename T, bool ADD>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(RMS_WIDE_THREADS)
 rmsnorm_wide_kernel(float* __restrict__ x, const float* __restrict__ partial, int KS, const float* __restrict__ w,
                     const int* __restrict__ rows, T* __restrict__ out, int n_rows, int H, float eps) {
-  __shared__ float red[4];
+  constexpr int NT = RMS_WIDE_THREADS, PER = 2, SPAN = NT * 4 * PER;   // floats a pass covers
+  __shared__ float red[NT / 64];
   const int r = blockIdx.x;
   float* src = x + (size_t)(rows ? rows[r] : r) * H;
   const size_t count = (size_t)n_rows * H;
   const float* prow = partial + (size_t)r * H;
   T* dst = out + (size_t)r * H;
-  float4 v[8];
+  float4 v[PER];
   auto fetch = [&](int base) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int k = base + threadIdx.x * 4 + i * 1024;
+    for (int i = 0; i < PER; ++i) {
+      const int k = base + threadIdx.x * 4 + i * NT * 4;
       v[i] = *reinterpret_cast<const float4*>(src + (k < H ? k : 0));
     }
     if (ADD) {
-      for (int s = 0; s < KS; ++s) {
-        float4 q[8];
+      for (int s0 = 0; s0 < KS; s0 += 4) {
+        float4 q[4][PER];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int k = base + threadIdx.x * 4 + i * 1024;
-          q[i] = *reinterpret_cast<const float4*>(prow + s * count + (k < H ? k : 0));
-        }
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          v[i].x += q[i].x;
-          v[i].y += q[i].y;
-          v[i].z += q[i].z;
-          v[i].w += q[i].w;
-        }
+          for (int i = 0; i < PER; ++i) {
+            const int k = base + threadIdx.x * 4 + i * NT * 4;
+            q[j][i] = *reinterpret_cast<const float4*>(prow + (size_t)(s0 + j < KS ? s0 + j : s0) * count + (k < H ? k : 0));
+          }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (s0 + j < KS) {
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+              v[i].x += q[j][i].x;
+              v[i].y += q[j][i].y;
+              v[i].z += q[j][i].z;
+              v[i].w += q[j][i].w;
+            }
+          }
       }
     }
   };
@@ -130,31 +139,31 @@ rmsnorm_wide_kernel(float* __restrict__ x, const float* __restrict__ partial, in
     st<T>(dst + k + 3, val.w * scale * g.w);
   };
   float ss = 0.f;
-  for (int base = 0; base < H; base += 8192) {
+  for (int base = 0; base < H; base += SPAN) {
     fetch(base);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int k = base + threadIdx.x * 4 + i * 1024;
+    for (int i = 0; i < PER; ++i) {
+      const int k = base + threadIdx.x * 4 + i * NT * 4;
       if (k < H) {
         if (ADD) *reinterpret_cast<float4*>(src + k) = v[i];
         ss = rms_accumulate(ss, v[i]);
       }
     }
   }
-  ss = block_sum<256>(ss, red);
+  ss = block_sum<NT>(ss, red);
   const float scale = 1.0f / sqrtf(ss / (float)H + eps);
-  if (H <= 8192) {   // the row is still in registers
+  if (H <= SPAN) {   // the row is still in registers
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int k = threadIdx.x * 4 + i * 1024;
+    for (int i = 0; i < PER; ++i) {
+      const int k = threadIdx.x * 4 + i * NT * 4;
       if (k < H) scaled(k, v[i], scale);
     }
     return;
   }
-  for (int base = 0; base < H; base += 8192) {
+  for (int base = 0; base < H; base += SPAN) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int k = base + threadIdx.x * 4 + i * 1024;
+    for (int i = 0; i < PER; ++i) {
+      const int k = base + threadIdx.x * 4 + i * NT * 4;
       if (k < H) scaled(k, *reinterpret_cast<const float4*>(src + k), scale);     // this thread's own store above
     }
   }
@@ -167,9 +176,9 @@ extern "C" int ti_rmsnorm(int out_dtype, const float* x, const float* w, const i
   if (n_rows == 0) return 0;
   if (H % 4 == 0 && H > RMS_WIDE_FROM && (((uintptr_t)x | (uintptr_t)w) & 15) == 0) {
     if (out_dtype == TI_F32)
-      rmsnorm_wide_kernel<float, false><<<n_rows, 256, 0, stream>>>((float*)x, nullptr, 0, w, rows, (float*)out, n_rows, H, eps);
+      rmsnorm_wide_kernel<float, false><<<n_rows, RMS_WIDE_THREADS, 0, stream>>>((float*)x, nullptr, 0, w, rows, (float*)out, n_rows, H, eps);
     else
-      rmsnorm_wide_kernel<bf16_t, false><<<n_rows, 256, 0, stream>>>((float*)x, nullptr, 0, w, rows, (bf16_t*)out, n_rows, H, eps);
+      rmsnorm_wide_kernel<bf16_t, false><<<n_rows, RMS_WIDE_THREADS, 0, stream>>>((float*)x, nullptr, 0, w, rows, (bf16_t*)out, n_rows, H, eps);
     TI_LAUNCH_CHECK();
     return 0;
   }
@@ -357,7 +366,7 @@ template <typename T>
 static void launch_rmsnorm_add_partials(float* x, const float* partial, int KS, const float* w, T* out, int n_rows,
                                         int H, float eps, hipStream_t stream) {
   if (H > RMS_WIDE_FROM) {
-    rmsnorm_wide_kernel<T, true><<<n_rows, 256, 0, stream>>>(x, partial, KS, w, nullptr, out, n_rows, H, eps);
+    rmsnorm_wide_kernel<T, true><<<n_rows, RMS_WIDE_THREADS, 0, stream>>>(x, partial, KS, w, nullptr, out, n_rows, H, eps);
     return;
   }
   const int grid = (n_rows + 3) / 4;
