@@ -801,10 +801,11 @@ def test_linear_bf16_wide_weight_at_17_to_64_rows(ops, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(17, 1024, 2048), (64, 1024, 3072), (40, 512, 1024), (33, 96, 1024),
                                    (20, 2048, 1024), (24, 256, 2048), (136, 1024, 2048), (300, 1000, 3072),
-                                   (65, 520, 1024), (512, 1024, 2048)])
+                                   (65, 520, 1024), (512, 1024, 2048), (2048, 1024, 2048), (1100, 1030, 3072)])
 def test_partial_sums_left_to_the_next_norm(ops, M, N, K):
     """A product into the residual whose launch would have few tiles (17..64 rows and few columns:
-    MFMAs fed from memory; up to ~512 rows: 64 x 64 tiles) splits K over workgroups.
+    MFMAs fed from memory; up to ~512 rows: 64 x 64 tiles; a whole prompt times a weight of ~1,024
+    rows: 128 x 128 tiles, each shared by two to four workgroups) splits K over workgroups.
     With `may_defer` its partial sums wait for whatever reads the residual next: the norm adds
     them on its way, any other launch (or `flush`) adds them with a kernel of their own.  All
     three give the bits of the product that adds them at once, and match float64."""

@@ -1816,6 +1816,30 @@ extern "C" int ti_gemm_bf16_add_split(const void* A, const void* W, void* out, i
     if (!defer && small && !((long)M * K >= 128 * 1024 || (K >= 3072 && (long)M * K >= 96 * 1024))) KS = 1;
     if (!defer && !small && KS < 4) KS = 1;
   }
+  // Many rows times a weight of few rows (o and down of a whole prompt): 64 x 64 tiles are what fills
+  // the chip, and they pull four bytes into a compute unit where a 128 x 128 tile pulls two.  When the
+  // 128 x 128 tiles are at most half as many as the units, K is split between two to four workgroups
+  // per tile instead: the same bytes as one round of 128 x 128 tiles, on all units.
+  if (KS == 1 && !small && g_add_split && g_use_pipelined && defer && epi == TI_EPI_ADD_F32 && partial && M >= 256 &&
+      K % 64 == 0 && lda % 8 == 0 && !((uintptr_t)A & 15) && !((uintptr_t)W & 15) && !((uintptr_t)partial & 15)) {
+    const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    int ks = (int)std::min<long>(4, compute_units() / std::max<long>(1, tiles128));
+    while (ks > 1 && ((K / 64) / ks < 8 || (long)ks * M * N * 4 > partial_bytes)) --ks;
+    if (ks >= 2) {
+      int rc_ = launch_pipelined<128, 128, 2, 4, TI_EPI_STORE_F32>((const bf16_t*)A, (const bf16_t*)W, partial, M, N, K, lda,
+                                                                   stream, ks);
+      if (rc_) return rc_;
+      if (defer == 1) {
+        *splits = ks;
+      } else {
+        const size_t count = (size_t)M * N;
+        gemm_partials_add_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>((float*)out, (const float*)partial,
+                                                                                    ks, count);
+      }
+      TI_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   if (KS == 1) {
     ti_set_error("gemm_bf16_add_split: serves more than 16 rows added into a product of few tiles, K a multiple of 64");
     return 3;
