@@ -1192,6 +1192,15 @@ extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K,
   // 128-row tiles while they make no more workgroups than there are compute units (1,024 rows of
   // the 32 column tiles of Qwen3-0.6B), else 256-row tiles, which load less per flop
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+  // Few tiles (a short portion beside decoded tokens): a launch of tiles whose columns are whole heads
+  // leaves most compute units idle, and each workgroup that does run finishes 128 rows of heads by
+  // itself; the product in 64 x 64 tiles followed by the kernel that prepares whole steps is faster
+  // then (8 decoded tokens beside 128 of a prompt, Qwen3-0.6B's sizes: 2.47 -> 2.29 ms a step; from
+  // 512 rows on this kernel wins).  Not when a test asks for a tile.
+  if (!g_qkv_rows && tiles128 * 2 < compute_units()) {
+    ti_set_error("gemm_bf16_qkv_prep: %ld tiles of 128 x 128 are left to the product and the preparation kernel", tiles128);
+    return 3;
+  }
   const bool rows128 = g_qkv_rows ? g_qkv_rows == 128 : tiles128 <= compute_units();
   int rc_ = rows128 ? launch_qkv_prep<128, 2, 4>(A, W, M, N, K, lda, ep, stream)
                     : launch_qkv_prep<256, 4, 2>(A, W, M, N, K, lda, ep, stream);
