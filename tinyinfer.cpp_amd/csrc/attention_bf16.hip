@@ -22,6 +22,7 @@
 //            together and share them in the cache.
 // (The reference scans positions with 16-lane groups and FMA for both cases:
 // /root/reference/src/cuda/attention.cu:107-198.)
+#include <type_traits>
 #include "common.h"
 #include "tinyinfer_kernels.h"
 #include "tinyinfer_kernels_tuning.h"
@@ -553,30 +554,38 @@ attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ pa
   const float2* pm = reinterpret_cast<const float2*>(part_ml) + ((size_t)ridx * n_head + head) * n_splits;
   const float* po = part_o + ((size_t)ridx * n_head + head) * n_splits * HD + d;
   // every thread works the weights of the splits out for itself: they are few, and no thread waits
-  // for another
-  if (n_splits <= 8) {
-    // everything asked for at once (splits beyond the last repeat it and count for nothing)
-    float v[8];
-    float2 ml[8];
+  // for another.  Up to 16 splits: everything asked for at once, one round trip to memory (splits
+  // beyond the last repeat it and count for nothing).
+  auto at_once = [&](auto cap_tag) {
+    constexpr int CAP = decltype(cap_tag)::value;
+    float v[CAP];
+    float2 ml[CAP];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < CAP; ++j) {
       const int sj = j < n_splits ? j : n_splits - 1;
       ml[j] = pm[sj];
       v[j] = po[(size_t)sj * HD];
     }
     float mm = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+    for (int j = 0; j < CAP; ++j)
       if (j < n_splits) mm = fmaxf(mm, ml[j].x);
     float acc = 0.f, lt = 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+    for (int j = 0; j < CAP; ++j)
       if (j < n_splits) {
         const float w = split_weight(ml[j].x, mm);
         lt = fmaf(ml[j].y, w, lt);
         acc = split_accumulate(acc, v[j], w);
       }
     out[((size_t)m_row * n_head + head) * HD + d] = f2bf(acc * (1.0f / lt));
+  };
+  if (n_splits <= 8) {
+    at_once(std::integral_constant<int, 8>{});
+    return;
+  }
+  if (n_splits <= 16) {
+    at_once(std::integral_constant<int, 16>{});
     return;
   }
   float mm = -INFINITY;
