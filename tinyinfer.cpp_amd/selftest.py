@@ -92,6 +92,16 @@ def case_linear(ops, rng) -> int:
     ops.linear(_dev(a, torch.bfloat16), _dev(w, torch.bfloat16), out, "swiglu")
     swi = g / (1 + np.exp(-g)) * u
     fails += _say("product + SwiGLU (bfloat16 out)", float(np.abs(_f64(out) - swi).max()), 0.005 * np.abs(swi).max() + 1e-3)
+    # few rows times a long K (the token rows go through LDS in pieces; with a long K under few weight
+    # rows the sums of several workgroups are left to whatever reads the residual next)
+    for M, N, K in ((7, 2100, 5120), (16, 2064, 17408)):
+        a, w = _bf16(rng.uniform(-1, 1, (M, K))), _bf16(rng.uniform(-1, 1, (N, K)))
+        base = rng.normal(size=(M, N)).astype(np.float32)
+        out = _dev(base.copy())
+        ops.linear(_dev(a, torch.bfloat16), _dev(w, torch.bfloat16), out, "add", may_defer=True)
+        ops.flush()
+        fails += _say(f"product {M}x{N}x{K} + residual add (K in pieces)", float(np.abs(_f64(out) - (a @ w.T + base)).max()),
+                      2e-5 * K)
     return fails
 
 
@@ -121,7 +131,16 @@ def case_rmsnorm(ops, rng) -> int:
     want = xd / np.sqrt((xd * xd).mean(-1, keepdims=True) + eps) * w
     out = torch.empty(rows, n, device="cuda")
     ops.rmsnorm(_dev(x), _dev(w), eps, out)
-    return _say("RMSNorm 3x1024", float(np.abs(_f64(out) - want).max()), 1e-4)
+    fails = _say("RMSNorm 3x1024", float(np.abs(_f64(out) - want).max()), 1e-4)
+    # rows wider than 4,096 take a workgroup each
+    rows, n = 5, 5120
+    x, w = rng.uniform(-1, 1, (rows, n)).astype(np.float32), rng.uniform(-1, 1, n).astype(np.float32)
+    xd = x.astype(np.float64)
+    want = xd / np.sqrt((xd * xd).mean(-1, keepdims=True) + eps) * w
+    out = torch.empty(rows, n, device="cuda")
+    ops.rmsnorm(_dev(x), _dev(w), eps, out)
+    fails += _say("RMSNorm 5x5120", float(np.abs(_f64(out) - want).max()), 1e-4)
+    return fails
 
 
 def _rotate(x, positions, theta):
