@@ -886,11 +886,12 @@ def test_rmsnorm_that_adds_partial_sums(ops, rows, H, KS):
         assert (f64(out) - ref_rmsnorm(want_x, w, 1e-6)).abs().max() < (1e-5 if dtype == torch.float32 else 0.03)
 
 
-@pytest.mark.parametrize("tile", [1, 3, 6])
+@pytest.mark.parametrize("tile", [1, 3, 5, 6])
 @pytest.mark.parametrize("M,N,K", [(300, 520, 128), (257, 384, 192), (130, 200, 64), (700, 96, 320)])
 def test_linear_bf16_every_tile(ops, tile, M, N, K):
-    """Each tile of the pipelined kernel (256 x 128 with eight wavefronts, 128 x 64, 64 x 64), whatever
-    the dispatch would have chosen for the shape, with every epilogue, against float64."""
+    """Each tile of the pipelined kernel (256 x 128 with eight wavefronts, 128 x 64, 64 x 128 for the SwiGLU
+    epilogue, 64 x 64), whatever the dispatch would have chosen for the shape, with every epilogue, against
+    float64."""
     if not ops.use_fast_gemm:
         pytest.skip("bfloat16 MFMA kernels are switched off")
     lib = ops.lib("gemm_bf16")
@@ -919,6 +920,32 @@ def test_linear_bf16_every_tile(ops, tile, M, N, K):
         assert (f64(out) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
     finally:
         lib.ti_gemm_bf16_force_tile(0)
+
+
+@pytest.mark.parametrize("M", [17, 40, 64])
+def test_swiglu_of_up_to_64_rows_under_a_wide_weight(ops, M):
+    """17 to 64 rows times a stacked [gate; up] weight of 32,768 rows take 64 x 128 tiles (twice the weight
+    under way per workgroup); the bits are those of the 128 x 64 tiles, and the values match float64."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    F, K = 16384, 1024
+    g = torch.Generator().manual_seed(M)
+    a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    w = dev((torch.rand(2 * F, K, generator=g) * 2 - 1).to(torch.bfloat16) * 0.1)
+    ref = ref_linear(a.cpu(), w.cpu())
+    want = ref[:, :F] / (1 + torch.exp(-ref[:, :F])) * ref[:, F:]
+    lib = ops.lib("gemm_bf16")
+    outs = []
+    try:
+        for tile in (0, 3):
+            lib.ti_gemm_bf16_force_tile(tile)
+            out = torch.empty(M, F, device="cuda", dtype=torch.bfloat16)
+            ops.linear(a, w, out, "swiglu")
+            assert (f64(out) - want).abs().max() < 0.005 * want.abs().max() + 2e-4 * K
+            outs.append(out)
+    finally:
+        lib.ti_gemm_bf16_force_tile(0)
+    assert torch.equal(outs[0], outs[1])
 
 
 def test_linear_bf16_rows_do_not_depend_on_the_batch(ops):

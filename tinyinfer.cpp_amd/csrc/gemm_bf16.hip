@@ -1209,7 +1209,7 @@ extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K,
   return 0;
 }
 
-// for measurements: 0 = choose the tile by the shape, 1 = 256 x 128, 3 = 128 x 64, 6 = 64 x 64
+// for measurements: 0 = choose the tile by the shape, 1 = 256 x 128, 3 = 128 x 64, 5 = 64 x 128 (SwiGLU only), 6 = 64 x 64
 static int g_force_tile = 0;
 extern "C" void ti_gemm_bf16_force_tile(int which) { g_force_tile = which; }
 
@@ -1221,13 +1221,22 @@ template <int EPI>
 static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
                              hipStream_t s) {
   const int cols = (EPI == TI_EPI_SWIGLU) ? 2 : 1;   // a SwiGLU workgroup covers BN / 2 output columns
+  constexpr bool SW = EPI == TI_EPI_SWIGLU;
   const long big = (long)((M + 255) / 256) * ((N * cols + 127) / 128);
   const long mid = (long)((M + 127) / 128) * ((N * cols + 63) / 64);
   const bool whole_rounds = big >= 256 && (big % 256 == 0 || big % 256 >= 192);
   int tile = (big >= 1024 || whole_rounds) ? 1 : (mid >= 512 ? 3 : 6);
   if (M <= 64 && tile == 1) tile = 6;                // few rows times a wide weight: no 256-row tile
+  // Up to 64 rows times a stacked [gate; up] weight: such a product waits for the weight from memory, and
+  // a 128 x 64 tile, half of whose rows are empty then, has 8 of its 24 KB a stage in weights.  A 64 x 128
+  // tile has 16 of 24, two workgroups to a unit as well: twice the weight under way (Qwen3-32B's gate/up
+  // at 64 rows 141 -> 115 us, 8B's 52 -> 45); a weight that gives it fewer workgroups than half the
+  // units stays with the narrower tile (0.6B's: 10.0 against 10.6 us).
+  if (SW && M <= 64 && (long)(N * cols + 127) / 128 * 2 >= compute_units()) tile = 5;
   if (g_force_tile) tile = g_force_tile;
   if (tile == 1) return launch_pipelined<256, 128, 4, 2, EPI>(A, W, out, M, N, K, lda, s);
+  if constexpr (EPI == TI_EPI_SWIGLU)
+    if (tile == 5) return launch_pipelined<64, 128, 2, 2, EPI>(A, W, out, M, N, K, lda, s);
   if constexpr (EPI != TI_EPI_SWIGLU)                // a SwiGLU wavefront needs two column tiles
     if (tile == 6) return launch_pipelined<64, 64, 2, 2, EPI>(A, W, out, M, N, K, lda, s);
   return launch_pipelined<128, 64, 4, 1, EPI>(A, W, out, M, N, K, lda, s);
