@@ -6,7 +6,7 @@ import pytest
 from tinyinfer_amd.cache import CacheError, CacheManager, OutOfPages
 from tinyinfer_amd.engine.scheduler import Scheduler, SchedulerError
 from tinyinfer_amd.sampling import SamplingParams, uniform
-from tinyinfer_amd.spec import PagedKVNeed, StateNeed
+from tinyinfer_amd.spec import PagedKVNeed, PagedRowsNeed, StateNeed
 
 FULL = PagedKVNeed(2, 16, None)
 WIN = PagedKVNeed(2, 16, 10)
@@ -112,6 +112,28 @@ def test_window_group_gives_pages_back_as_the_window_passes():
     m.release("a")
     m.release("b")
     assert m.groups[0].pool.num_free == 20 and m.groups[1].pool.num_free == 20
+    m.check()
+
+
+def test_pages_of_rows_of_another_shape_are_a_group_of_their_own():
+    """A part that keeps rows of its own per token (neither keys nor values) gets pages, block tables and the
+    window rule like any other paged group, apart from groups of another need."""
+    rows = PagedRowsNeed((24,), float32=True, window=6)
+    m = manager(groups=((FULL, 1), (rows, 2), (PagedRowsNeed((24,), float32=True, window=6), 1), (PagedRowsNeed((24,)), 1)),
+                page_size=4, pages=12)
+    assert [type(g.need).__name__ for g in m.groups] == ["PagedKVNeed", "PagedRowsNeed", "PagedRowsNeed", "PagedRowsNeed"]
+    assert m.groups[1].need == m.groups[2].need != m.groups[3].need
+    m.admit("a")
+    for _ in range(21):
+        m.reserve("a", 1)
+        m.commit("a", 1)
+        m.check()
+    assert sum(p >= 0 for p in m.table(0, "a")) == 6 and sum(p >= 0 for p in m.table(3, "a")) == 6
+    # the next token is position 21 and reads rows 16..21: pages 0..3 are gone
+    assert [p >= 0 for p in m.table(1, "a")] == [False] * 4 + [True] * 2
+    assert m.groups[1].pool.num_free == 10
+    m.release("a")
+    assert all(g.pool.num_free == 12 for g in m.groups)
     m.check()
 
 

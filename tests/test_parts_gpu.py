@@ -123,7 +123,7 @@ def register_toys():
     import tinyinfer_amd as ti
     from tinyinfer_amd.parts import Part
     from tinyinfer_amd.parts.base import join
-    from tinyinfer_amd.spec import LayerSpec, ModelSpec, PartSpec, StateNeed, TensorNeed
+    from tinyinfer_amd.spec import LayerSpec, ModelSpec, PagedRowsNeed, PartSpec, StateNeed, TensorNeed
 
     class DecayMixer(Part):
         """A mixer with state of its own: s_t = decay * s_{t-1} + h_t W^T; out_t = s_t.
@@ -153,6 +153,40 @@ def register_toys():
                     s = self.decay * s + u[t]
                     x[t] += s
                 state[slot] = s
+
+    class WindowMean(Part):
+        """A mixer with pages of its own: every token keeps u_t = h_t W^T (one row of 32-bit numbers per
+        token and layer, in pages the cache manager hands out and takes back); out_t is the mean of
+        the rows of the last `window` tokens."""
+        family = "mixer"
+
+        def __init__(self, prefix, hidden, window):
+            super().__init__(prefix)
+            self.hidden, self.window = hidden, window
+
+        def tensors(self):
+            return {join(self.prefix, "w"): TensorNeed((self.hidden, self.hidden), "matrix", ("normal", 0.0, 0.2))}
+
+        def load(self, tensors):
+            self.w = tensors[join(self.prefix, "w")]
+
+        def cache_need(self):
+            return PagedRowsNeed((self.hidden,), float32=True, window=self.window)
+
+        def forward(self, ctx, h, x):
+            group, layer = ctx.binding(self)
+            pool = ctx.page_pool(group, layer)               # [pages, P, hidden] float32
+            view = ctx.cache_view(group)
+            P = view.page_size
+            u = h.float() @ self.w.float().T
+            for e, (row0, n, start, slot) in enumerate(ctx.entries):
+                table = view.table[e].tolist()
+                for i in range(n):
+                    p = start + i
+                    assert table[p // P] >= 0
+                    pool[table[p // P], p % P] = u[row0 + i]
+                    rows = [pool[table[q // P], q % P] for q in range(max(0, p - self.window + 1), p + 1)]
+                    x[row0 + i] += torch.stack(rows).mean(0)
 
     class BareBlock(Part):
         """An arrangement with a mixer and nothing else: x += mixer(cast(x))."""
@@ -245,6 +279,9 @@ def register_toys():
             elif kind == "decay":
                 layers.append(LayerSpec(f"l.{i}", PartSpec("bare"), {
                     "mixer": PartSpec("toy_decay", {"hidden": H, "decay": c["decay"]}, "mix")}))
+            elif kind == "memory":
+                layers.append(LayerSpec(f"l.{i}", PartSpec("bare"), {
+                    "mixer": PartSpec("toy_window_mean", {"hidden": H, "window": c["memory_window"]}, "mem")}))
             elif kind == "bare_attention":
                 layers.append(LayerSpec(f"l.{i}", PartSpec("bare"), {"mixer": attn}))
             else:
@@ -258,6 +295,7 @@ def register_toys():
                          schedule=c.get("schedule"))
 
     ti.register_part("mixer", "toy_decay", DecayMixer)
+    ti.register_part("mixer", "toy_window_mean", WindowMean)
     ti.register_part("ffn", "toy_routed", RoutedFFN)
     ti.register_part("pos", "toy_pair_rotary", PairRotary)
     ti.register_part("block", "bare", BareBlock)
@@ -294,6 +332,10 @@ def toy_plain(cfg, w, toks):
             for t in range(T):
                 s = cfg["decay"] * s + u[t]
                 out[t] = s
+            x = x + out
+        elif kind == "memory":
+            u = x @ w[p + ".mem.w"].T
+            out = np.stack([u[max(0, t - cfg["memory_window"] + 1):t + 1].mean(0) for t in range(T)])
             x = x + out
         else:
             full = kind in ("full", "routed")
@@ -372,6 +414,47 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     assert engine.cache.slot("c") == 0                      # the slot a held
     for r in reqs:
         assert np.abs(np.concatenate(got[r]) - want[r]).max() < 2e-4, r
+
+
+def test_toy_mixer_with_pages_of_its_own(tmp_path):
+    """A mixer that keeps a row of its own per token in pages (neither keys nor values) behind a window:
+    registered in this file, built, stepped in portions beside another request, with so few pages that
+    the ones the window has passed are handed out again; against the whole-sequence numpy model."""
+    import tinyinfer_amd as ti
+    cfg = dict(TOY, layers=["memory", "full", "memory"], memory_window=6)
+    engine, w = toy_engine(tmp_path, cfg, max_tokens=72)
+    needs = sorted(type(n).__name__ for n, _ in engine.model.cache_groups)
+    assert needs == ["PagedKVNeed", "PagedRowsNeed"]
+    groups = {type(n).__name__: i for i, (n, _) in enumerate(engine.model.cache_groups)}
+    mem = groups["PagedRowsNeed"]
+    assert engine.page_pool(mem, 1).shape == (18, 4, 32) and engine.page_pool(mem, 1).dtype == torch.float32
+    reqs = {"a": random_tokens(50, 90, 3), "b": random_tokens(21, 90, 4)}
+    want = {r: toy_plain(cfg, w, t) for r, t in reqs.items()}
+    got = {r: [] for r in reqs}
+
+    def run(entries):
+        logits = engine.step(entries).cpu().numpy()
+        i = 0
+        for e in entries:
+            got[e.request].append(logits[i:i + len(e.tokens)])
+            i += len(e.tokens)
+
+    def feed(r, lo, hi):
+        return ti.StepEntry(r, reqs[r][lo:hi], list(range(hi - lo)))
+    free_before = engine.cache.groups[mem].pool.num_free
+    run([feed("a", 0, 13), feed("b", 0, 2)])
+    run([feed("a", 13, 14), feed("b", 2, 21)])
+    engine.release("b")
+    for t in range(14, 30):
+        run([feed("a", t, t + 1)])
+    run([feed("a", 30, 50)])
+    # behind the window of 6 the memory's pages have gone back: a request of 50 tokens holds at most 3 of them
+    assert len([p for p in engine.cache.table(mem, "a") if p >= 0]) <= 3
+    engine.cache.check()
+    for r in reqs:
+        assert np.abs(np.concatenate(got[r]) - want[r]).max() < 2e-4, r
+    engine.release("a")
+    assert engine.cache.groups[mem].pool.num_free == free_before
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

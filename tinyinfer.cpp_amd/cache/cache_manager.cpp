@@ -20,7 +20,7 @@ namespace tinyinfer {
 
 bool CacheNeed::operator==(const CacheNeed& o) const {
   return kind == o.kind && kv_heads == o.kv_heads && head_dim == o.head_dim && window == o.window &&
-         state_shape == o.state_shape;
+         state_shape == o.state_shape && row_shape == o.row_shape && rows_f32 == o.rows_f32;
 }
 
 // `scatter_window` > 1: the pages are first handed out in a fixed pseudo-random order within
@@ -78,7 +78,7 @@ CacheManager::CacheManager(const std::vector<std::pair<CacheNeed, int>>& groups,
     Group grp;
     grp.need = g.first;
     grp.n_layers = g.second;
-    grp.paged = g.first.kind == CacheNeed::PagedKV;
+    grp.paged = g.first.paged();
     if (grp.paged) {
       grp.pool.reset(new PagePool(num_pages, scatter_window));
       paged_.push_back((int)groups_.size());

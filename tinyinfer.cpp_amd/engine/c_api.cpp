@@ -85,6 +85,13 @@ Json cache_need_json(const CacheNeed& n) {
     j.set("kv_heads", n.kv_heads);
     j.set("head_dim", n.head_dim);
     j.set("window", n.window > 0 ? Json(n.window) : Json());
+  } else if (n.kind == CacheNeed::PagedRows) {
+    j.set("kind", "paged_rows");
+    Json s = Json::array();
+    for (int64_t v : n.row_shape) s.push(v);
+    j.set("row_shape", s);
+    j.set("float32", n.rows_f32);
+    j.set("window", n.window > 0 ? Json(n.window) : Json());
   } else {
     j.set("kind", "state");
     Json s = Json::array();
@@ -98,6 +105,11 @@ CacheNeed cache_need_from(const Json& c) {
   if (c.at("kind").as_string() == "state") {
     n.kind = CacheNeed::State;
     for (const Json& s : c.at("shape").items()) n.state_shape.push_back(s.as_int());
+  } else if (c.at("kind").as_string() == "paged_rows") {
+    n.kind = CacheNeed::PagedRows;
+    for (const Json& s : c.at("row_shape").items()) n.row_shape.push_back(s.as_int());
+    n.rows_f32 = c.has("float32") && c.at("float32").as_bool();
+    n.window = (c.has("window") && !c.at("window").is_null()) ? (int)c.at("window").as_int() : 0;
   } else {
     n.kind = CacheNeed::PagedKV;
     n.kv_heads = (int)c.at("kv_heads").as_int();

@@ -11,6 +11,7 @@ include/inference.h); this object reads from it.
   ctx.buf(name, shape, dtype)  scratch memory, the same for the same name in every layer and step
   ctx.binding(part)            (group, cache layer) of the part's cache in this run of its layer
   ctx.kv_pool(group, layer)    [pages, 2, kv heads, P, head_dim]
+  ctx.page_pool(group, layer)  [pages, P, ...]: the pages of a part that keeps rows of its own per token
   ctx.cache_view(group)        .table int32 [entries, pages per request], .page_size
   ctx.state(group, layer)      float32 [slots, ...]; index with an entry's state slot
 """
@@ -81,6 +82,13 @@ class StepContext:
         native.call("ti_ctx_kv_pool", self._native, group, layer, ctypes.byref(out))
         t = native.wrap(out)
         return t.view(t.shape[0], 2, t.shape[1] // 2, t.shape[2], t.shape[3])
+
+    def page_pool(self, group: int, layer: int):
+        """The pages of one cache layer as the library lays them out: [pages, P, ...] for a need of rows of
+        its own (`PagedRowsNeed`), [pages, 2 x kv heads, P, head_dim] for keys and values."""
+        out = native.ti_tensor()
+        native.call("ti_ctx_kv_pool", self._native, group, layer, ctypes.byref(out))
+        return native.wrap(out)
 
     def cache_view(self, group: int) -> CacheView:
         out, page = native.ti_tensor(), ctypes.c_int()

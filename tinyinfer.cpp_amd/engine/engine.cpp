@@ -528,6 +528,12 @@ Engine::Engine(std::shared_ptr<Model> model_, const EngineOptions& o)
     size_t per_layer;
     if (g.first.kind == CacheNeed::PagedKV) {
       per_layer = (size_t)num_pages * 2 * g.first.kv_heads * page_size * g.first.head_dim * dtype_size(act_dtype);
+    } else if (g.first.kind == CacheNeed::PagedRows) {
+      if (g.first.row_shape.empty() || g.first.row_shape.size() > 2)
+        throw EngineError("a paged cache of rows needs a row shape of one or two dimensions");
+      size_t n = 1;
+      for (int64_t s : g.first.row_shape) n *= (size_t)s;
+      per_layer = (size_t)num_pages * page_size * n * (g.first.rows_f32 ? 4 : dtype_size(act_dtype));
     } else {
       size_t n = 1;
       for (int64_t s : g.first.state_shape) n *= (size_t)s;
@@ -569,8 +575,16 @@ size_t Engine::cache_bytes() const {
 }
 Tensor Engine::kv_pool(int group, int layer) const {
   const auto& g = model->cache_groups.at(group);
-  if (g.first.kind != CacheNeed::PagedKV) throw EngineError("cache group " + std::to_string(group) + " has no pages");
+  if (!g.first.paged()) throw EngineError("cache group " + std::to_string(group) + " has no pages");
   if (layer < 0 || layer >= g.second) throw EngineError("cache group " + std::to_string(group) + " has no layer " + std::to_string(layer));
+  if (g.first.kind == CacheNeed::PagedRows) {
+    std::vector<int64_t> shape = {num_pages, (int64_t)page_size};
+    for (int64_t s : g.first.row_shape) shape.push_back(s);
+    Tensor t((char*)impl_->storage[group].data() + (size_t)layer * impl_->layer_bytes[group],
+             g.first.rows_f32 ? DType::F32 : act_dtype, {shape[0], shape[1], shape[2]});
+    if (shape.size() == 4) t = Tensor(t.data, t.dtype, {shape[0], shape[1], shape[2], shape[3]});
+    return t;
+  }
   return Tensor((char*)impl_->storage[group].data() + (size_t)layer * impl_->layer_bytes[group], act_dtype,
                 {num_pages, 2 * (int64_t)g.first.kv_heads, (int64_t)page_size, (int64_t)g.first.head_dim});
 }

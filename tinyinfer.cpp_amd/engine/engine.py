@@ -168,6 +168,12 @@ class Engine:
         t = native.wrap(out)
         return t.view(t.shape[0], 2, t.shape[1] // 2, t.shape[2], t.shape[3])
 
+    def page_pool(self, group: int, layer: int):
+        """The pages of one cache layer as the library lays them out ([pages, P, ...] for a `PagedRowsNeed`)."""
+        out = native.ti_tensor()
+        native.call("ti_engine_kv_pool", self._ptr, group, layer, ctypes.byref(out))
+        return native.wrap(out)
+
     def state(self, group: int, layer: int):
         out = native.ti_tensor()
         native.call("ti_engine_state", self._ptr, group, layer, ctypes.byref(out))

@@ -230,9 +230,15 @@ struct TensorNeed {
   bool optional = false;                 // absent from the checkpoint is allowed
 };
 struct CacheNeed {
-  enum Kind { PagedKV, State } kind = PagedKV;
-  int kv_heads = 0, head_dim = 0, window = 0;    // PagedKV; window 0: every key is kept
+  // PagedKV: keys and values per token, in the layout the attention kernels read.  PagedRows: whatever a
+  // token keeps, `row_shape` elements per token and layer in pages of their own layout [page][row][...]
+  // (a mixer with another kind of memory than keys and values).  State: a fixed size per request.
+  enum Kind { PagedKV, State, PagedRows } kind = PagedKV;
+  int kv_heads = 0, head_dim = 0, window = 0;    // PagedKV; window (PagedRows too) 0: every token is kept
   std::vector<int64_t> state_shape;              // State: float32 per request and layer, zeroed at admission
+  std::vector<int64_t> row_shape;                // PagedRows: one or two dimensions, in the compute dtype ...
+  bool rows_f32 = false;                         // ... or in float32
+  bool paged() const { return kind != State; }
   bool operator==(const CacheNeed& o) const;
 };
 
@@ -425,7 +431,7 @@ class StepContext {
   Tensor buf(const std::string& name, DType dt, std::initializer_list<int64_t> dims) { return ws.tensor(name, dt, dims); }
   // the cache of the part that is running: (group, cache layer) as the model bound it for this run
   std::pair<int, int> binding(const Part* part) const;
-  Tensor kv_pool(int group, int layer) const;                 // [pages][2][kv heads][P][head_dim]
+  Tensor kv_pool(int group, int layer) const;                 // [pages][2 x kv heads][P][head_dim]; PagedRows: [pages][P][row...]
   Ops::CacheView cache_view(int group) const;                 // the block-table rows of the step's entries
   Tensor state(int group, int layer) const;                   // f32 [slots][...]
   // a list a part planned for this step (device memory), and values

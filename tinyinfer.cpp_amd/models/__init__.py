@@ -1,2 +1,2 @@
-from ..spec import ModelSpec, LayerSpec, PartSpec, TensorNeed, PagedKVNeed, StateNeed
+from ..spec import ModelSpec, LayerSpec, PartSpec, TensorNeed, PagedKVNeed, PagedRowsNeed, StateNeed
 from .model import Model

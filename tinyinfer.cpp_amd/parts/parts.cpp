@@ -633,6 +633,11 @@ ForeignInfo read_description(const Json& d) {
     if (c.at("kind").as_string() == "state") {
       info.cache.kind = CacheNeed::State;
       for (const Json& s : c.at("shape").items()) info.cache.state_shape.push_back(s.as_int());
+    } else if (c.at("kind").as_string() == "paged_rows") {
+      info.cache.kind = CacheNeed::PagedRows;
+      for (const Json& s : c.at("row_shape").items()) info.cache.row_shape.push_back(s.as_int());
+      info.cache.rows_f32 = c.has("float32") && c.at("float32").as_bool();
+      info.cache.window = (c.has("window") && !c.at("window").is_null()) ? (int)c.at("window").as_int() : 0;
     } else {
       info.cache.kind = CacheNeed::PagedKV;
       info.cache.kv_heads = (int)c.at("kv_heads").as_int();

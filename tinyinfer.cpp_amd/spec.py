@@ -126,9 +126,24 @@ class StateNeed:
         return {"kind": "state", "shape": list(self.shape)}
 
 
+@dataclass(frozen=True)
+class PagedRowsNeed:
+    """Whatever a token keeps, `row_shape` elements per token and layer, in pages [page, row, ...] of
+    the compute dtype (`float32`: of float32): a mixer with another kind of memory than keys and
+    values.  `window` as for keys and values."""
+    row_shape: Tuple[int, ...]
+    float32: bool = False
+    window: Optional[int] = None
+
+    def to_dict(self) -> dict:
+        return {"kind": "paged_rows", "row_shape": list(self.row_shape), "float32": self.float32, "window": self.window}
+
+
 def cache_need_from_dict(d):
     if d is None:
         return None
     if d["kind"] == "state":
         return StateNeed(tuple(d["shape"]))
+    if d["kind"] == "paged_rows":
+        return PagedRowsNeed(tuple(d["row_shape"]), bool(d.get("float32")), d.get("window"))
     return PagedKVNeed(d["kv_heads"], d["head_dim"], d.get("window"))
