@@ -69,6 +69,8 @@ def test_context_splits_of_the_decode_kernel(monkeypatch):
     assert a.decode_splits(1, 8, 16, 4096, 2112) == 16         # bounded: 16 blocks of 16 keys a run at least
     assert a.decode_splits(1, 8, 16, 100, 100) == 1            # a short context is not split
     assert a.decode_splits(1, 1, 64, 10 ** 6, 10 ** 6) <= a.MAX_SPLITS
+    # half the bytes per token (head size 64): a run is worth its prologue only if twice as long
+    assert a.decode_splits(12, 8, 16, 4096, 2112, head_dim=64) <= a.decode_splits(12, 8, 16, 4096, 2112)
     for rows in range(1, 70):
         for context in (300, 2000, 9000, 40000):
             s = a.decode_splits(rows, 8, 16, context)

@@ -1123,8 +1123,8 @@ int ti_ops_timing_report(void* ops_, const char** out) {
   return give(out, a.dump());
   TI_END
 }
-int ti_decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units) {
-  return Ops::decode_splits(n_rows, kv_heads, heads, context, typical, units);
+int ti_decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units, int head_dim) {
+  return Ops::decode_splits(n_rows, kv_heads, heads, context, typical, units, head_dim);
 }
 
 }  // extern "C"

@@ -317,7 +317,7 @@ class Ops {
     int force_paired_tiles = -1;    // 1 / 0: that kernel with / without pairs, whatever the launch
     int force_decode_splits = 0;    // > 0: the decode attention cuts every context into this many runs
   } use;
-  static int decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units);
+  static int decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units, int head_dim = 128);
   // runs of keys for the prefill kernel with 64-row tiles, and whether it pairs a heavy with a light tile
   static int portion_launch(int n_tiles_small, int heads, int portion_context, int window, int units, bool* paired);
 
@@ -946,6 +946,6 @@ int ti_ops_switch(void* ops, const char* name, int value, int* old);
 int ti_ops_call(void* ops, const char* op, const ti_tensor* t, int n_t, const double* scalars, int n_scalars,
                 const char* text, ti_tensor* result);
 int ti_ops_timing_report(void* ops, const char** out_json);     // [{"name", "calls", "us"}] since timing was switched on
-int ti_decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units);
+int ti_decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units, int head_dim);
 int ti_portion_launch(int n_tiles_small, int heads, int portion_context, int window, int units, int* paired);
 }

@@ -187,7 +187,7 @@ def lib() -> ctypes.CDLL:
         handle.ti_uniform.restype = c_float
         handle.ti_uniform.argtypes = [c_u64, c_u64, c_u64]
         handle.ti_decode_splits.restype = c_int
-        handle.ti_decode_splits.argtypes = [c_int] * 6
+        handle.ti_decode_splits.argtypes = [c_int] * 7
         handle.ti_portion_launch.restype = c_int
         handle.ti_portion_launch.argtypes = [c_int] * 5 + [P(c_int)]
         handle.ti_detach_allocator.restype = None

@@ -15,9 +15,9 @@ def compute_units() -> int:
     return int(get_ops()._call("compute_units", libs=["core"]))
 
 
-def decode_splits(n_rows: int, kv_heads: int, heads: int, context: int, typical: int = 0) -> int:
+def decode_splits(n_rows: int, kv_heads: int, heads: int, context: int, typical: int = 0, head_dim: int = 128) -> int:
     """Into how many runs the decode kernel splits the context (`Ops::decode_splits`)."""
-    return int(native.lib().ti_decode_splits(n_rows, kv_heads, heads, context, typical or context, compute_units()))
+    return int(native.lib().ti_decode_splits(n_rows, kv_heads, heads, context, typical or context, compute_units(), head_dim))
 
 
 def portion_launch(ctx, heads: int, window: int):

@@ -615,7 +615,7 @@ void Ops::attention_rows(const Tensor& q, const Tensor& pool, const CacheView& v
 static const int MAX_SPLITS = 64;             // the merge kernel's limit
 static const int MIN_BLOCKS_PER_SPLIT = 16;   // four 16-key blocks per wavefront at least
 static const double SPLIT_PROLOGUE_US = 5.0;  // position, table row, query, page ids: before a workgroup's first key arrives
-static const double SPLIT_TOKEN_US = 0.019;   // per token of context that one workgroup walks
+static const double SPLIT_TOKEN_US = 0.019;   // per token of context that one workgroup walks, at 512 bytes of key and value a token
 static const double SPLIT_MERGE_US = 4.0;     // the merge kernel, which a launch without splits does without
 
 // Into how many runs the decode kernel splits the context.  `context`: the longest context the
@@ -623,13 +623,13 @@ static const double SPLIT_MERGE_US = 4.0;     // the merge kernel, which a launc
 // captured graph is sized for the longest sequence, but replayed mostly on shorter ones).  The
 // number that makes rounds x (prologue + run) + merge the least, rounds being the workgroups over
 // the compute units, rounded up.
-int Ops::decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units) {
+int Ops::decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units, int head_dim) {
   if (typical <= 0) typical = context;
   const int parts = (heads / kv_heads + 15) / 16;
   const long base = std::max(1L, (long)n_rows * kv_heads * parts);
   const int blocks = (std::max(1, context) + 15) / 16;
   const int limit = std::max(1, std::min(blocks / MIN_BLOCKS_PER_SPLIT, MAX_SPLITS));
-  const double walk = SPLIT_TOKEN_US * std::max(1, typical);
+  const double walk = SPLIT_TOKEN_US * std::max(1, typical) * (head_dim > 0 ? head_dim / 128.0 : 1.0);
   int best = 1;
   double best_cost = -1.0;
   for (int s = 1; s <= limit; ++s) {
@@ -684,7 +684,7 @@ bool Ops::attention_from_projections(const AttentionWork& work, Workspace& ws, c
   if ((head_dim != 64 && head_dim != 128) || P % 16 != 0 || heads / kv_heads > 16) return false;
   const int n = (int)work.M;
   const int context = window == 0 ? work.split_context : std::min(work.split_context, window + 16);
-  int S = decode_splits(n, kv_heads, heads, context, std::min(context, typical_context(work)), compute_units());
+  int S = decode_splits(n, kv_heads, heads, context, std::min(context, typical_context(work)), compute_units(), head_dim);
   if (use.force_decode_splits > 0) S = std::min(use.force_decode_splits, std::max(1, (context + 15) / 16));
   float *part_o = nullptr, *part_ml = nullptr;
   if (S > 1) {
@@ -744,7 +744,7 @@ void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& v
       if (done && n_dec) {
         const int* rows = work.decode_only ? nullptr : work.decode_rows;
         const int context = window == 0 ? work.split_context : std::min(work.split_context, window + 16);
-        const int S = decode_splits(n_dec, kv_heads, heads, context, std::min(context, typical_context(work)), units);
+        const int S = decode_splits(n_dec, kv_heads, heads, context, std::min(context, typical_context(work)), units, head_dim);
         float *part_o = nullptr, *part_ml = nullptr;
         if (S > 1) {
           part_o = (float*)ws.get("attn.part_o", (size_t)n_dec * heads * S * head_dim * 4);
