@@ -948,6 +948,36 @@ def test_swiglu_of_up_to_64_rows_under_a_wide_weight(ops, M):
     assert torch.equal(outs[0], outs[1])
 
 
+@pytest.mark.parametrize("M", [17, 40, 64])
+def test_stored_product_of_17_to_64_rows_under_a_large_weight_splits_k(ops, M):
+    """17 to 64 rows times a weight of 6,144 x 4,096 (the q/k/v projection of a large model), stored in
+    32-bit: K goes to several workgroups a tile and a kernel of its own adds their sums.  Against float64,
+    against the product with the split switched off (the same values up to the order of the sum), and a
+    row's bits do not depend on the rows beside it."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    N, K = 6144, 4096
+    g = torch.Generator().manual_seed(M)
+    a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    ref = ref_linear(a.cpu(), w.cpu())
+    out = torch.full((M + 1, N), 7.0, device="cuda")
+    ops.linear(a, w, out[:M], "store")
+    assert (f64(out[:M]) - ref).abs().max() < 2e-5 * K
+    assert bool((out[M] == 7.0).all())
+    try:
+        ops.use_split_k_add = False
+        plain_out = torch.empty(M, N, device="cuda")
+        ops.linear(a, w, plain_out, "store")
+    finally:
+        ops.use_split_k_add = True
+    assert (plain_out - out[:M]).abs().max() < 2e-5 * K
+    assert not torch.equal(plain_out, out[:M])              # the split did happen: another order of the sum
+    fewer = torch.empty(17, N, device="cuda")
+    ops.linear(a[M - 17:], w, fewer, "store")
+    assert torch.equal(fewer, out[M - 17:M])
+
+
 def test_linear_bf16_rows_do_not_depend_on_the_batch(ops):
     """Within one family of kernels a row's bits do not depend on the other rows: the tiled
     kernels (more than 64 rows), the kernels whose workgroups own 16 weight rows (9 to 64 rows

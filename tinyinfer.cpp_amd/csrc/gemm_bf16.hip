@@ -1913,6 +1913,47 @@ extern "C" int ti_gemm_bf16_pieces_any(const void* A, const void* W, void* out, 
   return 0;
 }
 
+// out[i] = partial[0][i] + ... + partial[KS - 1][i], in that order
+__global__ void __launch_bounds__(256)
+gemm_partials_sum_kernel(float* __restrict__ out, const float* __restrict__ partial, int KS, size_t count) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  float v = partial[i];
+  for (int s = 1; s < KS; ++s) v += partial[(size_t)s * count + i];
+  out[i] = v;
+}
+
+// The product that stores 32-bit results, for 17 to 64 rows times a large weight whose 64 x 64 tiles
+// are few (the q/k/v projection of a decode step of many requests with a large model: 96 to 160
+// workgroups that wait for the weight from memory with too little of it under way).  K is split over
+// four or eight workgroups a tile, which store their sums into `partial` [KS][M][N]; a kernel of its
+// own adds them up into `out` (Qwen3-8B's q/k/v at 64 rows: 27 -> 17 us).  The number of shares
+// depends on the weight's shape alone.  Returns 3 for what it does not serve.
+extern "C" int ti_gemm_bf16_store_split(const void* A, const void* W, void* out, int M, int N, int K, long lda,
+                                        void* partial, long partial_bytes, hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K, "gemm_bf16_store_split: bad sizes M=%d N=%d K=%d lda=%ld", M, N, K, lda);
+  int KS = 1;
+  if (g_add_split && g_use_pipelined && partial && M > 16 && M <= 64 && K % 64 == 0 && lda % 8 == 0 &&
+      !((uintptr_t)A & 15) && !((uintptr_t)W & 15) && !((uintptr_t)partial & 15) &&
+      large_weight(M, N, K, TI_EPI_STORE_F32) && !wide_rows_serves(M, N, K, TI_EPI_STORE_F32)) {
+    const long tiles = (N + 63) / 64;
+    const int nb = K / 64;
+    while (KS < 8 && tiles * KS * 2 <= 4L * compute_units() && nb / (KS * 2) >= 4 && (long)KS * 2 * 64 * 16 <= K) KS *= 2;
+    while (KS > 1 && (long)KS * M * N * 4 > partial_bytes) KS /= 2;
+  }
+  if (KS < 4) {
+    ti_set_error("gemm_bf16_store_split: serves 17 to 64 rows times a large weight of few tiles, K a multiple of 64");
+    return 3;
+  }
+  int rc_ = launch_pipelined<64, 64, 2, 2, TI_EPI_STORE_F32>((const bf16_t*)A, (const bf16_t*)W, partial, M, N, K, lda, stream,
+                                                             KS);
+  if (rc_) return rc_;
+  const size_t count = (size_t)M * N;
+  gemm_partials_sum_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>((float*)out, (const float*)partial, KS, count);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
 // hooks for tests of the kernel alone: any epilogue, K split `ks` ways (1: not split; partial sums
 // are added here)
 extern "C" int ti_gemm_bf16_mblocks_any(const void* A, const void* W, void* out, int M, int N, int K, long lda,

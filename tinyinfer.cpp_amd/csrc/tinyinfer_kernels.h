@@ -64,6 +64,10 @@ int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int N, int K, l
 int ti_gemm_bf16_add_split(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
                          void* partial, long partial_bytes, int defer, int* splits, hipStream_t stream);
 int ti_gemm_bf16_partials_add(float* out, const float* partial, int KS, long count, hipStream_t stream);
+// out = A W^T stored in 32-bit for 17..64 rows times a large weight of few tiles: K split over workgroups
+// (partial: workspace of partial_bytes), the shares added up by a kernel of its own; 3: not served
+int ti_gemm_bf16_store_split(const void* A, const void* W, void* out, int M, int N, int K, long lda, void* partial,
+                             long partial_bytes, hipStream_t stream);
 // the kernel of ti_gemm_bf16_add_split alone, for tests: any epilogue, 1..64 rows, K split ks ways
 int ti_gemm_bf16_mblocks_any(const void* A, const void* W, void* out, int M, int N, int K, long lda, int epi,
                              void* partial, int ks, hipStream_t stream);

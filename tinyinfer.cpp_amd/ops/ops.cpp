@@ -555,6 +555,14 @@ void Ops::linear(const Tensor& a, const Tensor& w, const Tensor& out, Epilogue e
       }
       if (rc != 3) check("gemm_bf16", rc, "linear(bf16, split K)");
     }
+    if (epi == Store && M > 16 && M <= 64 && use.split_k_add) {
+      void* stream = launch_stream();
+      if (!partials_.data()) partials_ = DeviceBuffer(PARTIALS_BYTES);
+      int rc = KERNEL("gemm_bf16", ti_gemm_bf16_store_split)(a.data, w.data, out.data, (int)M, (int)N, (int)K, lda,
+                                                             partials_.data(), (long)PARTIALS_BYTES, (hipStream_t)stream);
+      if (rc == 0) return;
+      if (rc != 3) check("gemm_bf16", rc, "linear(bf16, split K, stored)");
+    }
     int rc = KERNEL("gemm_bf16", ti_gemm_bf16)(a.data, w.data, out.data, (int)M, (int)N, (int)K, lda, (int)epi,
                                                (hipStream_t)launch_stream());
     if (rc == 0) return;
