@@ -123,7 +123,7 @@ def fill(engine, rids, context, rng, chunk=4096):
 def measure_decode(engine, sampler, batch, steps, warmup, context, rng, tag, kernel_times=False):
     """tokens/s and ms/step of `steps` decode steps at `batch`, every request at `context` tokens."""
     import torch
-    from tinyinfer_amd.engine import StepEntry
+    from tinyinfer_amd.engine import StepEntry, token_from_feedback
     from tinyinfer_amd.sampling import SamplingParams
     rids = [f"{tag}{i}" for i in range(batch)]
     fill(engine, rids, context, rng)
@@ -136,12 +136,29 @@ def measure_decode(engine, sampler, batch, steps, warmup, context, rng, tag, ker
         logits = engine.step_graph(entries) if graph else engine.step(entries)
         return sampler.sample(logits, greedy, nums, nums)            # reads the ids back: a full sync
 
-    for _ in range(warmup):
+    # As `run_requests` decodes: every step names its tokens by rows of the sampler's last call and is
+    # launched before the ids of the step before it are read, so the device does not wait for the host.
+    from_device = [StepEntry(r, [token_from_feedback(i)], (0,)) for i, r in enumerate(rids)]
+
+    def steps_ahead(n, ticket):
+        for _ in range(n):
+            now = sampler.sample_async(engine.step_graph(from_device), greedy, nums, nums, feed=engine)
+            sampler.collect(ticket)
+            ticket = now
+        return ticket
+
+    for _ in range(min(2, warmup)):
         last = one_step(last)
+    entries = [StepEntry(r, [t], (0,)) for r, t in zip(rids, last)]
+    ticket = sampler.sample_async(engine.step_graph(entries), greedy, nums, nums, feed=engine)
+    ticket = steps_ahead(max(0, warmup - 2), ticket)
+    last = sampler.collect(ticket)
+    entries = [StepEntry(r, [t], (0,)) for r, t in zip(rids, last)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        last = one_step(last)
+    ticket = sampler.sample_async(engine.step_graph(entries), greedy, nums, nums, feed=engine)
+    ticket = steps_ahead(steps - 1, ticket)
+    last = sampler.collect(ticket)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     table = None

@@ -369,6 +369,140 @@ def test_every_request_finishes_under_pressure(seed):
         assert len(p.entries) <= 3
 
 
+class AheadDriver(Driver):
+    """The same with the step behind each step planned and run before that step's tokens are
+    known, where the scheduler allows it: what `run_requests` does."""
+
+    def __init__(self, sched, next_token=lambda req: 7):
+        super().__init__(sched, next_token)
+        self.ahead_steps = 0
+        self.wasted_rows = 0
+
+    def feed(self, plan):
+        c = self.s.cache
+        for e in plan.entries:
+            if not c.has(e.request.key):
+                c.admit(e.request.key)
+            assert c.length(e.request.key) == e.start
+            c.reserve(e.request.key, e.n_tokens)
+        for e in plan.entries:
+            c.commit(e.request.key, e.n_tokens)
+        c.check()
+
+    def run(self, limit=10000):
+        c = self.s.cache
+        flying = None
+        while flying is not None or self.s.has_work():
+            if flying is None:
+                flying = self.s.plan()
+                self.feed(flying)
+            ahead = self.s.plan_ahead()
+            if ahead.entries:
+                self.feed(ahead)                      # launched before `flying`'s tokens are known
+                self.ahead_steps += 1
+            live = [e for e in flying.entries if not e.request.finish_reason]
+            self.wasted_rows += len(flying.entries) - len(live)
+            sampled = {e.request.number: self.next_token(e.request) for e in live if e.sample}
+            for r in self.s.commit(flying, sampled):
+                c.release(r.key)
+            self.history.append(flying)
+            flying = ahead if ahead.entries else None
+            limit -= 1
+            assert limit > 0, "the scheduler does not terminate"
+
+
+def test_a_step_is_planned_ahead_only_when_it_cannot_depend_on_the_last():
+    c = manager(pages=64, page_size=4, slots=4, max_seq=128)
+    s = Scheduler(c, max_batched_tokens=16, chunk_size=7)
+    a = s.add(list(range(5)), 4)
+    b = s.add(list(range(9)), 6)
+    d = AheadDriver(s)
+    p = s.plan()                                     # a whole, b's first portion
+    d.feed(p)
+    assert s.plan_ahead().entries == []              # a portion of a prompt is in the step
+    s.commit(p, {0: 7})
+    p = s.plan()                                     # a decodes, b's last two tokens
+    d.feed(p)
+    assert s.plan_ahead().entries == []
+    s.commit(p, {0: 7, 1: 7})
+    p = s.plan()                                     # both decode: a has 2 of 4, b 1 of 6
+    assert [(e.request.number, e.start, e.n_tokens) for e in p.entries] == [(0, 6, 1), (1, 9, 1)]
+    d.feed(p)
+    late = s.add([1, 2, 3], 2)
+    assert s.plan_ahead().entries == []              # somebody waits: the next step may admit them
+    s.abort(late)
+    ahead = s.plan_ahead()
+    assert [(e.request.number, e.start, e.n_tokens, e.sample) for e in ahead.entries] == [(0, 7, 1, True), (1, 10, 1, True)]
+    d.feed(ahead)
+    with pytest.raises(SchedulerError):
+        s.plan()                                     # not while a step planned ahead waits
+    s.commit(p, {0: 7, 1: 7})                        # a: 3 of 4, b: 2 of 6
+    assert s.plan_ahead().entries == []              # the step in flight gives a its last token: it ends there
+    assert s.commit(ahead, {0: 7, 1: 7}) == [a]
+    assert a.generated == [7] * 4 and b.generated == [7] * 3 and b.n_fed == 11
+    c.release(a.key)
+    d.run()
+    assert b.generated == [7] * 6 and not c.live_requests() and c.num_free_pages() == 64
+
+
+def test_a_request_ended_by_the_last_step_is_dropped_from_the_step_planned_ahead():
+    c = manager(pages=64, slots=2, max_seq=128)
+    s = Scheduler(c)
+    streams = {0: iter([5, 6, 99, 1, 2, 3, 4, 5, 6, 7]), 1: iter(range(100, 120))}
+    r = s.add([1, 2, 3], 10, eos_token_ids=(99,))
+    q = s.add([4, 5], 6, eos_token_ids=(99,))
+    d = AheadDriver(s, lambda req: next(streams[req.number]))
+    d.run()
+    assert r.generated == [5, 6] and r.finish_reason == "eos"
+    assert q.generated == list(range(100, 106)) and q.finish_reason == "length"
+    assert d.ahead_steps >= 3 and d.wasted_rows == 1           # r ran one token behind its last
+    assert not c.live_requests() and c.num_free_pages() == 64
+
+
+def test_no_step_is_planned_ahead_without_pages_for_it():
+    c = manager(groups=((FULL, 1),), pages=4, page_size=4, slots=2, max_seq=16)
+    s = Scheduler(c, chunk_size=64, max_batched_tokens=64)
+    a = s.add(list(range(6)), 10)
+    d = AheadDriver(s)
+    p = s.plan()
+    d.feed(p)
+    s.commit(p, {0: 7})
+    p = s.plan()                                     # token 7 of 16: 2 pages held, 2 free
+    d.feed(p)
+    c.admit("squatter")
+    c.reserve("squatter", 8)                         # takes the two free pages
+    assert c.num_free_pages() == 0
+    assert [e.start for e in s.plan_ahead().entries] == [7]     # position 7 lies in a page a holds
+    s.commit(p, {0: 7})
+    s.commit(None, {0: 7})
+    p = s.plan_ahead()                               # position 8 needs a page
+    assert p.entries == []
+    c.release("squatter")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_steps_planned_ahead_change_no_token(seed):
+    rng = random.Random(seed)
+    c = manager(groups=((FULL, 1), (WIN, 1)), pages=24, page_size=4, slots=3, max_seq=64)
+    s = Scheduler(c, max_batched_tokens=rng.choice([8, 16, 40]), chunk_size=rng.choice([3, 7, 32]))
+    eos = 999
+    reqs = [s.add([rng.randrange(50) for _ in range(rng.randrange(1, 30))], rng.randrange(1, 20), eos_token_ids=(eos,))
+            for _ in range(12)]
+    stops = {r.number: rng.choice([None, rng.randrange(0, 12)]) for r in reqs}
+
+    def token(req):
+        return eos if stops[req.number] == len(req.generated) else req.number * 1000 + len(req.generated)
+
+    d = AheadDriver(s, token)
+    d.run()
+    for r in reqs:
+        n = r.max_new_tokens if stops[r.number] is None else min(r.max_new_tokens, stops[r.number])
+        assert r.generated == [r.number * 1000 + i for i in range(n)]
+        assert r.finish_reason == ("eos" if n < r.max_new_tokens else "length")
+    assert not c.live_requests() and all(g.pool.num_free == 24 for _, g in c.paged_groups())
+    assert d.ahead_steps > 0
+
+
 def test_random_stream_is_keyed_by_seed_request_and_count():
     u = uniform(42, 3, 5)
     assert u == uniform(42, 3, 5) and 0.0 <= u < 1.0

@@ -173,6 +173,88 @@ def test_only_the_most_recent_step_shapes_keep_their_graphs(model_folders, monke
     assert len(captured) == 2
 
 
+@pytest.mark.parametrize("graph", [False, True])
+def test_a_step_takes_its_tokens_from_the_device(model_folders, graph):
+    """A step may name its tokens by rows of the sampler's last call instead of ids: it is then
+    launched before those ids are read.  Same logits bit for bit as the step that was given the
+    ids, with the rows in another order than the entries, step after step."""
+    import tinyinfer_amd as ti
+    from tinyinfer_amd.engine import EngineError
+    from tinyinfer_amd.sampling import Sampler, SamplingParams
+    d = model_folders("D", "bfloat16", True)
+    make = lambda: ti.Engine.from_folder(d, "bfloat16", page_size=16, max_tokens=384, max_requests=3, max_seq=128)
+    e1, e2 = make(), make()
+    assert e2.feedback_rows == 3
+    s1, s2 = Sampler(e1.ops), Sampler(e2.ops)
+    prompts = {"x": random_tokens(30, 333, 1), "y": random_tokens(9, 333, 2), "z": random_tokens(17, 333, 3)}
+    names = ["x", "y", "z"]
+    first = [ti.StepEntry(r, prompts[r], [len(prompts[r]) - 1]) for r in names]
+    params = [SamplingParams(), SamplingParams(0.9, 5, 0.95, 11), SamplingParams()]
+    run = lambda e, entries: e.step_graph(entries) if graph else e.step(entries)
+    ids = s1.sample(e1.step(first), params, [0, 1, 2], [0, 0, 0])
+    ticket = s2.sample_async(e2.step(first), params, [0, 1, 2], [0, 0, 0], feed=e2)
+    history = [ids]
+    for i in range(1, 24):
+        order = [2, 0, 1] if i % 2 else [1, 2, 0]              # entries in another order than the sampler's rows
+        a = run(e1, [ti.StepEntry(names[k], [ids[k]], [0]) for k in order])
+        b = run(e2, [ti.StepEntry(names[k], [ti.token_from_feedback(k)], [0]) for k in order])
+        back = [order.index(k) for k in range(3)]              # row of request k in this step's logits
+        a = a[back].contiguous()
+        b_rows = b[back].contiguous()
+        ids = s1.sample(a, params, [0, 1, 2], [i] * 3)
+        late = s2.collect(ticket)                               # the ids of the step before, read after this step's launch
+        assert late == history[-1], i
+        assert torch.equal(a, b_rows), i
+        ticket = s2.sample_async(b_rows, params, [0, 1, 2], [i] * 3, feed=e2)
+        history.append(ids)
+    assert s2.collect(ticket) == ids
+    with pytest.raises(EngineError, match="feedback"):
+        e2.step([ti.StepEntry("x", [ti.token_from_feedback(3)], [0])])
+    e2.cache.check()
+
+
+@pytest.mark.parametrize("dtype,graph", [("float32", False), ("float32", True), ("bfloat16", True)])
+def test_steps_launched_ahead_change_no_token(model_folders, dtype, graph):
+    """While every running request decodes, `run_requests` launches the next step before it has
+    read the last one's ids.  Nothing that is generated changes: requests of different lengths,
+    prompts in portions, temperature beside greedy, requests that an end-of-generation id stops in
+    the middle (their row in the step launched ahead runs for nothing), a callback per token."""
+    import tinyinfer_amd as ti
+    from tinyinfer_amd.api import run_requests
+    d = model_folders("D", "bfloat16", True)
+    prompts = [random_tokens(n, 333, 90 + n) for n in (21, 3, 50, 8)]
+    budgets = [40, 17, 28, 40]
+    sampling = [ti.SamplingParams(), ti.SamplingParams(0.8, 20, 0.9, 7), ti.SamplingParams(), ti.SamplingParams(1.1, 0, 1.0, 3)]
+
+    def run(ahead, eos):
+        engine = ti.Engine.from_folder(d, dtype, page_size=16, max_tokens=512, max_requests=4, max_seq=128)
+        sched = ti.Scheduler(engine.cache, max_batched_tokens=24, chunk_size=16)
+        reqs = [sched.add(p, n, sp, eos) for p, n, sp in zip(prompts, budgets, sampling)]
+        heard = {r.number: [] for r in reqs}
+        stats = ti.GenerationStats()
+        run_requests(engine, sched, stats=stats, on_token=lambda r, t: heard[r.number].append(t), use_graph=graph,
+                     run_ahead=ahead)
+        assert all(heard[r.number] == list(r.generated) for r in reqs)
+        assert not engine.cache.live_requests()
+        engine.cache.check()
+        return [list(r.generated) for r in reqs], [r.finish_reason for r in reqs], stats
+
+    plain_run, reasons, st0 = run(False, [])
+    ahead_run, reasons1, st1 = run(True, [])
+    assert ahead_run == plain_run and reasons1 == reasons == ["length"] * 4
+    assert [len(g) for g in plain_run] == budgets
+    assert st1.steps == st0.steps and st1.decode_tokens == st0.decode_tokens
+    assert st0.steps_ahead == 0 and st1.steps_ahead >= 10
+    if dtype == "float32":
+        # ids that stop the first and the third request in the middle, at different steps
+        eos = [plain_run[0][25], plain_run[2][11]]
+        cut, why, st2 = run(False, eos)
+        cut1, why1, st3 = run(True, eos)
+        assert cut1 == cut and why1 == why and why.count("eos") >= 2
+        assert st3.decode_tokens >= st2.decode_tokens           # rows that ran for nothing are counted
+        assert st3.steps_ahead >= 10
+
+
 def test_preemption_recomputes_and_changes_nothing(model_folders):
     """With too few pages the youngest request gives way and is fed again later;
     in 32-bit the tokens are the ones a roomy pool gives."""

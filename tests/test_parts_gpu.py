@@ -414,6 +414,12 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     assert engine.cache.slot("c") == 0                      # the slot a held
     for r in reqs:
         assert np.abs(np.concatenate(got[r]) - want[r]).max() < 2e-4, r
+    # parts from outside the library read token ids only: such an engine offers no token feedback,
+    # and a token that names a row of it is refused like any id outside the vocabulary
+    from tinyinfer_amd.engine import EngineError
+    assert engine.feedback_rows == 0
+    with pytest.raises(EngineError, match="outside the vocabulary"):
+        engine.step([ti.StepEntry("c", [ti.token_from_feedback(0)], [0])])
 
 
 def test_toy_mixer_with_pages_of_its_own(tmp_path):

@@ -9,12 +9,12 @@ from .registry import register_architecture, registered_architectures, config_an
 from .parts.registry import register_part, build_part
 from . import parts as _parts          # noqa: F401  registers the built-in parts
 from .models import Model, ModelSpec, LayerSpec, PartSpec
-from .engine import Engine, StepEntry
+from .engine import Engine, StepEntry, token_from_feedback
 from .engine.scheduler import Scheduler, Request
 from .sampling import SamplingParams
 from .api import LLM, generate_ids, GenerationStats
 
 __all__ = ["ConfigError", "read_config_json", "Qwen3Config", "register_architecture",
            "registered_architectures", "config_and_spec", "register_part", "build_part",
-           "Model", "ModelSpec", "LayerSpec", "PartSpec", "Engine", "StepEntry", "Scheduler", "Request",
+           "Model", "ModelSpec", "LayerSpec", "PartSpec", "Engine", "StepEntry", "token_from_feedback", "Scheduler", "Request",
            "SamplingParams", "LLM", "generate_ids", "GenerationStats"]

@@ -30,13 +30,17 @@ class GenerationStats:
     decode_tokens: int = 0
     steps: int = 0
     preemptions: int = 0
+    steps_ahead: int = 0             # of `steps`: launched before the ids of the step before were read
 
 
 def run_requests(engine: Engine, scheduler: Scheduler, sampler: Optional[Sampler] = None,
-                 stats: Optional[GenerationStats] = None, on_token=None, use_graph: bool = False) -> None:
+                 stats: Optional[GenerationStats] = None, on_token=None, use_graph: bool = False,
+                 run_ahead: bool = True) -> None:
     """Run until the scheduler has no work.  `on_token(request, token)` is called for every
     generated token.  When a step fails, every request the scheduler still holds is given back
-    to the cache before the error is raised."""
+    to the cache before the error is raised.  `run_ahead`: while every running request decodes
+    and nobody waits, the next step is launched before the last one's ids are read (it takes
+    them from the device); the tokens are the same, `on_token` hears them a step later."""
     native.ensure_kernels(["sampling"])
     raised = []
 
@@ -51,7 +55,7 @@ def run_requests(engine: Engine, scheduler: Scheduler, sampler: Optional[Sampler
     callback = native.ON_TOKEN(relay) if on_token else ctypes_null(native.ON_TOKEN)
     try:
         out = native.text("ti_run_requests", engine._ptr, scheduler._ptr, sampler._ptr if sampler else None,
-                          int(use_graph), callback)
+                          int(use_graph), int(run_ahead), callback)
     except native.EngineError:
         if raised:
             raise raised[0] from None
@@ -66,6 +70,7 @@ def run_requests(engine: Engine, scheduler: Scheduler, sampler: Optional[Sampler
         stats.decode_tokens += d["decode_tokens"]
         stats.steps += d["steps"]
         stats.preemptions += d["preemptions"]
+        stats.steps_ahead += d["steps_ahead"]
 
 
 def ctypes_null(kind):
@@ -77,14 +82,14 @@ def generate_ids(engine: Engine, prompts: Sequence[Sequence[int]], max_new_token
                  temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0, seed: int = 42,
                  eos_token_ids: Optional[Sequence[int]] = None, chunk_size: int = 512,
                  max_batched_tokens: int = 2048, use_graph: bool = False,
-                 stats: Optional[GenerationStats] = None) -> List[List[int]]:
+                 stats: Optional[GenerationStats] = None, run_ahead: bool = True) -> List[List[int]]:
     """Generated token ids for each prompt (the prompt itself is not repeated)."""
     if eos_token_ids is None:
         eos_token_ids = engine.model.spec.eos_token_ids
     scheduler = Scheduler(engine.cache, max_batched_tokens=max_batched_tokens, chunk_size=chunk_size)
     params = SamplingParams(float(temperature), int(top_k), float(top_p), int(seed))
     requests: List[Request] = [scheduler.add(p, max_new_tokens, params, eos_token_ids) for p in prompts]
-    run_requests(engine, scheduler, stats=stats, use_graph=use_graph)
+    run_requests(engine, scheduler, stats=stats, use_graph=use_graph, run_ahead=run_ahead)
     return [list(r.generated) for r in requests]
 
 

@@ -9,12 +9,15 @@
 TI_ERROR_API
 
 // ------------------------------------------------------------------ embedding
-// x[m, :] = float(E[tok[m], :])
+// x[m, :] = float(E[t, :]) with t = tok[m], or, where tok[m] is below zero, t = fed[-1 - tok[m]]:
+// an id that an earlier kernel on the stream (the sampler) left on the device, so that the host
+// can launch a step before it has read the step before.
 template <typename T>
-__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tok,
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tok, const int* __restrict__ fed, int n_fed,
                              float* __restrict__ x, int H, int V) {
   const int m = blockIdx.x;
-  const int t = tok[m];
+  int t = tok[m];
+  if (t < 0 && fed && -1 - t < n_fed) t = fed[-1 - t];
   float* row = x + (size_t)m * H;
   if (t < 0 || t >= V) {   // the host refuses such ids; never read out of bounds
     for (int i = threadIdx.x; i < H; i += blockDim.x) row[i] = 0.f;
@@ -24,18 +27,23 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
   for (int i = threadIdx.x; i < H; i += blockDim.x) row[i] = ld<T>(src + i);
 }
 
-extern "C" int ti_embed(int dtype, const void* table, const int* tok, float* x, int M, int H, int V,
-                        hipStream_t stream) {
-  TI_REQUIRE(M >= 0 && H > 0 && V > 0, "embed: bad sizes M=%d H=%d V=%d", M, H, V);
+extern "C" int ti_embed_fed(int dtype, const void* table, const int* tok, const int* fed, int n_fed, float* x, int M, int H,
+                            int V, hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && H > 0 && V > 0 && n_fed >= 0, "embed: bad sizes M=%d H=%d V=%d n_fed=%d", M, H, V, n_fed);
   if (M == 0) return 0;
   if (dtype == TI_F32)
-    embed_kernel<float><<<M, 256, 0, stream>>>((const float*)table, tok, x, H, V);
+    embed_kernel<float><<<M, 256, 0, stream>>>((const float*)table, tok, fed, n_fed, x, H, V);
   else if (dtype == TI_BF16)
-    embed_kernel<bf16_t><<<M, 256, 0, stream>>>((const bf16_t*)table, tok, x, H, V);
+    embed_kernel<bf16_t><<<M, 256, 0, stream>>>((const bf16_t*)table, tok, fed, n_fed, x, H, V);
   else
     TI_REQUIRE(false, "embed: unknown dtype %d", dtype);
   TI_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int ti_embed(int dtype, const void* table, const int* tok, float* x, int M, int H, int V,
+                        hipStream_t stream) {
+  return ti_embed_fed(dtype, table, tok, nullptr, 0, x, M, H, V, stream);
 }
 
 // -------------------------------------------------------------------- RMSNorm

@@ -22,6 +22,9 @@ extern "C" {
 
 // ---- libti_core: embedding, norms, rotation, cache write (templated on the storage dtype)
 int ti_embed(int dtype, const void* table, const int* tok, float* x, int M, int H, int V, hipStream_t stream);
+// the same; a token below zero stands for fed[-1 - token], an id an earlier kernel on the stream left (fed may be null)
+int ti_embed_fed(int dtype, const void* table, const int* tok, const int* fed, int n_fed, float* x, int M, int H, int V,
+                 hipStream_t stream);
 // out[r] = rmsnorm(x[rows ? rows[r] : r]) * w, in `out_dtype`
 int ti_rmsnorm(int out_dtype, const float* x, const float* w, const int* rows, void* out, int n_rows, int H, float eps,
                hipStream_t stream);

@@ -145,7 +145,7 @@ Workspace& workspace_of(Ops* ops) {
 
 struct SchedulerHandle {
   std::unique_ptr<Scheduler> s;
-  Plan last;
+  Plan last, ahead;          // `ahead`: planned behind `last` before `last` was committed; it is next to be committed
   std::map<int64_t, std::shared_ptr<Request>> all;
 };
 Json request_json(const Request& r) {
@@ -738,6 +738,7 @@ int ti_engine_info(void* engine, const char** out) {
   j.set("num_graphs", (int64_t)e.num_graphs());
   j.set("cache_bytes", (int64_t)e.cache_bytes());
   j.set("table_width", e.cache->table_width);
+  j.set("feedback_rows", e.feedback_rows());
   Json keys = Json::array();
   for (const auto& k : e.graph_keys()) keys.push(k);
   j.set("graphs", keys);
@@ -799,9 +800,8 @@ int ti_sampler_create(void* ops, void** out) {
   TI_END
 }
 void ti_sampler_release(void* sampler) { delete static_cast<Sampler*>(sampler); }
-int ti_sampler_sample(void* sampler, const ti_tensor* logits, int n, const float* temperature, const int* top_k,
-                      const float* top_p, const uint64_t* seeds, const int64_t* requests, const int64_t* counters, int* out) {
-  TI_BEGIN
+static std::vector<SamplingParams> sampling_params(int n, const float* temperature, const int* top_k, const float* top_p,
+                                                   const uint64_t* seeds) {
   std::vector<SamplingParams> params(n);
   for (int i = 0; i < n; ++i) {
     params[i].temperature = temperature[i];
@@ -809,8 +809,38 @@ int ti_sampler_sample(void* sampler, const ti_tensor* logits, int n, const float
     params[i].top_p = top_p[i];
     params[i].seed = seeds[i];
   }
-  const std::vector<int> ids = static_cast<Sampler*>(sampler)->sample(T(logits, 0), params, std::vector<int64_t>(requests, requests + n),
+  return params;
+}
+int ti_sampler_sample(void* sampler, const ti_tensor* logits, int n, const float* temperature, const int* top_k,
+                      const float* top_p, const uint64_t* seeds, const int64_t* requests, const int64_t* counters, int* out) {
+  TI_BEGIN
+  const std::vector<int> ids = static_cast<Sampler*>(sampler)->sample(T(logits, 0), sampling_params(n, temperature, top_k, top_p, seeds),
+                                                                      std::vector<int64_t>(requests, requests + n),
                                                                       std::vector<int64_t>(counters, counters + n));
+  memcpy(out, ids.data(), (size_t)n * 4);
+  TI_END
+}
+int ti_sampler_sample_async(void* sampler, const ti_tensor* logits, int n, const float* temperature, const int* top_k,
+                            const float* top_p, const uint64_t* seeds, const int64_t* requests, const int64_t* counters,
+                            void* feed_engine, uint64_t* out_ticket) {
+  TI_BEGIN
+  int* feed = nullptr;
+  if (feed_engine) {
+    Engine& e = *static_cast<Engine*>(feed_engine);
+    if (!e.token_feedback()) throw EngineError("this engine has no token feedback (its model has parts from outside the library)");
+    if (n > e.feedback_rows())
+      throw EngineError(std::to_string(n) + " rows of logits but the token feedback holds " + std::to_string(e.feedback_rows()));
+    feed = e.token_feedback();
+  }
+  *out_ticket = static_cast<Sampler*>(sampler)->sample_async(T(logits, 0), sampling_params(n, temperature, top_k, top_p, seeds),
+                                                             std::vector<int64_t>(requests, requests + n),
+                                                             std::vector<int64_t>(counters, counters + n), feed);
+  TI_END
+}
+int ti_sampler_collect(void* sampler, uint64_t ticket, int n, int* out) {
+  TI_BEGIN
+  const std::vector<int> ids = static_cast<Sampler*>(sampler)->collect(ticket);
+  if ((int)ids.size() != n) throw KernelError("sample: the call drew " + std::to_string(ids.size()) + " ids, not " + std::to_string(n));
   memcpy(out, ids.data(), (size_t)n * 4);
   TI_END
 }
@@ -837,13 +867,10 @@ int ti_scheduler_add(void* scheduler, int n_prompt, const int* prompt, int max_n
   *out_number = r->number;
   TI_END
 }
-int ti_scheduler_plan(void* scheduler, const char** out) {
-  TI_BEGIN
-  SchedulerHandle& h = *static_cast<SchedulerHandle*>(scheduler);
-  h.last = h.s->plan();
+static Json plan_json(const Plan& plan) {
   Json j = Json::object();
   Json es = Json::array();
-  for (const auto& e : h.last.entries) {
+  for (const auto& e : plan.entries) {
     Json r = Json::object();
     r.set("number", e.request->number);
     r.set("start", e.start);
@@ -853,9 +880,24 @@ int ti_scheduler_plan(void* scheduler, const char** out) {
   }
   j.set("entries", es);
   Json pre = Json::array();
-  for (const auto& r : h.last.preempted) pre.push(r->number);
+  for (const auto& r : plan.preempted) pre.push(r->number);
   j.set("preempted", pre);
-  return give(out, j.dump());
+  return j;
+}
+int ti_scheduler_plan(void* scheduler, const char** out) {
+  TI_BEGIN
+  SchedulerHandle& h = *static_cast<SchedulerHandle*>(scheduler);
+  if (!h.ahead.entries.empty()) throw SchedulerError("a step planned ahead waits to be committed");
+  h.last = h.s->plan();
+  return give(out, plan_json(h.last).dump());
+  TI_END
+}
+int ti_scheduler_plan_ahead(void* scheduler, const char** out) {
+  TI_BEGIN
+  SchedulerHandle& h = *static_cast<SchedulerHandle*>(scheduler);
+  if (!h.ahead.entries.empty()) throw SchedulerError("a step planned ahead waits to be committed");
+  h.ahead = h.s->plan_ahead(h.last);
+  return give(out, plan_json(h.ahead).dump());
   TI_END
 }
 int ti_scheduler_commit(void* scheduler, int n, const int64_t* numbers, const int* tokens, const char** out) {
@@ -865,6 +907,11 @@ int ti_scheduler_commit(void* scheduler, int n, const int64_t* numbers, const in
   for (int i = 0; i < n; ++i) sampled[numbers[i]] = tokens[i];
   Json done = Json::array();
   for (const auto& r : h.s->commit(h.last, sampled)) done.push(r->number);
+  // what was planned ahead is the next to be committed, without the requests that have just ended
+  h.last = Plan();
+  for (const auto& e : h.ahead.entries)
+    if (e.request->finish_reason.empty()) h.last.entries.push_back(e);
+  h.ahead = Plan();
   return give(out, done.dump());
   TI_END
 }
@@ -907,7 +954,7 @@ int ti_scheduler_request(void* scheduler, int64_t number, const char** out) {
   return give(out, request_json(*it->second).dump());
   TI_END
 }
-int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph, int (*on_token)(int64_t, int),
+int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph, int run_ahead, int (*on_token)(int64_t, int),
                     const char** out_stats) {
   TI_BEGIN
   SchedulerHandle& h = *static_cast<SchedulerHandle*>(scheduler);
@@ -917,7 +964,7 @@ int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph,
     cb = [on_token](const Request& r, int tok) {
       if (on_token(r.number, tok) != 0) throw EngineError("the token callback stopped the run");
     };
-  run_requests(*static_cast<Engine*>(engine), *h.s, static_cast<Sampler*>(sampler), &st, cb, use_graph != 0);
+  run_requests(*static_cast<Engine*>(engine), *h.s, static_cast<Sampler*>(sampler), &st, cb, use_graph != 0, run_ahead != 0);
   Json j = Json::object();
   j.set("prefill_ms", st.prefill_ms);
   j.set("prefill_tokens", st.prefill_tokens);
@@ -925,6 +972,7 @@ int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph,
   j.set("decode_tokens", st.decode_tokens);
   j.set("steps", st.steps);
   j.set("preemptions", st.preemptions);
+  j.set("steps_ahead", st.steps_ahead);
   return give(out_stats, j.dump());
   TI_END
 }

@@ -80,6 +80,11 @@ struct Engine::Impl {
   std::map<std::string, int> shapes_seen;
   bool foreign = false;
   size_t max_step_graphs = 32;
+  DeviceBuffer feedback;                    // int32 [max_requests]: ids a sampler left for the next step
+  int feedback_rows = 0;
+
+  // a token is an id of the vocabulary, or names a row of the feedback buffer
+  bool token_ok(int t, int64_t V) const { return t >= 0 ? t < V : -1 - t < feedback_rows; }
 
   explicit Impl(Engine& e) : e(e) {}
   ~Impl() {
@@ -128,7 +133,7 @@ struct Engine::Impl {
     reqs.reserve(entries.size());
     for (const auto& en : entries) {
       if (en.tokens.size() != 1 || !c.has(en.request) || c.reserved(en.request) != c.length(en.request)) return false;
-      if (en.tokens[0] < 0 || en.tokens[0] >= V) return false;           // the general path names the token
+      if (!token_ok(en.tokens[0], V)) return false;                      // the general path names the token
       for (int w : en.want)
         if (w != 0) return false;
       if (en.start >= 0 && en.start != c.length(en.request)) return false;
@@ -162,9 +167,10 @@ struct Engine::Impl {
         if (!seen.insert(en.request).second) throw EngineError("request " + name + " appears twice in one step");
         if (en.tokens.empty()) throw EngineError("request " + name + ": an entry needs at least one token");
         for (int t : en.tokens)
-          if (t < 0 || t >= V)
+          if (!token_ok(t, V))
             throw EngineError("request " + name + ": token id " + std::to_string(t) + " is outside the vocabulary [0, " +
-                              std::to_string(V) + ")");
+                              std::to_string(V) + ")" +
+                              (t < 0 && feedback_rows ? " and names no row of the token feedback (" + std::to_string(feedback_rows) + " rows)" : ""));
         for (int w : en.want)
           if (w < 0 || w >= (int)en.tokens.size())
             throw EngineError("request " + name + ": wanted place " + std::to_string(w) + " is outside its " +
@@ -291,6 +297,8 @@ struct Engine::Impl {
 
     ctx.meta_dev = dev;
     ctx.tokens = dev + o_tok;
+    ctx.fed_tokens = (const int*)feedback.data();
+    ctx.n_fed_tokens = feedback_rows;
     ctx.positions = dev + o_pos;
     ctx.slots = dev + o_slot;
     ctx.out_rows = n_want ? dev + o_out : nullptr;
@@ -548,6 +556,11 @@ Engine::Engine(std::shared_ptr<Model> model_, const EngineOptions& o)
     p.prepare(ops, max_seq);          // tables that depend on the longest sequence
   });
   impl_->foreign = model->has_foreign_parts();
+  if (!impl_->foreign) {
+    impl_->feedback_rows = cache->max_requests;
+    impl_->feedback = DeviceBuffer((size_t)impl_->feedback_rows * 4);
+    ops.fill_zero(impl_->feedback.data(), (size_t)impl_->feedback_rows * 4);
+  }
   synchronize();
 }
 
@@ -556,6 +569,8 @@ Engine::~Engine() {}
 Tensor Engine::step(const std::vector<StepEntry>& entries) { return impl_->step(entries); }
 Tensor Engine::step_graph(const std::vector<StepEntry>& entries) { return impl_->step_graph(entries); }
 void Engine::release(int64_t request) { cache->release(request); }
+int* Engine::token_feedback() { return (int*)impl_->feedback.data(); }
+int Engine::feedback_rows() const { return impl_->feedback_rows; }
 void Engine::synchronize() { hip_check(hipStreamSynchronize(impl_->stream), "hipStreamSynchronize"); }
 void Engine::logits_to_host(const Tensor& logits, float* out) {
   if (!logits.defined()) return;

@@ -24,6 +24,13 @@ from ..ops.kernels import Ops, required_libraries
 from ..weights.loader import DTYPES, load_weights
 
 
+def token_from_feedback(row: int) -> int:
+    """In place of a token id: the id that the sampler's last call with `feed=engine` wrote to row
+    `row` of the engine's token feedback.  The step then needs no id that the host has not read yet,
+    so it can be launched before the step before it has finished."""
+    return -1 - int(row)
+
+
 @dataclass
 class StepEntry:
     """The next tokens of one request, and the places among them (0-based) whose
@@ -61,6 +68,7 @@ class Engine:
         info = self.info()
         self.page_size, self.max_seq, self.num_pages = info["page_size"], info["max_seq"], info["num_pages"]
         self.table_width = info["table_width"]
+        self.feedback_rows = info["feedback_rows"]     # 0: no token feedback (a model with parts from outside the library)
         self.cache = CacheManager(_borrowed=native.pointer("ti_engine_cache", self._ptr), _owner=self)
         self.ops = Ops(_borrowed=native.pointer("ti_engine_ops", self._ptr))
 

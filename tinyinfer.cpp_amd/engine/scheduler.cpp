@@ -150,6 +150,35 @@ Plan Scheduler::plan() {
   return plan;
 }
 
+// The step after `last`, planned before `last`'s tokens are known: possible when `last` decodes
+// one token of every running request, nobody waits, none of them ends with `last`'s token by its
+// length, and the pages for one more token each are free.  Every request then decodes one more
+// token, whatever `last` samples; the ids come from the device (token_from_feedback).  A request
+// that `last`'s token ends (an end-of-generation id) has run one token for nothing.  An empty plan
+// if any of this does not hold.  Call it after `last` has been launched and before it is committed.
+Plan Scheduler::plan_ahead(const Plan& last) const {
+  Plan ahead;
+  if (last.entries.empty() || !waiting.empty() || last.entries.size() != running.size()) return ahead;
+  std::vector<std::pair<std::shared_ptr<Request>, int>> batch;
+  for (const auto& e : last.entries) {
+    const Request& r = *e.request;
+    if (e.n_tokens != 1 || !e.sample || !r.finish_reason.empty()) return ahead;
+    if (std::find(running.begin(), running.end(), e.request) == running.end()) return ahead;
+    if ((int)r.generated.size() + 1 >= r.max_new_tokens) return ahead;
+    batch.emplace_back(e.request, 2);           // n_fed does not count `last`'s token yet
+  }
+  if (new_pages(batch) > 0) return ahead;
+  for (const auto& e : last.entries) {
+    PlannedEntry a;
+    a.request = e.request;
+    a.start = e.start + 1;
+    a.n_tokens = 1;
+    a.sample = true;
+    ahead.entries.push_back(a);
+  }
+  return ahead;
+}
+
 std::vector<std::shared_ptr<Request>> Scheduler::commit(const Plan& plan, const std::map<int64_t, int>& sampled) {
   std::vector<std::shared_ptr<Request>> done;
   for (const auto& e : plan.entries) {
@@ -196,7 +225,7 @@ void Scheduler::abort_all() {
 
 // The loop of /root/reference/src/main.cpp:210-297 with admission, portions and preemption added.
 void run_requests(Engine& engine, Scheduler& scheduler, Sampler* sampler, GenerationStats* stats,
-                  const std::function<void(const Request&, int)>& on_token, bool use_graph) {
+                  const std::function<void(const Request&, int)>& on_token, bool use_graph, bool run_ahead) {
   std::unique_ptr<Sampler> own;
   if (!sampler) {
     own.reset(new Sampler(engine.ops));
@@ -204,60 +233,117 @@ void run_requests(Engine& engine, Scheduler& scheduler, Sampler* sampler, Genera
   }
   GenerationStats local;
   GenerationStats& st = stats ? *stats : local;
-  try {
-    while (scheduler.has_work()) {
-      Plan plan = scheduler.plan();
-      st.preemptions += (int64_t)plan.preempted.size();
-      std::vector<StepEntry> entries;
-      entries.reserve(plan.entries.size());
-      bool decode_only = true;
-      int64_t n_tok = 0;
-      for (const auto& e : plan.entries) {
-        StepEntry se;
-        se.request = e.request->key();
+  // A step that has been launched and not yet read.
+  struct Launched {
+    Plan plan;
+    std::vector<std::shared_ptr<Request>> asked;     // row i of the sampler's call
+    uint64_t ticket = 0;
+    bool sampled = false, decode_only = true;
+    int64_t n_tok = 0;
+  };
+  int* feedback = run_ahead ? engine.token_feedback() : nullptr;
+  std::unique_ptr<Launched> flying, next;
+
+  // `before`: the step whose ids this one takes from the device (null: it has every id on the host)
+  auto launch = [&](Plan plan, const Launched* before) {
+    std::unique_ptr<Launched> f(new Launched());
+    std::map<int64_t, int> row_before;
+    if (before)
+      for (size_t i = 0; i < before->asked.size(); ++i) row_before[before->asked[i]->number] = (int)i;
+    std::vector<StepEntry> entries;
+    entries.reserve(plan.entries.size());
+    for (const auto& e : plan.entries) {
+      StepEntry se;
+      se.request = e.request->key();
+      if (before)
+        se.tokens.assign(1, token_from_feedback(row_before.at(e.request->number)));
+      else
         se.tokens.assign(e.request->tokens.begin() + e.start, e.request->tokens.begin() + e.start + e.n_tokens);
-        if (e.sample) se.want.push_back(e.n_tokens - 1);
-        se.start = e.start;
-        entries.push_back(std::move(se));
-        decode_only = decode_only && e.n_tokens == 1;
-        n_tok += e.n_tokens;
+      if (e.sample) se.want.push_back(e.n_tokens - 1);
+      se.start = e.start;
+      entries.push_back(std::move(se));
+      f->decode_only = f->decode_only && e.n_tokens == 1;
+      f->n_tok += e.n_tokens;
+      if (e.sample) f->asked.push_back(e.request);
+    }
+    Tensor logits = use_graph ? engine.step_graph(entries) : engine.step(entries);
+    if (!f->asked.empty()) {
+      std::vector<SamplingParams> params;
+      std::vector<int64_t> numbers, counters;
+      for (const auto& r : f->asked) {
+        params.push_back(r->params);
+        numbers.push_back(r->number);
+        counters.push_back((int64_t)r->generated.size() + (before ? 1 : 0));
       }
-      const auto t0 = std::chrono::steady_clock::now();
-      Tensor logits = use_graph ? engine.step_graph(entries) : engine.step(entries);
-      std::vector<std::shared_ptr<Request>> asked;
-      for (const auto& e : plan.entries)
-        if (e.sample) asked.push_back(e.request);
-      std::map<int64_t, int> sampled;
-      if (!asked.empty()) {
-        std::vector<SamplingParams> params;
-        std::vector<int64_t> numbers, counters;
-        for (const auto& r : asked) {
-          params.push_back(r->params);
-          numbers.push_back(r->number);
-          counters.push_back((int64_t)r->generated.size());
+      const bool feed = feedback && (int)f->asked.size() <= engine.feedback_rows();
+      f->ticket = sampler->sample_async(logits, params, numbers, counters, feed ? feedback : nullptr);
+      f->sampled = true;
+    }
+    f->plan = std::move(plan);
+    return f;
+  };
+
+  auto t_mark = std::chrono::steady_clock::now();
+  // read the step's ids, commit them, give back what ended
+  auto settle = [&](Launched& f) {
+    std::map<int64_t, int> sampled;
+    if (f.sampled) {
+      f.sampled = false;
+      const std::vector<int> toks = sampler->collect(f.ticket);
+      for (size_t i = 0; i < f.asked.size(); ++i) sampled[f.asked[i]->number] = toks[i];
+    } else {
+      engine.synchronize();
+    }
+    const auto now = std::chrono::steady_clock::now();
+    const double ms = std::chrono::duration<double, std::milli>(now - t_mark).count();
+    t_mark = now;
+    if (f.decode_only) {
+      st.decode_ms += ms;
+      st.decode_tokens += f.n_tok;
+    } else {
+      st.prefill_ms += ms;
+      st.prefill_tokens += f.n_tok;
+    }
+    st.steps += 1;
+    // a step launched ahead may hold requests that the step before it ended: their row ran for nothing
+    Plan live;
+    live.preempted = f.plan.preempted;
+    for (const auto& e : f.plan.entries)
+      if (e.request->finish_reason.empty()) live.entries.push_back(e);
+    std::map<int64_t, size_t> had;
+    for (const auto& e : live.entries) had[e.request->number] = e.request->generated.size();
+    for (const auto& done : scheduler.commit(live, sampled)) engine.release(done->key());
+    if (on_token)
+      for (const auto& e : live.entries)
+        if (e.sample && e.request->generated.size() > had[e.request->number]) on_token(*e.request, e.request->generated.back());
+  };
+
+  try {
+    while (flying || scheduler.has_work()) {
+      if (!flying) {
+        Plan plan = scheduler.plan();
+        st.preemptions += (int64_t)plan.preempted.size();
+        flying = launch(std::move(plan), nullptr);
+      }
+      // while the device works on that step: the next one, if it needs nothing the step decides
+      if (feedback && flying->sampled && (int)flying->asked.size() <= engine.feedback_rows()) {
+        Plan ahead = scheduler.plan_ahead(flying->plan);
+        if (!ahead.entries.empty()) {
+          try {
+            next = launch(std::move(ahead), flying.get());
+            st.steps_ahead += 1;
+          } catch (const OutOfPages&) {
+            next.reset();                    // the step has taken nothing: decided again once this one is read
+          }
         }
-        const std::vector<int> toks = sampler->sample(logits, params, numbers, counters);
-        for (size_t i = 0; i < asked.size(); ++i) sampled[asked[i]->number] = toks[i];
-      } else {
-        engine.synchronize();
       }
-      const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
-      if (decode_only) {
-        st.decode_ms += ms;
-        st.decode_tokens += n_tok;
-      } else {
-        st.prefill_ms += ms;
-        st.prefill_tokens += n_tok;
-      }
-      st.steps += 1;
-      std::map<int64_t, size_t> before;
-      for (const auto& r : asked) before[r->number] = r->generated.size();
-      for (const auto& done : scheduler.commit(plan, sampled)) engine.release(done->key());
-      if (on_token)
-        for (const auto& r : asked)
-          if (r->generated.size() > before[r->number]) on_token(*r, r->generated.back());
+      settle(*flying);
+      flying = std::move(next);
+      next.reset();
     }
   } catch (...) {
+    for (auto* f : {flying.get(), next.get()})
+      if (f && f->sampled) sampler->drop(f->ticket);
     // whatever the scheduler still holds goes back to the cache: the next call starts clean
     scheduler.abort_all();
     throw;
@@ -272,7 +358,7 @@ std::vector<std::vector<int>> generate(Engine& engine, const std::vector<std::ve
   Scheduler scheduler(*engine.cache, o.max_batched_tokens, o.chunk_size);
   std::vector<std::shared_ptr<Request>> requests;
   for (const auto& p : prompts) requests.push_back(scheduler.add(p, o.max_new_tokens, o.sampling, eos));
-  run_requests(engine, scheduler, nullptr, stats, nullptr, o.use_graph);
+  run_requests(engine, scheduler, nullptr, stats, nullptr, o.use_graph, o.run_ahead);
   std::vector<std::vector<int>> out;
   for (const auto& r : requests) out.push_back(r->generated);
   return out;

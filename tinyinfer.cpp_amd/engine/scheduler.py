@@ -112,6 +112,16 @@ class Scheduler:
         return Plan([PlannedEntry(self._requests[e["number"]], e["start"], e["n_tokens"], e["sample"]) for e in d["entries"]],
                     [self._requests[n] for n in d["preempted"]])
 
+    def plan_ahead(self) -> Plan:
+        """The step behind the last `plan()` (or `plan_ahead()`), before that one is committed: one
+        more token of every running request, if all of them decode, nobody waits, none ends with the
+        last step's token by its length and the pages are free; else an empty plan.  The next
+        `commit` is for the earlier plan, the one after it for this one (without the requests that
+        the earlier one ended)."""
+        d = json.loads(native.text("ti_scheduler_plan_ahead", self._ptr))
+        return Plan([PlannedEntry(self._requests[e["number"]], e["start"], e["n_tokens"], e["sample"]) for e in d["entries"]],
+                    [])
+
     def commit(self, plan: Plan, sampled: Dict[int, int]) -> List[Request]:
         """The step of the last `plan()` ran.  `sampled[request.number]` is the token drawn for every
         entry that asked for one.  Returns the requests that finished; their pages and slots are to be

@@ -263,7 +263,8 @@ class Ops {
   void set_stream(void* s) { flush(); stream_ = s; }
   int compute_units();
 
-  void embed(const Tensor& table, const int* tokens, int64_t M, const Tensor& x);
+  // a token below zero stands for fed[-1 - token] (device memory, n_fed ids; may be null)
+  void embed(const Tensor& table, const int* tokens, int64_t M, const Tensor& x, const int* fed = nullptr, int n_fed = 0);
   // out[r] = rmsnorm(x[rows ? rows[r] : r]) * w
   void rmsnorm(const Tensor& x, const Tensor& w, float eps, const Tensor& out, const int* rows = nullptr, int64_t n_rows = 0);
   void rope_neox(const Tensor& x, const int* positions, const Tensor& inv_freq);      // in place on f32 [M, heads, hd]
@@ -374,9 +375,13 @@ struct AttentionWork {
 };
 
 // ---------------------------------------------------------------------------------- the step
+// In place of a token id: the id that the sampler's last call wrote to row `row` of the engine's
+// token feedback buffer (Engine::token_feedback).  The step then needs no id that the host has not
+// read yet, so it can be launched before the step before it has finished.
+inline int token_from_feedback(int row) { return -1 - row; }
 struct StepEntry {
   int64_t request = 0;
-  std::vector<int> tokens;     // the request's next tokens
+  std::vector<int> tokens;     // the request's next tokens (ids, or token_from_feedback(row))
   std::vector<int> want;       // places among them (0-based) whose logits are wanted
   int start = -1;              // the position of the first token, if the caller knows it: checked against the cache
 };
@@ -416,7 +421,9 @@ class StepContext {
   Workspace& ws;
   DType act_dtype;                        // dtype of activations and cache: the engine's compute dtype
   int64_t M = 0;                          // tokens in the step
-  const int* tokens = nullptr;            // device int32 [M]
+  const int* tokens = nullptr;            // device int32 [M]; an id below zero: fed_tokens[-1 - id] (token_from_feedback)
+  const int* fed_tokens = nullptr;        // device int32 [n_fed_tokens]: ids the sampler left on the device, or null
+  int n_fed_tokens = 0;
   const int* positions = nullptr;         // device int32 [M]
   const int* slots = nullptr;             // device int32 [M]: the token's entry = row of the block tables
   const int* out_rows = nullptr;          // device int32 [n_out]
@@ -712,6 +719,11 @@ class Engine {
   // other steps by shape once a shape has come twice)
   Tensor step_graph(const std::vector<StepEntry>& entries);
   void release(int64_t request);
+  // Device int32 [feedback_rows()]: where a sampler may leave the ids it draws, so that the next
+  // step can name them with token_from_feedback(row).  Null for a model with parts from outside
+  // the library (their embedding reads ids only).
+  int* token_feedback();
+  int feedback_rows() const;
   void logits_to_host(const Tensor& logits, float* out);    // synchronous copy
   void synchronize();
 
@@ -754,6 +766,14 @@ class Sampler {
   // generated counters[i] tokens so far.  Reads the ids back (a full synchronisation).
   std::vector<int> sample(const Tensor& logits, const std::vector<SamplingParams>& params,
                           const std::vector<int64_t>& requests, const std::vector<int64_t>& counters);
+  // The same without waiting: the ids are drawn and copied back behind whatever the stream holds,
+  // and `collect(ticket)` waits for them.  `device_out` (device int32 [n], e.g. the engine's token
+  // feedback) receives the ids too, for a step that is launched before they are read.  At most two
+  // calls may be under way; `drop` gives up a call whose ids are not needed.
+  uint64_t sample_async(const Tensor& logits, const std::vector<SamplingParams>& params, const std::vector<int64_t>& requests,
+                        const std::vector<int64_t>& counters, int* device_out = nullptr);
+  std::vector<int> collect(uint64_t ticket);
+  void drop(uint64_t ticket);
  private:
   Ops& ops_;
   struct Buffers;
@@ -789,6 +809,9 @@ class Scheduler {
                                const std::vector<int>& eos_token_ids = {});
   bool has_work() const { return !waiting.empty() || !running.empty(); }
   Plan plan();
+  // the step after `last` (launched, not yet committed) if it does not depend on what `last`
+  // samples: one more token of every running request; else an empty plan
+  Plan plan_ahead(const Plan& last) const;
   // the step ran; sampled[request number] for every entry that asked.  Returns the requests that
   // finished: their pages and slots are the caller's to give back.
   std::vector<std::shared_ptr<Request>> commit(const Plan& plan, const std::map<int64_t, int>& sampled);
@@ -809,11 +832,16 @@ class Scheduler {
 struct GenerationStats {
   double prefill_ms = 0, decode_ms = 0;
   int64_t prefill_tokens = 0, decode_tokens = 0, steps = 0, preemptions = 0;
+  int64_t steps_ahead = 0;             // of `steps`: launched before the ids of the step before were read
 };
 // Run until the scheduler has no work: plan, step, sample, commit, release.  When anything
 // throws, every request the scheduler still holds is given back to the cache first.
+// `run_ahead`: while every running request decodes and nobody waits, the next step is launched
+// before the ids of the last one are read (it takes them from the device), so the device does
+// not wait for the host between steps; tokens are the same, `on_token` hears them one step later.
 void run_requests(Engine& engine, Scheduler& scheduler, Sampler* sampler = nullptr, GenerationStats* stats = nullptr,
-                  const std::function<void(const Request&, int token)>& on_token = nullptr, bool use_graph = false);
+                  const std::function<void(const Request&, int token)>& on_token = nullptr, bool use_graph = false,
+                  bool run_ahead = true);
 struct GenerateOptions {
   int max_new_tokens = 128;
   SamplingParams sampling;
@@ -821,6 +849,7 @@ struct GenerateOptions {
   bool use_model_eos = true;
   int chunk_size = 512, max_batched_tokens = 2048;
   bool use_graph = false;
+  bool run_ahead = true;
 };
 std::vector<std::vector<int>> generate(Engine& engine, const std::vector<std::vector<int>>& prompts,
                                        const GenerateOptions& options = {}, GenerationStats* stats = nullptr);
@@ -925,18 +954,27 @@ int ti_sampler_create(void* ops, void** out);
 void ti_sampler_release(void* sampler);
 int ti_sampler_sample(void* sampler, const ti_tensor* logits, int n, const float* temperature, const int* top_k,
                       const float* top_p, const uint64_t* seeds, const int64_t* requests, const int64_t* counters, int* out);
+// without waiting: `ti_sampler_collect` waits for the ids.  `feed_engine` (or null): the ids also go to that engine's
+// token feedback, where its next step finds them under the token ids -1 - row.
+int ti_sampler_sample_async(void* sampler, const ti_tensor* logits, int n, const float* temperature, const int* top_k,
+                            const float* top_p, const uint64_t* seeds, const int64_t* requests, const int64_t* counters,
+                            void* feed_engine, uint64_t* out_ticket);
+int ti_sampler_collect(void* sampler, uint64_t ticket, int n, int* out);
 int ti_scheduler_create(void* cache, int max_batched_tokens, int chunk_size, int max_running, void** out);
 void ti_scheduler_release(void* scheduler);
 int ti_scheduler_add(void* scheduler, int n_prompt, const int* prompt, int max_new_tokens, float temperature, int top_k,
                      float top_p, uint64_t seed, int n_eos, const int* eos, int64_t* out_number);
 int ti_scheduler_plan(void* scheduler, const char** out_json);
+// the step behind the last plan, before that one is committed (Scheduler::plan_ahead); `ti_scheduler_commit` then
+// commits the last plan first and what was planned ahead at its next call
+int ti_scheduler_plan_ahead(void* scheduler, const char** out_json);
 int ti_scheduler_commit(void* scheduler, int n, const int64_t* numbers, const int* tokens, const char** out_finished_json);
 int ti_scheduler_abort(void* scheduler, int64_t number);
 int ti_scheduler_set_next_number(void* scheduler, int64_t number);
 int ti_scheduler_state(void* scheduler, const char** out_json);
 int ti_scheduler_request(void* scheduler, int64_t number, const char** out_json);
 // on_token returns 0; anything else stops the run (the requests still held are given back, and the call fails)
-int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph,
+int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph, int run_ahead,
                     int (*on_token)(int64_t number, int token), const char** out_stats_json);
 
 // the kernels through an Ops object (what the kernel tests and foreign parts call)

@@ -139,15 +139,19 @@ _SIGNATURES = {
     "ti_engine_synchronize": [c_void_p],
     "ti_sampler_create": [c_void_p, _OUT_PTR],
     "ti_sampler_sample": [c_void_p, _TT, c_int, P(c_float), P(c_int), P(c_float), P(c_u64), P(c_i64), P(c_i64), P(c_int)],
+    "ti_sampler_sample_async": [c_void_p, _TT, c_int, P(c_float), P(c_int), P(c_float), P(c_u64), P(c_i64), P(c_i64), c_void_p,
+                                P(c_u64)],
+    "ti_sampler_collect": [c_void_p, c_u64, c_int, P(c_int)],
     "ti_scheduler_create": [c_void_p, c_int, c_int, c_int, _OUT_PTR],
     "ti_scheduler_add": [c_void_p, c_int, P(c_int), c_int, c_float, c_int, c_float, c_u64, c_int, P(c_int), P(c_i64)],
     "ti_scheduler_plan": [c_void_p, _OUT_TEXT],
+    "ti_scheduler_plan_ahead": [c_void_p, _OUT_TEXT],
     "ti_scheduler_commit": [c_void_p, c_int, P(c_i64), P(c_int), _OUT_TEXT],
     "ti_scheduler_abort": [c_void_p, c_i64],
     "ti_scheduler_set_next_number": [c_void_p, c_i64],
     "ti_scheduler_state": [c_void_p, _OUT_TEXT],
     "ti_scheduler_request": [c_void_p, c_i64, _OUT_TEXT],
-    "ti_run_requests": [c_void_p, c_void_p, c_void_p, c_int, ON_TOKEN, _OUT_TEXT],
+    "ti_run_requests": [c_void_p, c_void_p, c_void_p, c_int, c_int, ON_TOKEN, _OUT_TEXT],
     "ti_ops_create": [c_void_p, _OUT_PTR],
     "ti_ops_switch": [c_void_p, c_char_p, c_int, P(c_int)],
     "ti_ops_timing_report": [c_void_p, _OUT_TEXT],

@@ -375,15 +375,15 @@ const Tensor& Rows::materialize(Ops& ops) const {
   return t;
 }
 
-void Ops::embed(const Tensor& table, const int* tokens, int64_t M, const Tensor& x) {
+void Ops::embed(const Tensor& table, const int* tokens, int64_t M, const Tensor& x, const int* fed, int n_fed) {
   TIMED("embed " + dims(x));
   require(table.ndim == 2 && x.ndim == 2, "embed: table and x must be matrices");
   const int64_t V = table.shape[0], H = table.shape[1];
   require(x.shape[0] == M && x.shape[1] == H && x.dtype == DType::F32,
           "embed: x " + x.describe() + " does not fit [" + std::to_string(M) + "," + std::to_string(H) + "] float32");
   require(table.contiguous() && x.contiguous(), "embed: table and x must be contiguous");
-  int rc = KERNEL("core", ti_embed)(code(table.dtype, "embed"), table.data, tokens, (float*)x.data, (int)M, (int)H, (int)V,
-                                    (hipStream_t)launch_stream());
+  int rc = KERNEL("core", ti_embed_fed)(code(table.dtype, "embed"), table.data, tokens, fed, fed ? n_fed : 0, (float*)x.data,
+                                        (int)M, (int)H, (int)V, (hipStream_t)launch_stream());
   check("core", rc, "embed");
 }
 

@@ -129,7 +129,7 @@ class Embedding final : public EmbeddingPart {
     return {{join(prefix, "weight"), n}};
   }
   void load(WeightSource& src) override { weight = src.fetch(join(prefix, "weight"), tensors()[0].second); }
-  void forward(StepContext& ctx, const Tensor& x) override { ctx.ops.embed(weight, ctx.tokens, ctx.M, x); }
+  void forward(StepContext& ctx, const Tensor& x) override { ctx.ops.embed(weight, ctx.tokens, ctx.M, x, ctx.fed_tokens, ctx.n_fed_tokens); }
   bool reads_through_ops() const override { return true; }
   std::vector<std::pair<std::string, Tensor>> held() const override { return {{"weight", weight}}; }
   int64_t vocab, dim;

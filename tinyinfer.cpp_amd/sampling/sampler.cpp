@@ -28,14 +28,33 @@ float uniform(uint64_t seed, uint64_t request, uint64_t n_generated) {
   return (float)(z >> 40) / 16777216.0f;
 }
 
+// Two sets of pinned host buffers take turns, so that a call can be prepared while the call before
+// it is still under way on the device.
 struct Sampler::Buffers {
+  struct Turn {
+    float* f_host = nullptr;     // temperature | top_p | uniform
+    int* i_host = nullptr;       // top_k | ids read back
+    hipEvent_t read_back = nullptr;
+    int n = 0;
+    uint64_t ticket = 0;         // the call whose ids lie here (0: none)
+    bool collected = true;
+  };
   int cap = 0;
-  float* f_host = nullptr;     // temperature | top_p | uniform
-  int* i_host = nullptr;       // top_k | ids read back
+  Turn turns[2];
+  uint64_t issued = 0;
   DeviceBuffer f_dev, i_dev, out_dev;
+  void free_host() {
+    for (Turn& t : turns) {
+      if (t.f_host) (void)hipHostFree(t.f_host);
+      if (t.i_host) (void)hipHostFree(t.i_host);
+      t.f_host = nullptr;
+      t.i_host = nullptr;
+    }
+  }
   ~Buffers() {
-    if (f_host) (void)hipHostFree(f_host);
-    if (i_host) (void)hipHostFree(i_host);
+    free_host();
+    for (Turn& t : turns)
+      if (t.read_back) (void)hipEventDestroy(t.read_back);
   }
 };
 
@@ -46,20 +65,27 @@ static void hip_check(hipError_t e, const char* what) {
   if (e != hipSuccess) throw KernelError(std::string(what) + ": " + hipGetErrorString(e));
 }
 
-std::vector<int> Sampler::sample(const Tensor& logits, const std::vector<SamplingParams>& params,
-                                 const std::vector<int64_t>& requests, const std::vector<int64_t>& counters) {
+uint64_t Sampler::sample_async(const Tensor& logits, const std::vector<SamplingParams>& params,
+                               const std::vector<int64_t>& requests, const std::vector<int64_t>& counters, int* device_out) {
   const int n = (int)logits.shape[0];
   if ((int)params.size() != n || (int)requests.size() != n || (int)counters.size() != n)
     throw KernelError("sample: one set of parameters, one request number and one counter per row of logits");
   hipStream_t stream = (hipStream_t)ops_.stream();
   Buffers& b = *b_;
+  Buffers::Turn& t = b.turns[b.issued & 1];
+  if (!t.collected)
+    throw KernelError("sample: two calls are under way whose ids have not been collected (Sampler::collect)");
   if (n > b.cap) {
+    for (const Buffers::Turn& other : b.turns)
+      if (!other.collected) throw KernelError("sample: more rows than before while a call is under way: collect it first");
     hip_check(hipStreamSynchronize(stream), "hipStreamSynchronize");
     const int cap = std::max(64, 2 * n);
-    if (b.f_host) (void)hipHostFree(b.f_host);
-    if (b.i_host) (void)hipHostFree(b.i_host);
-    hip_check(hipHostMalloc((void**)&b.f_host, (size_t)3 * cap * 4, hipHostMallocDefault), "hipHostMalloc");
-    hip_check(hipHostMalloc((void**)&b.i_host, (size_t)2 * cap * 4, hipHostMallocDefault), "hipHostMalloc");
+    b.free_host();
+    for (Buffers::Turn& u : b.turns) {
+      hip_check(hipHostMalloc((void**)&u.f_host, (size_t)3 * cap * 4, hipHostMallocDefault), "hipHostMalloc");
+      hip_check(hipHostMalloc((void**)&u.i_host, (size_t)2 * cap * 4, hipHostMallocDefault), "hipHostMalloc");
+      if (!u.read_back) hip_check(hipEventCreateWithFlags(&u.read_back, hipEventDisableTiming), "hipEventCreate");
+    }
     b.f_dev = DeviceBuffer((size_t)3 * cap * 4);
     b.i_dev = DeviceBuffer((size_t)cap * 4);
     b.out_dev = DeviceBuffer((size_t)cap * 4);
@@ -67,29 +93,56 @@ std::vector<int> Sampler::sample(const Tensor& logits, const std::vector<Samplin
   }
   bool greedy = true;
   for (const auto& p : params) greedy = greedy && p.temperature <= 0.f;
-  int* out = (int*)b.out_dev.data();
+  int* out = device_out ? device_out : (int*)b.out_dev.data();
   if (greedy) {
     ops_.argmax(logits, out);
   } else {
     const int cap = b.cap;
     for (int i = 0; i < n; ++i) {
-      b.f_host[i] = params[i].temperature;
-      b.f_host[cap + i] = params[i].top_p;
-      b.f_host[2 * cap + i] = uniform(params[i].seed, (uint64_t)requests[i], (uint64_t)counters[i]);
-      b.i_host[i] = params[i].effective_top_k();
+      t.f_host[i] = params[i].temperature;
+      t.f_host[cap + i] = params[i].top_p;
+      t.f_host[2 * cap + i] = uniform(params[i].seed, (uint64_t)requests[i], (uint64_t)counters[i]);
+      t.i_host[i] = params[i].effective_top_k();
     }
-    // the previous call ended with a read-back of its result, so the earlier copies out of the
-    // pinned buffers have finished
+    // this turn's earlier call has been collected: its copies out of these pinned buffers have
+    // finished.  The device copies are shared: the stream puts this call's behind the last call's kernel.
     ops_.flush();
-    hip_check(hipMemcpyAsync(b.f_dev.data(), b.f_host, (size_t)3 * cap * 4, hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
-    hip_check(hipMemcpyAsync(b.i_dev.data(), b.i_host, (size_t)cap * 4, hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+    hip_check(hipMemcpyAsync(b.f_dev.data(), t.f_host, (size_t)3 * cap * 4, hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+    hip_check(hipMemcpyAsync(b.i_dev.data(), t.i_host, (size_t)cap * 4, hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
     const float* fd = (const float*)b.f_dev.data();
     ops_.sample(logits, fd, (const int*)b.i_dev.data(), fd + cap, fd + 2 * cap, out);
   }
-  int* back = b.i_host + b.cap;
-  hip_check(hipMemcpyAsync(back, out, (size_t)n * 4, hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
-  hip_check(hipStreamSynchronize(stream), "hipStreamSynchronize");
-  return std::vector<int>(back, back + n);
+  hip_check(hipMemcpyAsync(t.i_host + b.cap, out, (size_t)n * 4, hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+  hip_check(hipEventRecord(t.read_back, stream), "hipEventRecord");
+  t.n = n;
+  t.collected = false;
+  t.ticket = ++b.issued;
+  return t.ticket;
+}
+
+std::vector<int> Sampler::collect(uint64_t ticket) {
+  Buffers& b = *b_;
+  for (Buffers::Turn& t : b.turns) {
+    if (t.ticket != ticket || t.collected) continue;
+    hip_check(hipEventSynchronize(t.read_back), "hipEventSynchronize");
+    t.collected = true;
+    const int* back = t.i_host + b.cap;
+    return std::vector<int>(back, back + t.n);
+  }
+  throw KernelError("sample: no call with ticket " + std::to_string(ticket) + " is waiting to be collected");
+}
+
+void Sampler::drop(uint64_t ticket) {
+  for (Buffers::Turn& t : b_->turns)
+    if (t.ticket == ticket && !t.collected) {
+      (void)hipEventSynchronize(t.read_back);
+      t.collected = true;
+    }
+}
+
+std::vector<int> Sampler::sample(const Tensor& logits, const std::vector<SamplingParams>& params,
+                                 const std::vector<int64_t>& requests, const std::vector<int64_t>& counters) {
+  return collect(sample_async(logits, params, requests, counters, nullptr));
 }
 
 }  // namespace tinyinfer

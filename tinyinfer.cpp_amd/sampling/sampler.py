@@ -44,15 +44,39 @@ class Sampler:
         except Exception:  # noqa: BLE001
             pass
 
+    @staticmethod
+    def _arguments(n, params, requests, counters):
+        mask = (1 << 64) - 1
+        return ((ctypes.c_float * n)(*[p.temperature for p in params]), (ctypes.c_int * n)(*[p.top_k for p in params]),
+                (ctypes.c_float * n)(*[p.top_p for p in params]), (ctypes.c_uint64 * n)(*[p.seed & mask for p in params]),
+                (ctypes.c_int64 * n)(*requests), (ctypes.c_int64 * n)(*counters))
+
     def sample(self, logits, params: Sequence[SamplingParams], requests: Sequence[int], counters: Sequence[int]) -> List[int]:
         """logits f32 [n, V]; row i belongs to request number `requests[i]`, which has generated
         `counters[i]` tokens so far."""
         n = logits.shape[0]
         native.ensure_kernels(["sampling"])
         out = (ctypes.c_int * n)()
-        mask = (1 << 64) - 1
         native.call("ti_sampler_sample", self._ptr, native.describe_many([logits]), n,
-                    (ctypes.c_float * n)(*[p.temperature for p in params]), (ctypes.c_int * n)(*[p.top_k for p in params]),
-                    (ctypes.c_float * n)(*[p.top_p for p in params]), (ctypes.c_uint64 * n)(*[p.seed & mask for p in params]),
-                    (ctypes.c_int64 * n)(*requests), (ctypes.c_int64 * n)(*counters), out)
+                    *self._arguments(n, params, requests, counters), out)
+        return list(out)
+
+    def sample_async(self, logits, params: Sequence[SamplingParams], requests: Sequence[int], counters: Sequence[int],
+                     feed=None):
+        """The same without waiting: returns a ticket for `collect`.  `feed`: an engine whose token
+        feedback receives the ids too, so that its next step can name them with
+        `token_from_feedback(row)` before they are read.  At most two calls may be under way."""
+        n = logits.shape[0]
+        native.ensure_kernels(["sampling"])
+        ticket = ctypes.c_uint64()
+        native.call("ti_sampler_sample_async", self._ptr, native.describe_many([logits]), n,
+                    *self._arguments(n, params, requests, counters), feed._ptr if feed is not None else None,
+                    ctypes.byref(ticket))
+        return (ticket.value, n)
+
+    def collect(self, ticket) -> List[int]:
+        """Wait for the ids of a `sample_async` call."""
+        number, n = ticket
+        out = (ctypes.c_int * n)()
+        native.call("ti_sampler_collect", self._ptr, number, n, out)
         return list(out)
