@@ -922,6 +922,48 @@ def test_linear_bf16_every_tile(ops, tile, M, N, K):
         lib.ti_gemm_bf16_force_tile(0)
 
 
+@pytest.mark.parametrize("M,N,K", [(2000, 5130, 192), (2048, 5120, 64), (1100, 9000, 128)])
+def test_columns_split_between_two_tile_shapes(ops, M, N, K):
+    """256 x 128 tiles that fill the compute units once or more and leave a round mostly empty: the columns
+    that make whole rounds take those tiles, the rest 128 x 64 tiles in a second launch.  Same bits as the
+    smaller tile everywhere, and the values of float64, for every epilogue."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    lib = ops.lib("gemm_bf16")
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    big = -(-M // 256) * -(-N // 128)
+    assert big >= units and 0 < big % units < units * 3 // 4 and big < 4 * units, "the shape does not take the rule"
+    g = torch.Generator().manual_seed(M + N)
+    a = (torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16)
+    w = (torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16)
+    base = torch.randn(M, N, generator=g)
+    ref = ref_linear(a, w)
+    got = {}
+    for split in (1, 0):
+        lib.ti_gemm_bf16_two_ranges(split)
+        try:
+            out = torch.empty(M, N, device="cuda")
+            ops.linear(dev(a), dev(w), out, "store")
+            added = dev(base.clone())
+            ops.linear(dev(a), dev(w), added, "add")
+            act = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+            ops.linear(dev(a), dev(w), act, "store_act")
+            paired = torch.empty(M, N // 2, device="cuda", dtype=torch.bfloat16)
+            ops.linear(dev(a), dev(w), paired, "swiglu")
+            got[split] = (out, added, act, paired)
+        finally:
+            lib.ti_gemm_bf16_two_ranges(1)
+    for x, y in zip(got[1], got[0]):
+        assert torch.equal(x, y)
+    tol = 2e-5 * K
+    assert (f64(got[1][0]) - ref).abs().max() < tol
+    assert (f64(got[1][1]) - (ref + f64(base))).abs().max() < tol
+    assert (f64(got[1][2]) - ref).abs().max() < 0.005 * ref.abs().max() + tol
+    gte, up = ref[:, :N // 2], ref[:, N // 2:]
+    want = gte / (1 + torch.exp(-gte)) * up
+    assert (f64(got[1][3]) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
+
+
 @pytest.mark.parametrize("M", [17, 40, 64])
 def test_swiglu_of_up_to_64_rows_under_a_wide_weight(ops, M):
     """17 to 64 rows times a stacked [gate; up] weight of 32,768 rows take 64 x 128 tiles (twice the weight
@@ -1331,6 +1373,20 @@ def test_qkv_product_with_prepared_heads(ops, tile_rows, M, nh, nkv, hd, K, P, n
     units), against the product followed by the kernel that prepares whole steps: the same bits
     in q and in the cache (rows that are no multiple of the tile, a last tile with a head beyond
     the matrix, no k/v heads)."""
+    qkv_prepared_case(ops, tile_rows, M, nh, nkv, hd, K, P, norm, rope)
+
+
+@pytest.mark.parametrize("M,nh,nkv,hd", [(2048, 32, 4, 128), (1900, 70, 5, 64)])
+def test_qkv_product_with_prepared_heads_in_two_ranges(ops, M, nh, nkv, hd):
+    """256-row tiles that would leave a round of workgroups mostly empty: the heads that make whole
+    rounds take them, the other heads 128-row tiles in a second launch.  The same bits."""
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    big = -(-M // 256) * ((nh + 2 * nkv) * hd // 128)
+    assert big >= units and 0 < big % units < units * 3 // 4, "the shape does not take the rule"
+    qkv_prepared_case(ops, 0, M, nh, nkv, hd, 64, 16, True, "table")
+
+
+def qkv_prepared_case(ops, tile_rows, M, nh, nkv, hd, K, P, norm, rope):
     if not ops.use_fast_gemm:
         pytest.skip("bfloat16 MFMA kernels are switched off")
     g = torch.Generator().manual_seed(M + nh)

@@ -855,7 +855,8 @@ __device__ __forceinline__ void qkv_rows_by_lanes(const QKVEpilogue& ep, float* 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_arg,
-                      int M, int N, int K, long lda, QKVEpilogue ep = QKVEpilogue{}) {
+                      int M, int N, int K, long lda, int n_first, QKVEpilogue ep = QKVEpilogue{}) {
+  // n_first: the output column the grid's first workgroup starts at (a launch may cover a range of columns)
   constexpr bool SW = (EPI == TI_EPI_SWIGLU);
   constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
   constexpr int NWV = WAVES_M * WAVES_N;                     // wavefronts: 4 or 8
@@ -875,7 +876,7 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int m0 = blockIdx.y * BM;
-  const int n0 = blockIdx.x * (SW ? BN / 2 : BN);
+  const int n0 = n_first + blockIdx.x * (SW ? BN / 2 : BN);
   const int lr = lane >> 3, lc = lane & 7;                   // row within a group of 8, slot within the row
 
   // the global row each of this lane's loads reads (clamped into the matrix: rows
@@ -1115,7 +1116,7 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
 static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
-                            hipStream_t s, int ksplit = 1) {
+                            hipStream_t s, int ksplit = 1, int n_first = 0, int n_end = -1) {
   constexpr int bytes = PSTAGES * (BM + BN) * PBK * 2;
   auto kernel = gemm_pipelined_kernel<BM, BN, WAVES_M, WAVES_N, EPI>;
   static bool ready = false;          // per instantiation: allow more than 64 KiB of dynamic LDS
@@ -1127,11 +1128,15 @@ static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, 
     ready = true;
   }
   const int bn = (EPI == TI_EPI_SWIGLU) ? BN / 2 : BN;
-  dim3 grid((N + bn - 1) / bn, (M + BM - 1) / BM, (EPI == TI_EPI_STORE_F32) ? ksplit : 1);
-  kernel<<<grid, WAVES_M * WAVES_N * 64, bytes, s>>>(A, W, out, M, N, K, lda, QKVEpilogue{});
+  // columns [n_first, n_end) of the output (all of them by default); n_end short of N is a multiple of the tile
+  if (n_end < 0) n_end = N;
+  dim3 grid((n_end - n_first + bn - 1) / bn, (M + BM - 1) / BM, (EPI == TI_EPI_STORE_F32) ? ksplit : 1);
+  kernel<<<grid, WAVES_M * WAVES_N * 64, bytes, s>>>(A, W, out, M, N, K, lda, n_first, QKVEpilogue{});
   return 0;
 }
 
+static int g_two_ranges = 1;     // a hook for measurements: 0 = never split the columns between two tile shapes
+extern "C" void ti_gemm_bf16_two_ranges(int on) { g_two_ranges = on; }
 static int g_qkv_rows = 0;       // hooks for measurements: 128 or 256 forces the tile's rows;
 static int g_qkv_min_rows = 17;  // the fewest rows served (fewer take the kernels with the norm in front)
 extern "C" void ti_gemm_bf16_qkv_prep_min_rows(int rows) { g_qkv_min_rows = rows; }
@@ -1150,7 +1155,7 @@ static int compute_units() {
 
 template <int BM, int WAVES_M, int WAVES_N>
 static int launch_qkv_prep(const void* A, const void* W, int M, int N, int K, long lda, const QKVEpilogue& ep,
-                           hipStream_t stream) {
+                           hipStream_t stream, int n_first = 0, int n_end = -1) {
   constexpr int BN = 128;
   constexpr int bytes = PSTAGES * (BM + BN) * PBK * 2;
   auto kernel = gemm_pipelined_kernel<BM, BN, WAVES_M, WAVES_N, TI_EPI_QKV_PREP>;
@@ -1162,8 +1167,9 @@ static int launch_qkv_prep(const void* A, const void* W, int M, int N, int K, lo
     }
     ready = true;
   }
-  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
-  kernel<<<grid, 512, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, nullptr, M, N, K, lda, ep);
+  if (n_end < 0) n_end = N;               // columns [n_first, n_end): whole heads
+  dim3 grid((n_end - n_first + BN - 1) / BN, (M + BM - 1) / BM);
+  kernel<<<grid, 512, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, nullptr, M, N, K, lda, n_first, ep);
   return 0;
 }
 
@@ -1202,8 +1208,21 @@ extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K,
     return 3;
   }
   const bool rows128 = g_qkv_rows ? g_qkv_rows == 128 : tiles128 <= compute_units();
-  int rc_ = rows128 ? launch_qkv_prep<128, 2, 4>(A, W, M, N, K, lda, ep, stream)
-                    : launch_qkv_prep<256, 4, 2>(A, W, M, N, K, lda, ep, stream);
+  // 256-row tiles that leave a round short of three quarters (Qwen3-8B's 48 heads over 2,048 rows: 8 x 48
+  // tiles on 256 units): the heads that make whole rounds take them, the other heads 128-row tiles in a
+  // launch of their own, as in the plain product
+  const int units = compute_units(), row_tiles = (M + 255) / 256;
+  const long big = (long)row_tiles * ((N + 127) / 128);
+  int rc_;
+  if (!rows128 && !g_qkv_rows && g_two_ranges && big >= units && big < 4L * units && big % units != 0 &&
+      big % units < units * 3 / 4 && (int)(big / units * units / row_tiles) >= 1) {
+    const int n_big = (int)(big / units * units / row_tiles) * 128;
+    rc_ = launch_qkv_prep<256, 4, 2>(A, W, M, N, K, lda, ep, stream, 0, n_big);
+    if (!rc_) rc_ = launch_qkv_prep<128, 2, 4>(A, W, M, N, K, lda, ep, stream, n_big, N);
+  } else {
+    rc_ = rows128 ? launch_qkv_prep<128, 2, 4>(A, W, M, N, K, lda, ep, stream)
+                  : launch_qkv_prep<256, 4, 2>(A, W, M, N, K, lda, ep, stream);
+  }
   if (rc_) return rc_;
   TI_LAUNCH_CHECK();
   return 0;
@@ -1224,8 +1243,9 @@ static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M,
   constexpr bool SW = EPI == TI_EPI_SWIGLU;
   const long big = (long)((M + 255) / 256) * ((N * cols + 127) / 128);
   const long mid = (long)((M + 127) / 128) * ((N * cols + 63) / 64);
-  const bool whole_rounds = big >= 256 && (big % 256 == 0 || big % 256 >= 192);
-  int tile = (big >= 1024 || whole_rounds) ? 1 : (mid >= 512 ? 3 : 6);
+  const int units = compute_units();
+  const bool whole_rounds = big >= units && (big % units == 0 || big % units >= units * 3 / 4);
+  int tile = (big >= 4 * units || whole_rounds) ? 1 : (mid >= 2 * units ? 3 : 6);
   if (M <= 64 && tile == 1) tile = 6;                // few rows times a wide weight: no 256-row tile
   // Up to 64 rows times a stacked [gate; up] weight: such a product waits for the weight from memory, and
   // a 128 x 64 tile, half of whose rows are empty then, has 8 of its 24 KB a stage in weights.  A 64 x 128
@@ -1233,6 +1253,20 @@ static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M,
   // at 64 rows 141 -> 115 us, 8B's 52 -> 45); a weight that gives it fewer workgroups than half the
   // units stays with the narrower tile (0.6B's: 10.0 against 10.6 us).
   if (SW && M <= 64 && (long)(N * cols + 127) / 128 * 2 >= compute_units()) tile = 5;
+  // 256 x 128 tiles that fill the units once or more and leave a round short of three quarters (Qwen3-32B's
+  // o and down projections over 2,048 rows: 8 x 40 tiles on 256 units): the columns that make whole rounds
+  // take those tiles, the rest 128 x 64 tiles in a launch of their own behind them, rather than everything
+  // the smaller tile, which needs a third more time per flop (those projections 548 -> 420 us on average;
+  // Qwen3-0.6B's gate/up, 8 x 48 tiles, likewise).
+  if (tile == 3 && big >= units && !g_force_tile && g_two_ranges) {
+    const int row_tiles = (M + 255) / 256;
+    const int col_tiles = (int)(big / units * units / row_tiles);
+    const int n_big = col_tiles * (128 / cols);         // output columns of the first range
+    if (col_tiles >= 1 && n_big < N) {
+      if (int rc = launch_pipelined<256, 128, 4, 2, EPI>(A, W, out, M, N, K, lda, s, 1, 0, n_big)) return rc;
+      return launch_pipelined<128, 64, 4, 1, EPI>(A, W, out, M, N, K, lda, s, 1, n_big, N);
+    }
+  }
   if (g_force_tile) tile = g_force_tile;
   if (tile == 1) return launch_pipelined<256, 128, 4, 2, EPI>(A, W, out, M, N, K, lda, s);
   if constexpr (EPI == TI_EPI_SWIGLU)
