@@ -206,6 +206,40 @@ def test_prepared_decode_attention_changes_only_rounding(model_folders):
         assert not np.array_equal(results[0][r][:1], results[0][r][1:2])
 
 
+@pytest.mark.parametrize("config,fused", [("D", True), ("D", False), ("B", True)])
+def test_page_ids_fetched_beside_the_position_change_no_bit(model_folders, config, fused):
+    """In a step of single tokens the decode attention fetches a row's page ids beside its position
+    instead of behind it (row m of the step is row m of the block tables).  With that switched off
+    the same steps give the same bits: requests that start in different steps, so that rows and
+    block-table rows are told apart, with pages that are used again."""
+    folder = model_folders(config, "bfloat16", True)
+    V = CONFIGS[config]["vocab_size"]
+    requests = {r: random_tokens(n, V, 50 + i) for i, (r, n) in enumerate((("a", 90), ("b", 41), ("c", 70), ("d", 55)))}
+    first = {"a": 50, "b": 21, "c": 30, "d": 35}                      # fed whole; the rest one token a step
+    trace = [{"entries": [(r, requests[r][:first[r]], [first[r] - 1]) for r in ("a", "b", "c")], "end": []}]
+    fed = dict(first)
+    live = ["a", "b", "c"]
+    for k in range(40):
+        if k == 20:                                                   # b is over; d takes its pages
+            trace.append({"entries": [("d", requests["d"][:first["d"]], [first["d"] - 1])], "end": []})
+            live = ["d", "c", "a"]
+        order = live[k % 3:] + live[:k % 3]                           # the rows of a step in changing order
+        trace.append({"entries": [(r, requests[r][fed[r]:fed[r] + 1], [0]) for r in order], "end": ["b"] if k == 19 else []})
+        for r in order:
+            fed[r] += 1
+    trace[-1]["end"] = list(live)
+    assert fed == {"a": 90, "b": 41, "c": 70, "d": 55}
+    results = []
+    for early in (True, False):
+        engine = build_engine(folder, "bfloat16", 256)
+        engine.ops.use_early_page_ids = early
+        engine.ops.use_fused_qk_decode = fused
+        results.append(replay(engine, trace))
+    for r in requests:
+        assert np.array_equal(results[0][r], results[1][r]), r
+        assert len(results[0][r]) == len(requests[r]) - first[r] + 1
+
+
 def test_prepared_qkv_product_changes_no_bit(model_folders):
     """Steps of many tokens prepare q and write the cache in the epilogue of the q/k/v product.
     With that switched off the same steps give the same bits (config D, head size 64)."""

@@ -1348,6 +1348,22 @@ def test_attention_bf16_decode_from_projections(ops, nh, nkv, hd, P, window, nor
                                           nh, nkv, hd, scale, window)
     assert torch.equal(pool_a.view(torch.int16), pool_b.view(torch.int16))
     assert torch.isfinite(out_b.float()).all()
+    # told that row m of the step is row m of the block tables, both kernels fetch the row's page ids beside
+    # the position instead of behind it: the same bits
+    assert torch.equal(ctx.slots.cpu(), torch.arange(M, dtype=torch.int32))
+    ctx.slots_are_rows = True
+    try:
+        out_a2 = torch.zeros_like(q)
+        ops.attention(ctx, view, q, pool_a, out_a2, nh, nkv, hd, scale, window)
+        assert torch.equal(out_a2.view(torch.int16), out_a.view(torch.int16))
+        pool_b2 = dev(pool.clone())
+        out_b2 = torch.zeros_like(q)
+        assert ops.attention_from_projections(ctx, view, qkv, q_w, k_w, 1e-5, inv_freq, tab, pool_b2, True, out_b2,
+                                              nh, nkv, hd, scale, window)
+        assert torch.equal(out_b2.view(torch.int16), out_b.view(torch.int16))
+        assert torch.equal(pool_b2.view(torch.int16), pool_b.view(torch.int16))
+    finally:
+        ctx.slots_are_rows = False
 
     def same_up_to_one_step(x, y):
         x, y = x.float(), y.float()

@@ -100,7 +100,9 @@ int ti_attention_decode_bf16(const void* q, const void* pool, const int* table, 
                              int n_head, int n_kv, int hd, int page_size, float scale, int window, int n_splits,
                              hipStream_t stream);
 // the same from the 32-bit projections: norm, rotation and the cache write of the row's own key and
-// value happen inside (head sizes 64 and 128, at most 16 q heads per kv head)
+// value happen inside (head sizes 64 and 128, at most 16 q heads per kv head).  slot may be null
+// (both entry points) where row m of the step is row m of the block tables and a table row has at
+// most 1,024 entries: the page ids are then fetched beside the position, not behind it
 int ti_attention_decode_prepared_bf16(const float* qkv, int row_width, const float* q_w, const float* k_w, float eps,
                                       const float* inv_freq, const float* rope_table, int table_len, void* pool,
                                       int write_kv, const int* table, int table_stride, const int* pos,

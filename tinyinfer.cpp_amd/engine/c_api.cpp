@@ -1006,6 +1006,7 @@ int ti_ops_switch(void* ops_, const char* name_, int value, int* old) {
   else if (name == "fused_qk_decode") flag(ops.use.fused_qk_decode);
   else if (name == "fused_qkv_prefill") flag(ops.use.fused_qkv_prefill);
   else if (name == "split_k_add") flag(ops.use.split_k_add);
+  else if (name == "early_page_ids") flag(ops.use.early_page_ids);
   else if (name == "deferred_add") flag(ops.use.deferred_add);
   else if (name == "paired_prefill") flag(ops.use.paired_prefill);
   else if (name == "portion_splits") flag(ops.use.portion_splits);
@@ -1120,6 +1121,7 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     w.max_context = (int)num(10);
     w.portion_context = (int)num(11);
     w.split_context = (int)num(12);
+    w.slots_are_rows = n_s > 15 && s[15] != 0;
     Workspace& ws = workspace_of(&ops);
     if (op == "attention") {
       ops.attention(w, ws, view_of(2, arg(1)), arg(0), arg(1), arg(3), (int)num(0), (int)num(1), (int)num(2), (float)num(3), (int)num(4));

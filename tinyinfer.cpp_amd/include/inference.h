@@ -315,6 +315,7 @@ class Ops {
   struct Switches {
     bool fast_gemm = true, fast_attention = true, fused_norm = true, fused_qk_decode = true, fused_qkv_prefill = true;
     bool split_k_add = true, deferred_add = true, paired_prefill = true, portion_splits = true;
+    bool early_page_ids = true;     // a step of single tokens: the decode attention fetches a row's page ids beside its position
     int force_paired_tiles = -1;    // 1 / 0: that kernel with / without pairs, whatever the launch
     int force_decode_splits = 0;    // > 0: the decode attention cuts every context into this many runs
   } use;
@@ -369,6 +370,7 @@ struct AttentionWork {
   const int* decode_rows = nullptr;  // rows of single-token entries (null when every entry is one)
   int n_decode_rows = 0;
   bool decode_only = false;
+  bool slots_are_rows = false;       // slots[m] == m for every row (a step of single tokens, one entry a row)
   int max_context = 0;               // longest context any row reads
   int portion_context = 0;           // ... over rows of entries of several tokens
   int split_context = 0;             // the context the decode kernel's runs are sized for

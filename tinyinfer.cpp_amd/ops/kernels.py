@@ -93,7 +93,7 @@ class NormedRows:
 _SWITCHES = {"use_fast_gemm": "fast_gemm", "use_fast_attention": "fast_attention", "use_fused_norm": "fused_norm",
              "use_fused_qk_decode": "fused_qk_decode", "use_fused_qkv_prefill": "fused_qkv_prefill",
              "use_split_k_add": "split_k_add", "use_deferred_add": "deferred_add", "use_paired_prefill": "paired_prefill",
-             "use_portion_splits": "portion_splits"}
+             "use_portion_splits": "portion_splits", "use_early_page_ids": "early_page_ids"}
 _LIB_OF = {"embed": "core", "rmsnorm": "core", "rope_neox": "core", "rope_table": "core", "qk_norm_rope_kv_write": "core",
            "qk_norm_inplace": "core", "argmax": "sampling", "sample": "sampling", "attention_rows": "attention_generic",
            "fill_random": "core", "fill_zero": "core"}
@@ -287,7 +287,8 @@ class Ops:
         """Attention of every row of the step over its request's pages."""
         t, n = self._work(ctx)
         libs = ["attention_generic"] + (["attention_bf16"] if q.dtype == native.torch().bfloat16 and self.use_fast_attention else [])
-        self._call("attention", [q, pool, view.table, out] + t, [heads, kv_heads, head_dim, scale, int(window or 0)] + n,
+        rows = [0.0, 0, 1] if getattr(ctx, "slots_are_rows", False) else []      # (unused, unused, slots[m] == m)
+        self._call("attention", [q, pool, view.table, out] + t, [heads, kv_heads, head_dim, scale, int(window or 0)] + n + rows,
                    fold=(1,), libs=libs)
 
     def attention_from_projections(self, ctx, view, qkv, q_w, k_w, eps, inv_freq, rope_table, pool, write_kv, out, heads,
@@ -298,7 +299,8 @@ class Ops:
             return False
         t, n = self._work(ctx)
         return bool(self._call("attention_from_projections", [qkv, pool, view.table, out] + t + [q_w, k_w, inv_freq, rope_table],
-                               [heads, kv_heads, head_dim, scale, int(window or 0)] + n + [eps, int(bool(write_kv))],
+                               [heads, kv_heads, head_dim, scale, int(window or 0)] + n + [eps, int(bool(write_kv))] +
+                               ([1] if getattr(ctx, "slots_are_rows", False) else []),
                                fold=(1,), libs=["attention_bf16", "core"]))
 
     # ------------------------------------------------------------------ sampling

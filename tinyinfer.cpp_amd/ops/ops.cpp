@@ -701,8 +701,9 @@ bool Ops::attention_from_projections(const AttentionWork& work, Workspace& ws, c
   }
   int rc = KERNEL("attention_bf16", ti_attention_decode_prepared_bf16)(
       (const float*)qkv.data, (int)qkv.shape[1], q_w, k_w, eps, rot.inv_freq, rot.table, rot.table_len, pool.data,
-      write_kv ? 1 : 0, view.table, view.table_width, work.positions, work.slots, out.data, part_o, part_ml, n, heads,
-      kv_heads, head_dim, P, scale, window, S, (hipStream_t)launch_stream());
+      write_kv ? 1 : 0, view.table, view.table_width, work.positions,
+      (work.slots_are_rows && view.table_width <= 1024 && use.early_page_ids) ? nullptr : work.slots, out.data, part_o, part_ml, n,
+      heads, kv_heads, head_dim, P, scale, window, S, (hipStream_t)launch_stream());
   if (rc == 3) return false;
   check("attention_bf16", rc, "attention(decode, prepared)");
   return true;
@@ -759,8 +760,9 @@ void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& v
           part_ml = (float*)ws.get("attn.part_ml", (size_t)n_dec * heads * S * 2 * 4);
         }
         int rc = KERNEL("attention_bf16", ti_attention_decode_bf16)(
-            q.data, pool.data, view.table, view.table_width, work.positions, work.slots, rows, out.data, part_o, part_ml,
-            n_dec, heads, kv_heads, head_dim, P, scale, window, S, (hipStream_t)stream);
+            q.data, pool.data, view.table, view.table_width, work.positions,
+            (work.slots_are_rows && !rows && view.table_width <= 1024 && use.early_page_ids) ? nullptr : work.slots, rows, out.data,
+            part_o, part_ml, n_dec, heads, kv_heads, head_dim, P, scale, window, S, (hipStream_t)stream);
         if (rc == 3) done = false;
         else check("attention_bf16", rc, "attention(decode)");
       }

@@ -457,6 +457,7 @@ class Attention final : public MixerPart {
     w.slots = ctx.slots;
     w.entry_meta = ctx.entry_meta;
     w.decode_only = ctx.decode_only;
+    w.slots_are_rows = ctx.decode_only;      // every entry is one row: a row's entry is the row itself
     w.max_context = ctx.max_context;
     w.split_context = ctx.max_context;
     if (!ctx.decode_only) {
