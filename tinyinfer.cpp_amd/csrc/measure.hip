@@ -35,19 +35,28 @@ extern "C" int ti_measure_read(const void* p, long bytes, void* sink, int blocks
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
-// every wavefront runs `iters` rounds of four independent 32x32x16 bfloat16 MFMAs on registers
+// every wavefront runs `iters` rounds of four independent 32x32x16 bfloat16 MFMAs on registers.  The
+// operands are scattered values (what the chip draws, and with it its clock, depends on the bits that
+// toggle: all-zero operands run a fifth faster than a model's), different in every lane and round.
 __global__ void __launch_bounds__(256) mfma_kernel(int iters, float* __restrict__ sink) {
-  bf16x8_t a, b;
-  for (int i = 0; i < 8; ++i) {
-    a[i] = (__bf16)(float)(threadIdx.x + i);
-    b[i] = (__bf16)(float)(threadIdx.x - i);
-  }
+  bf16x8_t a[4], b[4];
+  unsigned h = (blockIdx.x * 256u + threadIdx.x) * 2654435761u + 12345u;
+  for (int j = 0; j < 4; ++j)
+    for (int i = 0; i < 8; ++i) {
+      h = h * 1664525u + 1013904223u;
+      a[j][i] = (__bf16)(((int)(h >> 16) % 2001 - 1000) * 1e-3f);
+      h = h * 1664525u + 1013904223u;
+      b[j][i] = (__bf16)(((int)(h >> 16) % 2001 - 1000) * 2e-5f);
+    }
   float16_t c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
-  for (int it = 0; it < iters; ++it) {
-    c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c0, 0, 0, 0);
-    c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c1, 0, 0, 0);
-    c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c2, 0, 0, 0);
-    c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c3, 0, 0, 0);
+  for (int it = 0; it < iters; it += 4) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j], b[j], c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(j + 1) & 3], b[j], c1, 0, 0, 0);
+      c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(j + 2) & 3], b[j], c2, 0, 0, 0);
+      c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(j + 3) & 3], b[j], c3, 0, 0, 0);
+    }
   }
   float s = 0.f;
   for (int i = 0; i < 16; ++i) s += c0[i] + c1[i] + c2[i] + c3[i];

@@ -43,7 +43,7 @@ class StepEntry:
 class Engine:
     def __init__(self, model: Model, dtype: str = "bfloat16", page_size: int = 16, max_tokens: Optional[int] = None,
                  num_pages: Optional[int] = None, max_requests: int = 64, max_seq: Optional[int] = None,
-                 device: str = "cuda", max_step_graphs: Optional[int] = None):
+                 device: str = "cuda", max_step_graphs: Optional[int] = None, stream: Optional[int] = None):
         if dtype not in DTYPES:
             raise EngineError(f"dtype must be one of {sorted(DTYPES)}, got {dtype!r}")
         t = native.torch()
@@ -64,6 +64,8 @@ class Engine:
             options["max_seq"] = int(max_seq)
         if max_step_graphs is not None:
             options["max_step_graphs"] = int(max_step_graphs)
+        if stream is not None:
+            options["stream"] = int(stream)          # a HIP stream's handle (torch: Stream.cuda_stream); default: the null stream
         self._ptr = native.pointer("ti_engine_create", model._ptr, json.dumps(options).encode())
         info = self.info()
         self.page_size, self.max_seq, self.num_pages = info["page_size"], info["max_seq"], info["num_pages"]
