@@ -125,6 +125,44 @@ def test_engine_matches_plain(model_folders, name, sharp, page_size, dtype, mode
     assert err < tol, (err, tol, where)
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+@pytest.mark.parametrize("name,dtype,page_size,graph", [("B", "float32", 4, False), ("D", "float32", 16, True),
+                                                        ("B", "bfloat16", 16, True), ("D", "bfloat16", 32, False)])
+def test_steps_drawn_at_random_match_plain(model_folders, name, dtype, page_size, graph, seed):
+    """Steps cut at random: which live requests a step feeds, in which order, how many tokens each,
+    which places are wanted; the pool as tight as the trace allows; with graphs, the shapes that
+    repeat are replayed.  Only the wanted places come back, and each is the plain model's."""
+    folder = model_folders(name, "bfloat16", True)
+    requests = make_requests(CONFIGS[name]["vocab_size"])
+    want, tol = plain_logits(folder, requests, dtype)
+    trace = traces.at_random(requests, seed)
+    assert any(len(s["entries"]) >= 3 for s in trace) and any(len(t) == 1 for s in trace for _, t, _ in s["entries"])
+    engine = build_engine(folder, dtype, traces.max_pages(trace, page_size) * page_size, page_size)
+    from tinyinfer_amd.engine import StepEntry
+    fed = {r: 0 for r in requests}
+    worst_err, where = 0.0, None
+    for k, step in enumerate(trace):
+        entries = [StepEntry(r, t, w) for r, t, w in step["entries"]]
+        logits = (engine.step_graph(entries) if graph else engine.step(entries)).cpu().numpy().astype(np.float64)
+        i = 0
+        for r, t, w in step["entries"]:
+            for place in w:
+                err = float(np.abs(logits[i] - want[r][fed[r] + place]).max())
+                if err > worst_err:
+                    worst_err, where = err, (k, r, fed[r] + place)
+                i += 1
+            fed[r] += len(t)
+        assert i == logits.shape[0]
+        for r in step["end"]:
+            engine.release(r)
+        engine.cache.check()
+    assert not engine.cache.live_requests()
+    assert fed == {r: len(t) for r, t in requests.items()}
+    print(f"\n[{name} {dtype} P={page_size} graph={graph} seed={seed}] {len(trace)} steps, max |engine - plain| = "
+          f"{worst_err:.3e} at {where} (allowed {tol:.3e})")
+    assert worst_err < tol, (worst_err, tol, where)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_float32_weights_stay_32bit(model_folders, dtype):
     """A folder stored in float32: the float32 engine uses every bit of it."""

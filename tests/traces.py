@@ -86,6 +86,41 @@ def mixed(requests: Dict[str, Sequence[int]], prompt_len: Dict[str, int], live: 
     return steps
 
 
+def at_random(requests: Dict[str, Sequence[int]], seed: int, live: int = 4):
+    """Up to `live` requests at a time, drawn from a seed: which of them a step feeds (at least one;
+    the others sit out), how many tokens each gets (1 most often, else 2 to 40), and which of those
+    places are wanted (the last one always, so that a request can be followed; others at random, so
+    that the rows a step leaves out lie at changing places).  A request that is done ends at once;
+    the next in line takes its place in a later step."""
+    import random
+    rng = random.Random(seed)
+    waiting = list(requests)
+    rng.shuffle(waiting)
+    fed = {r: 0 for r in requests}
+    active: List[str] = []
+    steps = []
+    while waiting or active:
+        while waiting and len(active) < live and (not active or rng.random() < 0.6):
+            active.append(waiting.pop(0))
+        chosen = [r for r in active if rng.random() < 0.7] or [rng.choice(active)]
+        rng.shuffle(chosen)                                  # the rows of a step in changing order
+        entries, ended = [], []
+        for rid in chosen:
+            toks = list(requests[rid])
+            left = len(toks) - fed[rid]
+            n = 1 if rng.random() < 0.55 else rng.choice((2, 2, 3, 5, 8, 13, 16, 17, 31, 40))
+            n = min(n, left)
+            want = sorted(set([n - 1] + [i for i in range(n - 1) if rng.random() < 0.3]))
+            entries.append((rid, toks[fed[rid]:fed[rid] + n], want))
+            fed[rid] += n
+            if fed[rid] == len(toks):
+                ended.append(rid)
+        for rid in ended:
+            active.remove(rid)
+        steps.append({"entries": entries, "end": ended})
+    return steps
+
+
 def max_tokens(trace) -> int:
     held: Dict[str, int] = {}
     worst = 0
