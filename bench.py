@@ -33,12 +33,18 @@ BASE = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", head_dim=128
 MODELS = {
     "0.6b": dict(BASE, num_hidden_layers=28, hidden_size=1024, num_attention_heads=16, num_key_value_heads=8,
                  intermediate_size=3072, tie_word_embeddings=True),
+    "1.7b": dict(BASE, num_hidden_layers=28, hidden_size=2048, num_attention_heads=16, num_key_value_heads=8,
+                 intermediate_size=6144, tie_word_embeddings=True),
+    "4b": dict(BASE, num_hidden_layers=36, hidden_size=2560, num_attention_heads=32, num_key_value_heads=8,
+               intermediate_size=9728, tie_word_embeddings=True),
     "8b": dict(BASE, num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
                intermediate_size=12288, tie_word_embeddings=False),
+    "14b": dict(BASE, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8,
+                intermediate_size=17408, tie_word_embeddings=False),
     "32b": dict(BASE, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,
                 intermediate_size=25600, tie_word_embeddings=False),
 }
-NAMES = {"0.6b": "Qwen3-0.6B", "8b": "Qwen3-8B", "32b": "Qwen3-32B"}
+NAMES = {"0.6b": "Qwen3-0.6B", "1.7b": "Qwen3-1.7B", "4b": "Qwen3-4B", "8b": "Qwen3-8B", "14b": "Qwen3-14B", "32b": "Qwen3-32B"}
 MAX_SEQ = 4096            # context length a request may reach (more if --context asks for it)
 PAGE = 16
 PEAK_HBM = 8.0e12         # bytes/s, MI355X

@@ -1358,9 +1358,14 @@ static bool large_weight(int M, int N, int K, int epi) {
 #define GR_ROWS_BELOW 4096
 static int g_row_per_wave = 1;
 extern "C" void ti_gemm_bf16_row_per_wave(int on) { g_row_per_wave = on; }
+// Every workgroup (four weight rows) copies all M token rows into LDS: M / 4 times the bytes of its
+// weight rows.  Up to four tokens that is no more than the weight itself; beyond, the kernel is taken
+// only while its workgroups are no more than the compute units (Qwen3-0.6B's o and down, 1,024 rows: 4.7
+// against 7.5 us at 8 tokens), not for more rows (Qwen3-4B's o, 2,560 x 4,096: 10.8 us here, 6.1 in
+// workgroups of 16 rows; 1.7B's, 2,048 x 2,048: 3.9 against 3.0).
 static bool row_per_wave_serves(int M, int N, int K, int epi) {
-  return g_row_per_wave && M <= GR_MMAX && N < GR_ROWS_BELOW && K % 8 == 0 && K <= 64 * 8 * GR_LOADS &&
-         (epi == TI_EPI_STORE_F32 || epi == TI_EPI_ADD_F32);
+  return g_row_per_wave && M <= GR_MMAX && N < GR_ROWS_BELOW && (M <= 4 || N <= 4 * compute_units()) && K % 8 == 0 &&
+         K <= 64 * 8 * GR_LOADS && (epi == TI_EPI_STORE_F32 || epi == TI_EPI_ADD_F32);
 }
 
 template <int EPI, int MMAX, int NL>
@@ -1416,7 +1421,9 @@ static int skinny_waves_for(int grid, int K) {
 }
 
 static bool pieces_serves(int M, int N, int K, int epi);
-#define NORMED_WEIGHT_BELOW (64L << 20)   // weight elements from which the norm stays a kernel of its own
+#define NORMED_WEIGHT_BELOW (40L << 20)   // weight elements from which the norm stays a kernel of its own
+static long g_normed_weight_below = NORMED_WEIGHT_BELOW;
+extern "C" void ti_gemm_bf16_normed_weight_below(long elements) { g_normed_weight_below = elements > 0 ? elements : NORMED_WEIGHT_BELOW; }
 // out = rmsnorm(x; nw, eps) W^T for M <= 16 (see gemm_skinny_staged_kernel).  Returns 3 for
 // sizes it does not serve (M > 16, K not a multiple of 64 or above 4096).
 extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, const void* W, void* out,
@@ -1438,8 +1445,9 @@ extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, c
   }
   // Every workgroup here norms all M rows for itself, which pulls as many bytes through the caches as
   // its share of the weight has.  Under a large weight the kernel that keeps loads in flight gains more
-  // than the norm's own launch costs (Qwen3-8B's gate/up at 8 rows: 46 us here, 38 + 5 us there).
-  if ((long)(epi == TI_EPI_SWIGLU ? 2 : 1) * N * K >= NORMED_WEIGHT_BELOW && pieces_serves(M, N, K, epi)) {
+  // than the norm's own launch costs (Qwen3-8B's gate/up, 100 M elements, at 8 rows: 46 us here, 38 + 5 us
+  // there; Qwen3-4B's, 50 M: 29 against 21 + 2.5; Qwen3-1.7B's, 25 M, and 8B's q/k/v are faster here).
+  if ((long)(epi == TI_EPI_SWIGLU ? 2 : 1) * N * K >= g_normed_weight_below && pieces_serves(M, N, K, epi)) {
     ti_set_error("gemm_bf16_normed: a weight of %d x %d is left to the norm's kernel and the product's", N, K);
     return 3;
   }
@@ -1782,7 +1790,7 @@ static bool pieces_serves(int M, int N, int K, int epi) {
 // shape alone, so that a row's bits do not depend on the rows beside it.
 static int pieces_splits(int N, int K, long partial_bytes) {
   const int n_pieces = (K + SP_PIECE - 1) / SP_PIECE;
-  if (n_pieces < 16) return 1;
+  if (n_pieces < 16) return 1;      // (from 8 pieces on: Qwen3-4B's and 8B's down projections lose 1-3 % of the step)
   const int grid = (N + 15) / 16;
   int ks = std::min(n_pieces / 4, (4 * compute_units() + grid - 1) / grid);
   while (ks > 1 && (long)ks * 16 * N * 4 > partial_bytes) --ks;
