@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model 0.6b|8b|32b] [--context N] [--prefill-tokens N]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model 0.6b|1.7b|4b|8b|14b|32b] [--context N] [--prefill-tokens N]
 
 The default run has the layer sizes of Qwen3-0.6B with random weights in
 bfloat16: a batch of 8 requests, each holding 2,048 cached tokens (filled by

@@ -886,12 +886,12 @@ def test_rmsnorm_that_adds_partial_sums(ops, rows, H, KS):
         assert (f64(out) - ref_rmsnorm(want_x, w, 1e-6)).abs().max() < (1e-5 if dtype == torch.float32 else 0.03)
 
 
-@pytest.mark.parametrize("tile", [1, 3, 5, 6])
+@pytest.mark.parametrize("tile", [1, 3, 5, 6, 8, 9])
 @pytest.mark.parametrize("M,N,K", [(300, 520, 128), (257, 384, 192), (130, 200, 64), (700, 96, 320)])
 def test_linear_bf16_every_tile(ops, tile, M, N, K):
     """Each tile of the pipelined kernel (256 x 128 with eight wavefronts, 128 x 64, 64 x 128 for the SwiGLU
-    epilogue, 64 x 64), whatever the dispatch would have chosen for the shape, with every epilogue, against
-    float64."""
+    epilogue, 64 x 64, and 128 x 160 and 256 x 160 with four wavefronts, which the SwiGLU epilogue does not
+    take), whatever the dispatch would have chosen for the shape, with every epilogue, against float64."""
     if not ops.use_fast_gemm:
         pytest.skip("bfloat16 MFMA kernels are switched off")
     lib = ops.lib("gemm_bf16")
@@ -962,6 +962,41 @@ def test_columns_split_between_two_tile_shapes(ops, M, N, K):
     gte, up = ref[:, :N // 2], ref[:, N // 2:]
     want = gte / (1 + torch.exp(-gte)) * up
     assert (f64(got[1][3]) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
+
+
+@pytest.mark.parametrize("M,N,K", [(2000, 5120, 64), (1990, 2560, 128), (4000, 2560, 64)])
+def test_widths_that_160_divides_take_tiles_of_160_columns(ops, M, N, K):
+    """Where tiles of 256 x 160 or 128 x 160 make whole rounds of the compute units the dispatch takes them
+    (widths of 2,560 and 5,120).  Same bits as without them, and the values of float64."""
+    if not ops.use_fast_gemm:
+        pytest.skip("bfloat16 MFMA kernels are switched off")
+    lib = ops.lib("gemm_bf16")
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    assert (-(-M // 256) * (N // 160)) % units == 0 or (-(-M // 128) * (N // 160)) % units == 0, "the shape does not take the rule"
+    g = torch.Generator().manual_seed(M + N)
+    a = (torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16)
+    w = (torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16)
+    base = torch.randn(M, N, generator=g)
+    ref = ref_linear(a, w)
+    got = {}
+    for on in (1, 0):
+        lib.ti_gemm_bf16_tiles_160(on)
+        try:
+            out = torch.empty(M, N, device="cuda")
+            ops.linear(dev(a), dev(w), out, "store")
+            added = dev(base.clone())
+            ops.linear(dev(a), dev(w), added, "add")
+            act = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+            ops.linear(dev(a), dev(w), act, "store_act")
+            got[on] = (out, added, act)
+        finally:
+            lib.ti_gemm_bf16_tiles_160(1)
+    for x, y in zip(got[1], got[0]):
+        assert torch.equal(x, y)
+    tol = 2e-5 * K
+    assert (f64(got[1][0]) - ref).abs().max() < tol
+    assert (f64(got[1][1]) - (ref + f64(base))).abs().max() < tol
+    assert (f64(got[1][2]) - ref).abs().max() < 0.005 * ref.abs().max() + tol
 
 
 @pytest.mark.parametrize("M", [17, 40, 64])

@@ -986,11 +986,12 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
       if (ks + 1 < PBK / 16) {
         read_step(ks + 1, set ^ 1);
         // all but the TM + TN reads just issued are done: this k-step's fragments are there
+        if (TM + TN == 7) asm volatile("s_waitcnt lgkmcnt(7)" ::: "memory");
         if (TM + TN == 6) asm volatile("s_waitcnt lgkmcnt(6)" ::: "memory");
         if (TM + TN == 4) asm volatile("s_waitcnt lgkmcnt(4)" ::: "memory");
         if (TM + TN == 3) asm volatile("s_waitcnt lgkmcnt(3)" ::: "memory");
         if (TM + TN == 2) asm volatile("s_waitcnt lgkmcnt(2)" ::: "memory");
-        static_assert(TM + TN == 6 || TM + TN == 4 || TM + TN == 3 || TM + TN == 2, "a wait for every tile shape");
+        static_assert(TM + TN == 7 || TM + TN == 6 || TM + TN == 4 || TM + TN == 3 || TM + TN == 2, "a wait for every tile shape");
       } else {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       }
@@ -1135,6 +1136,8 @@ static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, 
   return 0;
 }
 
+static int g_tiles_160 = 1;      // a hook for measurements: 0 = no tiles of 160 columns
+extern "C" void ti_gemm_bf16_tiles_160(int on) { g_tiles_160 = on; }
 static int g_two_ranges = 1;     // a hook for measurements: 0 = never split the columns between two tile shapes
 extern "C" void ti_gemm_bf16_two_ranges(int on) { g_two_ranges = on; }
 static int g_qkv_rows = 0;       // hooks for measurements: 128 or 256 forces the tile's rows;
@@ -1228,7 +1231,8 @@ extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K,
   return 0;
 }
 
-// for measurements: 0 = choose the tile by the shape, 1 = 256 x 128, 3 = 128 x 64, 5 = 64 x 128 (SwiGLU only), 6 = 64 x 64
+// for measurements: 0 = choose the tile by the shape, 1 = 256 x 128, 3 = 128 x 64, 5 = 64 x 128 (SwiGLU only), 6 = 64 x 64,
+// 8 = 128 x 160, 9 = 256 x 160 (neither for SwiGLU)
 static int g_force_tile = 0;
 extern "C" void ti_gemm_bf16_force_tile(int which) { g_force_tile = which; }
 
@@ -1253,12 +1257,26 @@ static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M,
   // at 64 rows 141 -> 115 us, 8B's 52 -> 45); a weight that gives it fewer workgroups than half the
   // units stays with the narrower tile (0.6B's: 10.0 against 10.6 us).
   if (SW && M <= 64 && (long)(N * cols + 127) / 128 * 2 >= compute_units()) tile = 5;
+  // Widths that 160 columns divide (2,560 and 5,120 among Qwen3's): where tiles of 256 x 160 or 128 x 160,
+  // four wavefronts of 64 x 160 or 32 x 160, make whole rounds of the units, they are taken: a workgroup
+  // to a unit, fewer LDS reads and bytes from memory per matrix instruction than 256 x 128 (Qwen3-32B's o
+  // and down over 2,048 rows, 8 x 32 tiles: 212 and 604 us -> 180 and 554; Qwen3-4B's, 16 x 16 tiles of
+  // 128 x 160: 88 and 170 -> 75 and 141).
+  if constexpr (!SW) {
+    if (!g_force_tile && g_tiles_160 && M > 64 && N % 160 == 0) {
+      const long cols160 = N / 160;
+      const long wg256 = (long)((M + 255) / 256) * cols160, wg128 = (long)((M + 127) / 128) * cols160;
+      auto whole = [&](long wg) { return wg >= units && (wg % units == 0 || wg % units >= units * 7 / 8); };
+      if (whole(wg256)) tile = 9;
+      else if (whole(wg128) && wg128 <= 2L * units) tile = 8;
+    }
+  }
   // 256 x 128 tiles that fill the units once or more and leave a round short of three quarters (Qwen3-32B's
   // o and down projections over 2,048 rows: 8 x 40 tiles on 256 units): the columns that make whole rounds
   // take those tiles, the rest 128 x 64 tiles in a launch of their own behind them, rather than everything
   // the smaller tile, which needs a third more time per flop (those projections 548 -> 420 us on average;
   // Qwen3-0.6B's gate/up, 8 x 48 tiles, likewise).
-  if (tile == 3 && big >= units && !g_force_tile && g_two_ranges) {
+  if (tile == 3 && big >= units && !g_force_tile && g_two_ranges) {   // (not where a 160-column tile was chosen)
     const int row_tiles = (M + 255) / 256;
     const int col_tiles = (int)(big / units * units / row_tiles);
     const int n_big = col_tiles * (128 / cols);         // output columns of the first range
@@ -1268,6 +1286,10 @@ static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M,
     }
   }
   if (g_force_tile) tile = g_force_tile;
+  if constexpr (!SW) {
+    if (tile == 8) return launch_pipelined<128, 160, 4, 1, EPI>(A, W, out, M, N, K, lda, s);
+    if (tile == 9) return launch_pipelined<256, 160, 4, 1, EPI>(A, W, out, M, N, K, lda, s);
+  }
   if (tile == 1) return launch_pipelined<256, 128, 4, 2, EPI>(A, W, out, M, N, K, lda, s);
   if constexpr (EPI == TI_EPI_SWIGLU)
     if (tile == 5) return launch_pipelined<64, 128, 2, 2, EPI>(A, W, out, M, N, K, lda, s);

@@ -5,8 +5,9 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
-void ti_gemm_bf16_force_tile(int which);      // 1: 256 x 128, 3: 128 x 64, 5: 64 x 128 (SwiGLU only), 6: 64 x 64
+void ti_gemm_bf16_force_tile(int which);      // 1: 256 x 128, 3: 128 x 64, 5: 64 x 128 (SwiGLU only), 6: 64 x 64, 8: 128 x 160, 9: 256 x 160
 void ti_gemm_bf16_normed_weight_below(long elements);  // weights of fewer elements keep the norm inside the product (0: the default)
+void ti_gemm_bf16_tiles_160(int on);          // 0: no tiles of 160 columns
 void ti_gemm_bf16_two_ranges(int on);         // 0: never split a product's columns between 256 x 128 and 128 x 64 tiles
 void ti_gemm_bf16_skinny_waves(int waves);    // 4 or 8 wavefronts in the kernel for M <= 64
 void ti_gemm_bf16_qkv_prep_min_rows(int rows); // the fewest rows ti_gemm_bf16_qkv_prep serves (17)
