@@ -1257,6 +1257,14 @@ static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M,
   // at 64 rows 141 -> 115 us, 8B's 52 -> 45); a weight that gives it fewer workgroups than half the
   // units stays with the narrower tile (0.6B's: 10.0 against 10.6 us).
   if (SW && M <= 64 && (long)(N * cols + 127) / 128 * 2 >= compute_units()) tile = 5;
+  // 65 to 520 rows (a portion of a prompt beside decoded tokens) times a large weight wait for the weight,
+  // and every tile of rows pulls all of it in again.  129 to 256 rows under a stacked [gate; up] weight take
+  // one 256-row tile, not two of 128 (Qwen3-8B's at 136 rows 89 -> 65 us, 32B's 185 -> 163, 4B's 48 -> 40);
+  // from 385 rows on 128 x 64 tiles, not 64 x 64 (8B's q/k/v, o and down at 520 rows 63, 42 and 132 ->
+  // 47, 39 and 104 us).  Small weights are not what such a step waits for: they stay as they were.
+  const bool large = (long)N * cols * K >= (8L << 20);
+  if (SW && large && M > 128 && M <= 256 && tile == 3) tile = 1;
+  if (!SW && large && M > 384 && tile == 6) tile = 3;
   // Widths that 160 columns divide (2,560 and 5,120 among Qwen3's): where tiles of 256 x 160 or 128 x 160,
   // four wavefronts of 64 x 160 or 32 x 160, make whole rounds of the units, they are taken: a workgroup
   // to a unit, fewer LDS reads and bytes from memory per matrix instruction than 256 x 128 (Qwen3-32B's o
@@ -1904,8 +1912,9 @@ extern "C" int ti_gemm_bf16_add_split(const void* A, const void* W, void* out, i
   // the chip, and they pull four bytes into a compute unit where a 128 x 128 tile pulls two.  When the
   // 128 x 128 tiles are at most half as many as the units, K is split between two to four workgroups
   // per tile instead: the same bytes as one round of 128 x 128 tiles, on all units.
+  // (not under a weight of 64 Mi elements or more: Qwen3-32B's down projection at 264 rows 164 -> 199 us)
   if (KS == 1 && !small && g_add_split && g_use_pipelined && defer && epi == TI_EPI_ADD_F32 && partial && M >= 256 &&
-      K % 64 == 0 && lda % 8 == 0 && !((uintptr_t)A & 15) && !((uintptr_t)W & 15) && !((uintptr_t)partial & 15)) {
+      (long)N * K < (64L << 20) && K % 64 == 0 && lda % 8 == 0 && !((uintptr_t)A & 15) && !((uintptr_t)W & 15) && !((uintptr_t)partial & 15)) {
     const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     int ks = (int)std::min<long>(4, compute_units() / std::max<long>(1, tiles128));
     while (ks > 1 && ((K / 64) / ks < 8 || (long)ks * M * N * 4 > partial_bytes)) --ks;
