@@ -41,6 +41,12 @@ CONFIGS = {
               num_attention_heads=16, num_key_value_heads=8, head_dim=128, intermediate_size=3072,
               vocab_size=1500, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
               attention_bias=False, hidden_act="silu", max_position_embeddings=4096),
+    # one layer with the widths of Qwen3-4B: 2,560 is no multiple of 1,024 (other tiles of the products:
+    # 160 columns wide), 32 query heads on 8 kv heads, a feed-forward of 9,728
+    "F": dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=1, hidden_size=2560,
+              num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=9728,
+              vocab_size=1200, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+              attention_bias=False, hidden_act="silu", max_position_embeddings=4096),
 }
 
 

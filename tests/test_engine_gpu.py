@@ -323,6 +323,33 @@ def test_layers_of_real_width_match_plain(model_folders, dtype):
         assert err < tol, (r, err, tol)
 
 
+def test_a_layer_of_another_real_width_matches_plain(model_folders):
+    """One layer with the widths of Qwen3-4B in bfloat16: a prompt of 2,048 tokens whole (its o and down
+    projections take tiles of 128 x 160), seven short requests beside its first decoded token, then six steps
+    of all eight (products of 8 rows under weights of 2,560 and 9,728 columns), against the plain model."""
+    folder = model_folders("F", "bfloat16", True)
+    V = CONFIGS["F"]["vocab_size"]
+    requests = {"a": random_tokens(2055, V, 61)}
+    requests.update({f"s{i}": random_tokens(9, V, 70 + i) for i in range(7)})
+    want, tol = plain_logits(folder, requests, "bfloat16")
+    a = requests["a"]
+    shorts = [r for r in requests if r != "a"]
+    trace = [{"entries": [("a", a[:2048], [0, 1000, 2047])], "end": []},
+             {"entries": [("a", a[2048:2049], [0])] + [(r, requests[r][:3], [2]) for r in shorts], "end": []}]
+    for k in range(6):
+        trace.append({"entries": [("a", a[2049 + k:2050 + k], [0])] + [(r, requests[r][3 + k:4 + k], [0]) for r in shorts], "end": []})
+    trace[-1]["end"] = list(requests)
+    from tinyinfer_amd.engine import Engine
+    engine = Engine.from_folder(folder, "bfloat16", page_size=16, max_tokens=2048 + 64 + 7 * 16, max_requests=8, max_seq=2112)
+    got = replay(engine, trace)
+    rows = {"a": [0, 1000, 2047] + list(range(2048, 2055))}
+    rows.update({r: list(range(2, 9)) for r in shorts})
+    for r in requests:
+        err = np.abs(got[r] - want[r][rows[r]]).max()
+        print(f"\n[F bfloat16 {r}] max |engine - plain| = {err:.3e} (allowed {tol:.3e})")
+        assert err < tol, (r, err, tol)
+
+
 def test_steps_of_17_to_64_tokens_at_real_width(model_folders):
     """Steps of 17 to 64 tokens at the widths of Qwen3-0.6B: the products into the residual split
     K over workgroups and leave their partial sums to the norm that follows (the last one to a
