@@ -462,6 +462,91 @@ def test_sample_frequencies(ops):
     assert chi2 < 40.0          # 11 degrees of freedom: P(chi2 > 40) < 4e-5
 
 
+def check_draws(row, T, top_k, top_p, us, got):
+    """Every draw lies in its token's interval of the plain sampler's CDF (32-bit rounding of the running sums aside)."""
+    from plain.qwen3_plain import sample_distribution
+    p = sample_distribution(row.double().numpy(), T, top_k, top_p)
+    c = np.cumsum(p)
+    for u, tok in zip(us, got):
+        assert 0 <= tok < row.numel() and p[tok] > 0, (T, top_k, top_p, u, tok)
+        assert c[tok] - p[tok] - 1e-4 <= u <= c[tok] + 1e-4, (T, top_k, top_p, u, tok, c[tok] - p[tok], c[tok])
+
+
+def test_sample_of_a_long_row_by_many_workgroups(ops):
+    """A row of the real vocabulary's length, whose top-k cut is found by radix with many workgroups a row:
+    the draws lie where the plain sampler's CDF puts them, and are those of the one workgroup that walks the
+    row bit by bit, for cuts in the positive and in the negative logits, equal logits at the cut, NaN
+    in the row and greedy rows beside drawn ones; a second call finds the workspace as the first left it."""
+    g = torch.Generator().manual_seed(11)
+    V = 151936
+    us = np.linspace(0.003, 0.997, 24).astype(np.float32)
+    row = torch.randn(V, generator=g) * 3
+    row[1000:1040] = row[7]                                  # equal logits, far apart from the first of them
+    row[5] = float("nan")
+    row[150000] = float("nan")
+    low = -row.abs() - 0.5                                   # every logit negative
+    low[5] = low[150000] = 0.0
+    low[5] = float("nan")
+    for r in (row, low):
+        logits = dev(r[None, :].repeat(len(us), 1))
+        for T, top_k, top_p in ((0.8, 512, 1.0), (1.0, 50, 1.0), (0.7, 512, 0.9), (1.3, 20, 0.95), (1.0, 1, 1.0),
+                                (2.0, 3000, 0.999), (1.0, 2, 0.5)):
+            got = run_sample(ops, logits, T, top_k, top_p, us.tolist())
+            check_draws(r.nan_to_num(nan=-1e30), T, top_k, top_p, us, got)
+            ops.use_radix_sample = False
+            try:
+                walked = run_sample(ops, logits, T, top_k, top_p, us.tolist())
+            finally:
+                ops.use_radix_sample = True
+            differ = sum(a != b for a, b in zip(got, walked))
+            assert differ <= 1, (T, top_k, top_p, got, walked)      # a sum taken in another order may move one edge
+    # the cut lands in 40 equal logits: all of them stay
+    tie = torch.randn(V, generator=g)
+    tie[20000:20040] = 4.0
+    tie[3] = 9.0
+    big = tie > 4.0
+    k = int(big.sum()) + 5
+    got = run_sample(ops, dev(tie[None, :].repeat(len(us), 1)), 1.0, k, 1.0, us.tolist())
+    check_draws(tie, 1.0, k, 1.0, us, got)
+    assert any(20000 <= t < 20040 for t in got)
+    # rows of different kinds in one call
+    n = 6
+    logits = torch.randn(n, V, generator=g) * 2
+    logits[2] = float("nan")                                 # nothing to draw from: index 0
+    logits[3, :] = 1.5                                       # all equal: every index stays, far more than are collected
+    temp = torch.tensor([0.0, 1.0, 1.0, 1.0, 0.0, 0.9])
+    top_k = torch.tensor([7, 40, 40, 40, 0, 3500], dtype=torch.int32)
+    top_p = torch.tensor([1.0, 0.8, 1.0, 1.0, 1.0, 0.97])
+    u = torch.tensor([0.5, 0.31, 0.9, 0.25, 0.1, 0.77])
+    out = torch.empty(n, dtype=torch.int32, device="cuda")
+    for _ in range(2):
+        ops.sample(dev(logits), dev(temp), dev(top_k), dev(top_p), dev(u), out)
+        got = out.tolist()
+        assert got[0] == int(logits[0].argmax()) and got[4] == int(logits[4].argmax())
+        assert got[2] == 0
+        assert got[3] == int(0.25 * V)
+        check_draws(logits[1], 1.0, 40, 0.8, [0.31], [got[1]])
+        check_draws(logits[5], 0.9, 3500, 0.97, [0.77], [got[5]])
+    # a cut beyond what the radix kernels hold goes the long way, with the same meaning
+    got = run_sample(ops, dev(row[None, :].repeat(4, 1)), 1.0, 5000, 1.0, us[:4].tolist())
+    check_draws(row.nan_to_num(nan=-1e30), 1.0, 5000, 1.0, us[:4], got)
+
+
+def test_sample_with_more_equal_logits_at_the_cut_than_are_collected(ops):
+    """6,000 equal logits at the cut are more pairs than a row collects: the row is walked instead, and the
+    next call, which is served, finds the workspace clean."""
+    g = torch.Generator().manual_seed(12)
+    V = 40000
+    row = torch.randn(V, generator=g)
+    row[10000:16000] = 2.0
+    us = np.linspace(0.01, 0.99, 16).astype(np.float32)
+    k = int((row > 2.0).sum()) + 10
+    got = run_sample(ops, dev(row[None, :].repeat(16, 1)), 1.0, k, 1.0, us.tolist())
+    check_draws(row, 1.0, k, 1.0, us, got)
+    got = run_sample(ops, dev(row[None, :].repeat(16, 1)), 1.0, 30, 1.0, us.tolist())
+    check_draws(row, 1.0, 30, 1.0, us, got)
+
+
 # ------------------------------------------------- bfloat16 matrix-core products
 @pytest.mark.parametrize("M,N,K", [
     (1, 48, 64), (5, 261, 1024), (8, 1000, 96), (16, 17, 200), (17, 130, 72), (33, 64, 3072), (64, 151, 256),

@@ -137,9 +137,13 @@ int ti_argmax(const float* logits, int* out, void* scratch, int n_rows, int V, h
 // allocating routine; calls that overlap on one GPU share the array and race.  The reference has no
 // counterpart (its argmax needs no scratch: /root/reference/src/cuda/sample.cu:13-54).
 int ti_argmax_static(const float* logits, int* out, int n_rows, int V, hipStream_t stream);
-// temperature, top-k (0: all), top-p and one uniform number per row
+// temperature, top-k (0: all), top-p and one uniform number per row.  scratch: ti_sample_scratch_bytes(n_rows)
+// bytes, zero before the first call and touched by nothing else since (the kernels leave them at zero; calls
+// that overlap on one workspace race), or null: then one workgroup walks a whole row, as it does for the rows
+// that have no top-k cut.
+long ti_sample_scratch_bytes(int n_rows);
 int ti_sample(const float* logits, const float* temp, const int* top_k, const float* top_p, const float* uni, int* out,
-              int n_rows, int V, hipStream_t stream);
+              void* scratch, int n_rows, int V, hipStream_t stream);
 
 
 // ---- libti_measure: what the GPU delivers, for the bench tool's fractions

@@ -1007,6 +1007,7 @@ int ti_ops_switch(void* ops_, const char* name_, int value, int* old) {
   else if (name == "fused_qkv_prefill") flag(ops.use.fused_qkv_prefill);
   else if (name == "split_k_add") flag(ops.use.split_k_add);
   else if (name == "early_page_ids") flag(ops.use.early_page_ids);
+  else if (name == "radix_sample") flag(ops.use.radix_sample);
   else if (name == "deferred_add") flag(ops.use.deferred_add);
   else if (name == "paired_prefill") flag(ops.use.paired_prefill);
   else if (name == "portion_splits") flag(ops.use.portion_splits);

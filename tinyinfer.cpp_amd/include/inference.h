@@ -316,6 +316,7 @@ class Ops {
     bool fast_gemm = true, fast_attention = true, fused_norm = true, fused_qk_decode = true, fused_qkv_prefill = true;
     bool split_k_add = true, deferred_add = true, paired_prefill = true, portion_splits = true;
     bool early_page_ids = true;     // a step of single tokens: the decode attention fetches a row's page ids beside its position
+    bool radix_sample = true;       // draws with a top-k cut: many workgroups share a row (else one walks it bit by bit)
     int force_paired_tiles = -1;    // 1 / 0: that kernel with / without pairs, whatever the launch
     int force_decode_splits = 0;    // > 0: the decode attention cuts every context into this many runs
   } use;
@@ -329,6 +330,7 @@ class Ops {
   int units_ = 0;
   DeviceBuffer partials_;
   DeviceBuffer argmax_scratch_;
+  DeviceBuffer sample_scratch_;       // zero between calls
   struct { void* out = nullptr; int64_t count = 0; int splits = 0; } pending_;
   struct Timing;
   friend struct TimedScope;

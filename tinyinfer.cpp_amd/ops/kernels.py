@@ -93,7 +93,8 @@ class NormedRows:
 _SWITCHES = {"use_fast_gemm": "fast_gemm", "use_fast_attention": "fast_attention", "use_fused_norm": "fused_norm",
              "use_fused_qk_decode": "fused_qk_decode", "use_fused_qkv_prefill": "fused_qkv_prefill",
              "use_split_k_add": "split_k_add", "use_deferred_add": "deferred_add", "use_paired_prefill": "paired_prefill",
-             "use_portion_splits": "portion_splits", "use_early_page_ids": "early_page_ids"}
+             "use_portion_splits": "portion_splits", "use_early_page_ids": "early_page_ids",
+             "use_radix_sample": "radix_sample"}
 _LIB_OF = {"embed": "core", "rmsnorm": "core", "rope_neox": "core", "rope_table": "core", "qk_norm_rope_kv_write": "core",
            "qk_norm_inplace": "core", "argmax": "sampling", "sample": "sampling", "attention_rows": "attention_generic",
            "fill_random": "core", "fill_zero": "core"}

@@ -793,7 +793,18 @@ void Ops::sample(const Tensor& logits, const float* temperature, const int* top_
   TIMED("sample " + dims(logits));
   require(logits.ndim == 2 && logits.dtype == DType::F32 && logits.contiguous(),
           "sample: logits must be contiguous float32 [n, V]");
-  int rc = KERNEL("sampling", ti_sample)((const float*)logits.data, temperature, top_k, top_p, uniform, out,
+  void* scratch = nullptr;
+  if (use.radix_sample) {
+    const int64_t rows = std::max<int64_t>(logits.shape[0], 8);
+    const size_t need = (size_t)KERNEL("sampling", ti_sample_scratch_bytes)((int)rows);
+    if (sample_scratch_.bytes() < need) {
+      flush();
+      sample_scratch_ = DeviceBuffer(need);
+      fill_zero(sample_scratch_.data(), need);     // the kernels leave it at zero
+    }
+    scratch = sample_scratch_.data();
+  }
+  int rc = KERNEL("sampling", ti_sample)((const float*)logits.data, temperature, top_k, top_p, uniform, out, scratch,
                                          (int)logits.shape[0], (int)logits.shape[1], (hipStream_t)launch_stream());
   check("sampling", rc, "sample");
 }
