@@ -6,9 +6,10 @@
 // Temperature sampling draws by inverse CDF over the index order from one
 // uniform number per row, which the host derives from (seed, request, number of
 // tokens generated), so a draw does not depend on what else is in the batch.
-// The cuts are found without sorting: the k-th largest logit, and the logit at
-// which the descending cumulative mass reaches top_p, each by 32 steps of
-// bisection over the order-preserving integer image of the floats; every sum is
+// The cuts are the k-th largest logit and the logit at which the descending
+// cumulative mass reaches top_p, both found on the order-preserving integer
+// image of the floats: by radix with many workgroups a row where there is a
+// top-k cut, else by 32 steps of bisection each in one workgroup.  Every sum is
 // reduced in a fixed order, so the result is reproducible.
 #include <algorithm>
 #include <mutex>
@@ -283,8 +284,9 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temp, 
 #define S_BINS 2048
 #define S_CAND 4096                              // pairs a row may collect (and the finish sorts in LDS)
 #define S_MAX_K 3584                             // the largest cut served: room for equals and prefix-mates
+#define S_LOADS 8                                // loads of a thread that are under way at a time
 #define S_STAGE 512                              // pairs a workgroup gathers in LDS before it asks for room
-#define S_HEAD_WORDS (2 * S_BINS + 64)           // two histograms, the count of pairs (and padding)
+#define S_HEAD_WORDS (2 * S_BINS + 64)           // two histograms, the count of pairs, pass 1's bin (and padding)
 #define S_ROW_WORDS (S_HEAD_WORDS + 2 * S_CAND)
 
 __device__ __forceinline__ float key_value(uint32_t key) {
@@ -353,7 +355,7 @@ template <int PASS>
 __global__ void __launch_bounds__(256)
 sample_pass_kernel(const float* __restrict__ logits, const float* __restrict__ temp, const int* __restrict__ top_k,
                    int* __restrict__ scratch, int V) {
-  __shared__ int s_hist[S_BINS];
+  __shared__ int s_hist[PASS == 2 ? 1 : S_BINS];
   __shared__ unsigned long long s_stage[PASS == 2 ? S_STAGE : 1];
   __shared__ int s_sum[256], s_above[257], s_res[2], s_count, s_base;
   const int r = blockIdx.y;
@@ -365,11 +367,15 @@ sample_pass_kernel(const float* __restrict__ logits, const float* __restrict__ t
   int* n_cand = hist2 + S_BINS;
   unsigned long long* cand = reinterpret_cast<unsigned long long*>(hist1 + S_HEAD_WORDS);
   int b1 = 0, above1 = 0, b2 = 0, above2 = 0;
-  if (PASS >= 1) {
+  if (PASS == 1) {
     bin_of_kth(hist1, k, s_sum, s_above, s_res, b1, above1);
+    if (blockIdx.x == 0 && threadIdx.x == 0) n_cand[1] = b1, n_cand[2] = above1;   // pass 2 need not look again
     if (b1 < 0) return;                            // a row of NaN
   }
   if (PASS == 2) {
+    b1 = n_cand[1];
+    above1 = n_cand[2];
+    if (b1 < 0) return;
     bin_of_kth(hist2, k - above1, s_sum, s_above, s_res, b2, above2);
     if (b2 < 0) return;
     if (threadIdx.x == 0) s_count = 0;
@@ -379,22 +385,29 @@ sample_pass_kernel(const float* __restrict__ logits, const float* __restrict__ t
     __syncthreads();
   }
   const uint32_t prefix = ((uint32_t)b1 << 11) | (uint32_t)b2;
-  for (int i = blockIdx.x * 256 + threadIdx.x; i < V; i += gridDim.x * 256) {
-    const float v = row[i];
-    if (!(v == v)) continue;                       // NaN is never drawn
-    const uint32_t key = order_key(v);
-    if (PASS == 0) {
-      atomicAdd(&s_hist[key >> 21], 1);
-    } else if (PASS == 1) {
-      if ((key >> 21) == (uint32_t)b1) atomicAdd(&s_hist[(key >> 10) & (S_BINS - 1)], 1);
-    } else if ((key >> 10) >= prefix) {
-      const unsigned long long pair = ((unsigned long long)key << 32) | (uint32_t)~i;
-      const int at = atomicAdd(&s_count, 1);
-      if (at < S_STAGE) {
-        s_stage[at] = pair;
-      } else {                                     // more than the stage holds: one by one
-        const int g = atomicAdd(n_cand, 1);
-        if (g < S_CAND) cand[g] = pair;
+  // S_LOADS loads are under way at a time: one load a turn leaves a wavefront waiting for memory 37 times over
+  for (int base = blockIdx.x * (256 * S_LOADS) + threadIdx.x; base < V; base += gridDim.x * (256 * S_LOADS)) {
+    float v[S_LOADS];
+#pragma unroll
+    for (int u = 0; u < S_LOADS; ++u) v[u] = base + 256 * u < V ? row[base + 256 * u] : __uint_as_float(0x7fc00000u);
+#pragma unroll
+    for (int u = 0; u < S_LOADS; ++u) {
+      if (!(v[u] == v[u])) continue;               // NaN is never drawn
+      const int i = base + 256 * u;
+      const uint32_t key = order_key(v[u]);
+      if (PASS == 0) {
+        atomicAdd(&s_hist[key >> 21], 1);
+      } else if (PASS == 1) {
+        if ((key >> 21) == (uint32_t)b1) atomicAdd(&s_hist[(key >> 10) & (S_BINS - 1)], 1);
+      } else if ((key >> 10) >= prefix) {
+        const unsigned long long pair = ((unsigned long long)key << 32) | (uint32_t)~i;
+        const int at = atomicAdd(&s_count, 1);
+        if (at < S_STAGE) {
+          s_stage[at] = pair;
+        } else {                                   // more than the stage holds: one by one
+          const int g = atomicAdd(n_cand, 1);
+          if (g < S_CAND) cand[g] = pair;
+        }
       }
     }
   }
@@ -412,8 +425,25 @@ sample_pass_kernel(const float* __restrict__ logits, const float* __restrict__ t
   }
 }
 
-// sorts a[0..n) of LDS downwards, n <= S_CAND; every thread of the workgroup calls it
-__device__ void sort_down(unsigned long long* a, int n) {
+// sorts a[0..n) of LDS downwards, n <= S_CAND, no two entries equal; every thread of the workgroup calls it.
+// Up to S_BY_RANK entries each thread counts the entries above its own and puts it there (n reads that the
+// whole wavefront shares, no barrier between them); more are sorted by a bitonic network, a barrier a stage.
+// tmp: room for S_BY_RANK entries.
+#define S_BY_RANK 1024
+__device__ void sort_down(unsigned long long* a, int n, unsigned long long* tmp) {
+  if (n <= S_BY_RANK) {
+    const int i = threadIdx.x;
+    if (i < n) {
+      const unsigned long long x = a[i];
+      int above = 0;
+      for (int j = 0; j < n; ++j) above += a[j] > x ? 1 : 0;
+      tmp[above] = x;
+    }
+    __syncthreads();
+    if (i < n) a[i] = tmp[i];
+    __syncthreads();
+    return;
+  }
   int p2 = 1;
   while (p2 < n) p2 <<= 1;
   for (int i = n + threadIdx.x; i < p2; i += SNT) a[i] = 0ull;     // below every pair
@@ -509,7 +539,7 @@ sample_finish_kernel(const float* __restrict__ logits, const float* __restrict__
   }
   for (int i = threadIdx.x; i < n; i += SNT) s_pair[i] = cand[i];
   __syncthreads();
-  sort_down(s_pair, n);                            // by (key, ~index): of equal logits the lowest index first
+  sort_down(s_pair, n, reinterpret_cast<unsigned long long*>(s_w));                            // by (key, ~index): of equal logits the lowest index first
   const float T = temp[r];
   if (!(T > 0.f)) {
     if (threadIdx.x == 0) out[r] = (int)~(uint32_t)s_pair[0];
@@ -538,7 +568,7 @@ sample_finish_kernel(const float* __restrict__ logits, const float* __restrict__
     s_pair[i] = (pr << 32) | (pr >> 32);           // (~index, key)
   }
   __syncthreads();
-  sort_down(s_pair, m);
+  sort_down(s_pair, m, reinterpret_cast<unsigned long long*>(s_w));
   for (int i = threadIdx.x; i < m; i += SNT) s_w[i] = expf((key_value((uint32_t)s_pair[i]) - mx) * inv_t);
   __syncthreads();
   const float target = uni[r] * scan_in_place(s_w, m, s_wave);
@@ -620,8 +650,8 @@ extern "C" int ti_sample(const float* logits, const float* temp, const int* top_
   if (!scratch) {
     sample_kernel<<<n_rows, SNT, 0, stream>>>(logits, temp, top_k, top_p, uni, out, V);
   } else {
-    const int most = n_rows <= 8 ? 64 : (n_rows <= 32 ? 32 : 16);
-    const dim3 grid(std::min(most, (V + 255) / 256), n_rows);
+    const int most = n_rows <= 8 ? 80 : (n_rows <= 32 ? 32 : 16), span = 256 * S_LOADS;
+    const dim3 grid(std::min(most, (V + span - 1) / span), n_rows);
     sample_pass_kernel<0><<<grid, 256, 0, stream>>>(logits, temp, top_k, (int*)scratch, V);
     sample_pass_kernel<1><<<grid, 256, 0, stream>>>(logits, temp, top_k, (int*)scratch, V);
     sample_pass_kernel<2><<<grid, 256, 0, stream>>>(logits, temp, top_k, (int*)scratch, V);
