@@ -32,13 +32,13 @@ def required_libraries(dtype: str):
 
 
 def header_signatures(text: str) -> Dict[str, tuple]:
-    """{function: (restype, [argtypes])} of the `int ti_...(...)` and `void ti_...(...)`
+    """{function: (restype, [argtypes])} of the `int ti_...(...)`, `long ti_...(...)` and `void ti_...(...)`
     declarations of a kernels' header: pointers and streams as void pointers, int, long and
     float as themselves.  A declaration with any other type raises."""
     import re
     text = re.sub(r"//[^\n]*", "", text)
     out = {}
-    for ret, name, args in re.findall(r"\b(int|void)\s+(ti_\w+)\s*\(([^)]*)\)\s*;", text):
+    for ret, name, args in re.findall(r"\b(int|long|void)\s+(ti_\w+)\s*\(([^)]*)\)\s*;", text):
         types = []
         for arg in (a.strip() for a in args.split(",")):
             if not arg or arg == "void":
@@ -51,7 +51,7 @@ def header_signatures(text: str) -> Dict[str, tuple]:
             if len(words) < 2 or kind not in _C_TYPES:
                 raise KernelError(f"tinyinfer_kernels.h: cannot read the argument {arg!r} of {name}")
             types.append(_C_TYPES[kind])
-        out[name] = (ctypes.c_int if ret == "int" else None, types)
+        out[name] = ({"int": ctypes.c_int, "long": ctypes.c_long, "void": None}[ret], types)
     return out
 
 
