@@ -126,14 +126,15 @@ def fill(engine, rids, context, rng, chunk=4096):
     torch.cuda.synchronize()
 
 
-def measure_decode(engine, sampler, batch, steps, warmup, context, rng, tag, kernel_times=False):
-    """tokens/s and ms/step of `steps` decode steps at `batch`, every request at `context` tokens."""
+def measure_decode(engine, sampler, batch, steps, warmup, context, rng, tag, kernel_times=False, draw=None):
+    """tokens/s and ms/step of `steps` decode steps at `batch`, every request at `context` tokens.
+    draw: (temperature, top_k, top_p) for the sampler, or None for the greedy choice."""
     import torch
     from tinyinfer_amd.engine import StepEntry, token_from_feedback
     from tinyinfer_amd.sampling import SamplingParams
     rids = [f"{tag}{i}" for i in range(batch)]
     fill(engine, rids, context, rng)
-    greedy = [SamplingParams()] * batch
+    greedy = [SamplingParams(draw[0], draw[1], draw[2], 1) if draw else SamplingParams()] * batch
     nums = list(range(batch))
     last = rng.integers(0, engine.model.vocab_size, size=batch).tolist()
 
@@ -247,6 +248,9 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048, help="cached tokens each decoding request holds")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--temperature", type=float, default=0.0, help="decode draws its tokens at this temperature (0: greedy)")
+    ap.add_argument("--top-k", type=int, default=0, help="with --temperature: the sampler's cut (0: its default, 512)")
+    ap.add_argument("--top-p", type=float, default=1.0, help="with --temperature: the sampler's top-p")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--no-peaks", action="store_true", help="skip measuring the GPU's read bandwidth and MFMA rate")
     ap.add_argument("--kernel-times", action="store_true", help="a table of the decode step's calls, timed with events")
@@ -294,6 +298,7 @@ def main() -> int:
                                     "decode_context": context, "model": NAMES[args.model]}}), flush=True)
         return 0
     p_s = tps = ms = None
+    draw = (args.temperature, args.top_k, args.top_p) if args.temperature > 0 else None
     if args.only != "decode":
         say(f"prefill of {prefill_tokens} tokens ...")
         p_s = measure_prefill(engine, rng, prefill_tokens)
@@ -306,7 +311,7 @@ def main() -> int:
     if args.only != "prefill":
         say(f"decode at batch {args.batch} ...")
         tps, ms, table = measure_decode(engine, sampler, args.batch, args.steps, args.warmup, context, rng, "m",
-                                        args.kernel_times)
+                                        args.kernel_times, draw)
         if table:
             print_table(table, f"a decode step at batch {args.batch}, call by call (not from the graph):")
     points = {}
@@ -314,7 +319,7 @@ def main() -> int:
         for b, k in ((1, args.steps), (64, max(16, args.steps // 4))):
             say(f"decode at batch {b} ...")
             points[f"decode_b{b}"] = round(measure_decode(engine, sampler, b, k, max(4, args.warmup // 2), context, rng,
-                                                          f"p{b}_")[0], 1)
+                                                          f"p{b}_", draw=draw)[0], 1)
 
     ctx_mean = context + args.warmup + args.steps / 2.0
     step_bytes = nums["weight_bytes"] + args.batch * ctx_mean * nums["kv_bytes_per_token"]
@@ -342,7 +347,8 @@ def main() -> int:
                    "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
                    "tied_head": bool(cfg["tie_word_embeddings"]),
                    "global_batch": args.batch, "cached_tokens": context, "seq_len": max_seq, "page_size": PAGE,
-                   "prefill_tokens": prefill_tokens, "parallelism": "single GPU", "decode_graph": True},
+                   "prefill_tokens": prefill_tokens, "parallelism": "single GPU", "decode_graph": True,
+                   "sampling": f"temperature {args.temperature} top-k {args.top_k or 512} top-p {args.top_p}" if draw else "greedy"},
         "prefill": prefill, "roofline": roofline, "points": points,
     }
     print(json.dumps(out), flush=True)

@@ -425,19 +425,24 @@ sample_pass_kernel(const float* __restrict__ logits, const float* __restrict__ t
   }
 }
 
-// sorts a[0..n) of LDS downwards, n <= S_CAND, no two entries equal; every thread of the workgroup calls it.
-// Up to S_BY_RANK entries each thread counts the entries above its own and puts it there (n reads that the
-// whole wavefront shares, no barrier between them); more are sorted by a bitonic network, a barrier a stage.
-// tmp: room for S_BY_RANK entries.
+// sorts a[0..n) of LDS downwards by the entries' upper words, n <= S_CAND; every thread of the workgroup
+// calls it.  Up to S_BY_RANK entries each thread counts the entries above its own and puts it there (n reads
+// that the whole wavefront shares, a compare and an add each, no barrier between them); entries with equal
+// upper words take neighbouring places in the order in which they come.  More entries are sorted by a
+// bitonic network on the whole entries, a barrier a stage.  tmp: room for S_BY_RANK entries and as many counters.
 #define S_BY_RANK 1024
 __device__ void sort_down(unsigned long long* a, int n, unsigned long long* tmp) {
   if (n <= S_BY_RANK) {
+    int* taken = reinterpret_cast<int*>(tmp + S_BY_RANK);
     const int i = threadIdx.x;
+    if (i < n) taken[i] = 0;
+    __syncthreads();
     if (i < n) {
       const unsigned long long x = a[i];
+      const uint32_t mine = (uint32_t)(x >> 32);
       int above = 0;
-      for (int j = 0; j < n; ++j) above += a[j] > x ? 1 : 0;
-      tmp[above] = x;
+      for (int j = 0; j < n; ++j) above += (uint32_t)(a[j] >> 32) > mine ? 1 : 0;
+      tmp[above + atomicAdd(&taken[above], 1)] = x;
     }
     __syncthreads();
     if (i < n) a[i] = tmp[i];
@@ -523,6 +528,7 @@ sample_finish_kernel(const float* __restrict__ logits, const float* __restrict__
     sample_row_by_bisection(logits, temp, top_k, top_p, uni, out, V, r);
     return;
   }
+  const float T = temp[r], p_keep = top_p[r], u = uni[r];
   int* head = scratch + (size_t)r * S_ROW_WORDS;
   const unsigned long long* cand = reinterpret_cast<const unsigned long long*>(head + S_HEAD_WORDS);
   const int n = head[2 * S_BINS];
@@ -539,16 +545,18 @@ sample_finish_kernel(const float* __restrict__ logits, const float* __restrict__
   }
   for (int i = threadIdx.x; i < n; i += SNT) s_pair[i] = cand[i];
   __syncthreads();
-  sort_down(s_pair, n, reinterpret_cast<unsigned long long*>(s_w));                            // by (key, ~index): of equal logits the lowest index first
-  const float T = temp[r];
-  if (!(T > 0.f)) {
-    if (threadIdx.x == 0) out[r] = (int)~(uint32_t)s_pair[0];
+  sort_down(s_pair, n, reinterpret_cast<unsigned long long*>(s_w));                            // by key
+  if (!(T > 0.f)) {                                // of equal logits the lowest index
+    const uint32_t top = (uint32_t)(s_pair[0] >> 32);
+    for (int i = threadIdx.x; i < n; i += SNT)
+      if ((uint32_t)(s_pair[i] >> 32) == top) atomicMin(&s_at, (int)~(uint32_t)s_pair[i]);
+    __syncthreads();
+    if (threadIdx.x == 0) out[r] = s_at;
     return;
   }
   int m = pairs_at_least(s_pair, n, (uint32_t)(s_pair[min(k, n) - 1] >> 32), &s_n);
   const float mx = key_value((uint32_t)(s_pair[0] >> 32));
   const float inv_t = 1.0f / T;
-  const float p_keep = top_p[r];
   if (p_keep < 1.0f) {
     for (int i = threadIdx.x; i < m; i += SNT) s_w[i] = expf((key_value((uint32_t)(s_pair[i] >> 32)) - mx) * inv_t);
     __syncthreads();
@@ -571,7 +579,7 @@ sample_finish_kernel(const float* __restrict__ logits, const float* __restrict__
   sort_down(s_pair, m, reinterpret_cast<unsigned long long*>(s_w));
   for (int i = threadIdx.x; i < m; i += SNT) s_w[i] = expf((key_value((uint32_t)s_pair[i]) - mx) * inv_t);
   __syncthreads();
-  const float target = uni[r] * scan_in_place(s_w, m, s_wave);
+  const float target = u * scan_in_place(s_w, m, s_wave);
   for (int i = threadIdx.x; i < m; i += SNT)
     if (target < s_w[i]) atomicMin(&s_at, i);
   __syncthreads();

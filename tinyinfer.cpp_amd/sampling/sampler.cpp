@@ -32,8 +32,8 @@ float uniform(uint64_t seed, uint64_t request, uint64_t n_generated) {
 // it is still under way on the device.
 struct Sampler::Buffers {
   struct Turn {
-    float* f_host = nullptr;     // temperature | top_p | uniform
-    int* i_host = nullptr;       // top_k | ids read back
+    float* f_host = nullptr;     // temperature | top_p | uniform | top_k (as integers): one copy takes them to the device
+    int* i_host = nullptr;       // ids read back
     hipEvent_t read_back = nullptr;
     int n = 0;
     uint64_t ticket = 0;         // the call whose ids lie here (0: none)
@@ -42,7 +42,7 @@ struct Sampler::Buffers {
   int cap = 0;
   Turn turns[2];
   uint64_t issued = 0;
-  DeviceBuffer f_dev, i_dev, out_dev;
+  DeviceBuffer f_dev, out_dev;
   void free_host() {
     for (Turn& t : turns) {
       if (t.f_host) (void)hipHostFree(t.f_host);
@@ -82,12 +82,11 @@ uint64_t Sampler::sample_async(const Tensor& logits, const std::vector<SamplingP
     const int cap = std::max(64, 2 * n);
     b.free_host();
     for (Buffers::Turn& u : b.turns) {
-      hip_check(hipHostMalloc((void**)&u.f_host, (size_t)3 * cap * 4, hipHostMallocDefault), "hipHostMalloc");
-      hip_check(hipHostMalloc((void**)&u.i_host, (size_t)2 * cap * 4, hipHostMallocDefault), "hipHostMalloc");
+      hip_check(hipHostMalloc((void**)&u.f_host, (size_t)4 * cap * 4, hipHostMallocDefault), "hipHostMalloc");
+      hip_check(hipHostMalloc((void**)&u.i_host, (size_t)cap * 4, hipHostMallocDefault), "hipHostMalloc");
       if (!u.read_back) hip_check(hipEventCreateWithFlags(&u.read_back, hipEventDisableTiming), "hipEventCreate");
     }
-    b.f_dev = DeviceBuffer((size_t)3 * cap * 4);
-    b.i_dev = DeviceBuffer((size_t)cap * 4);
+    b.f_dev = DeviceBuffer((size_t)4 * cap * 4);
     b.out_dev = DeviceBuffer((size_t)cap * 4);
     b.cap = cap;
   }
@@ -102,17 +101,16 @@ uint64_t Sampler::sample_async(const Tensor& logits, const std::vector<SamplingP
       t.f_host[i] = params[i].temperature;
       t.f_host[cap + i] = params[i].top_p;
       t.f_host[2 * cap + i] = uniform(params[i].seed, (uint64_t)requests[i], (uint64_t)counters[i]);
-      t.i_host[i] = params[i].effective_top_k();
+      reinterpret_cast<int*>(t.f_host)[3 * cap + i] = params[i].effective_top_k();
     }
     // this turn's earlier call has been collected: its copies out of these pinned buffers have
     // finished.  The device copies are shared: the stream puts this call's behind the last call's kernel.
     ops_.flush();
-    hip_check(hipMemcpyAsync(b.f_dev.data(), t.f_host, (size_t)3 * cap * 4, hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
-    hip_check(hipMemcpyAsync(b.i_dev.data(), t.i_host, (size_t)cap * 4, hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+    hip_check(hipMemcpyAsync(b.f_dev.data(), t.f_host, (size_t)4 * cap * 4, hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
     const float* fd = (const float*)b.f_dev.data();
-    ops_.sample(logits, fd, (const int*)b.i_dev.data(), fd + cap, fd + 2 * cap, out);
+    ops_.sample(logits, fd, reinterpret_cast<const int*>(fd + 3 * cap), fd + cap, fd + 2 * cap, out);
   }
-  hip_check(hipMemcpyAsync(t.i_host + b.cap, out, (size_t)n * 4, hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+  hip_check(hipMemcpyAsync(t.i_host, out, (size_t)n * 4, hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
   hip_check(hipEventRecord(t.read_back, stream), "hipEventRecord");
   t.n = n;
   t.collected = false;
@@ -126,7 +124,7 @@ std::vector<int> Sampler::collect(uint64_t ticket) {
     if (t.ticket != ticket || t.collected) continue;
     hip_check(hipEventSynchronize(t.read_back), "hipEventSynchronize");
     t.collected = true;
-    const int* back = t.i_host + b.cap;
+    const int* back = t.i_host;
     return std::vector<int>(back, back + t.n);
   }
   throw KernelError("sample: no call with ticket " + std::to_string(ticket) + " is waiting to be collected");
