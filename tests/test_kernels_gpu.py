@@ -426,6 +426,15 @@ def test_sample_keeps_every_logit_equal_to_the_kth(ops):
     from plain.qwen3_plain import sample_distribution, draw
     p = sample_distribution(row[0].double().numpy(), 1.0, 2, 1.0)
     assert [draw(p, x) for x in u] == got
+    # -0 and +0 are equal logits too: a cut to the largest keeps both, by radix and by the walk
+    zeros = torch.tensor([[-1.0, -0.0, -2.0, 0.0, -3.0] + [-5.0] * 20])
+    for radix in (True, False):
+        ops.use_radix_sample = radix
+        try:
+            assert run_sample(ops, zeros.repeat(4, 1), 1.0, 1, 1.0, [0.1, 0.4, 0.6, 0.9]) == [1, 1, 3, 3]
+            assert run_sample(ops, zeros.repeat(2, 1), 0.0, 0, 1.0, [0.1, 0.9]) == [1, 1]      # greedy: the lowest index
+        finally:
+            ops.use_radix_sample = True
 
 
 def test_sample_matches_inverse_cdf(ops):

@@ -22,7 +22,8 @@ TI_ERROR_API
 #define SNT 1024
 
 __device__ __forceinline__ uint32_t order_key(float f) {
-  const uint32_t u = __float_as_uint(f);
+  uint32_t u = __float_as_uint(f);
+  if (u == 0x80000000u) u = 0u;                  // -0 and +0 are equal logits
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
