@@ -49,6 +49,27 @@ CONFIGS = {
               attention_bias=False, hidden_act="silu", max_position_embeddings=4096),
 }
 
+# Shapes at the edges of what a configuration may say: the largest and the smallest head, one head per group and
+# seventeen, a window on every layer, widths that are multiples of 8 only, an odd vocabulary.  Used in one way of
+# cutting the work each (tests/test_engine_gpu.py).
+_ODD = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", rope_theta=10000.0, rms_norm_eps=1e-6,
+            tie_word_embeddings=True, attention_bias=False, hidden_act="silu", max_position_embeddings=4096)
+ODD_CONFIGS = {
+    "head 256": dict(_ODD, num_hidden_layers=2, hidden_size=72, num_attention_heads=2, num_key_value_heads=1, head_dim=256,
+                     intermediate_size=100, vocab_size=301),
+    "head 16": dict(_ODD, num_hidden_layers=5, hidden_size=56, num_attention_heads=7, num_key_value_heads=7, head_dim=16,
+                    intermediate_size=24, vocab_size=97, rms_norm_eps=1e-4),
+    "head 80, a window of 5 everywhere": dict(_ODD, num_hidden_layers=2, hidden_size=128, num_attention_heads=4,
+                                              num_key_value_heads=2, head_dim=80, intermediate_size=192, vocab_size=513,
+                                              use_sliding_window=True, sliding_window=5, max_window_layers=0),
+    "head 112": dict(_ODD, num_hidden_layers=1, hidden_size=40, num_attention_heads=3, num_key_value_heads=3, head_dim=112,
+                     intermediate_size=88, vocab_size=1001, tie_word_embeddings=False, rope_theta=1e6),
+    "three heads a group, head 128": dict(_ODD, num_hidden_layers=2, hidden_size=192, num_attention_heads=12,
+                                          num_key_value_heads=4, head_dim=128, intermediate_size=320, vocab_size=777),
+    "seventeen heads on one group": dict(_ODD, num_hidden_layers=2, hidden_size=64, num_attention_heads=17,
+                                         num_key_value_heads=1, head_dim=64, intermediate_size=128, vocab_size=200),
+}
+
 
 def read_folder(path):
     """(config dict, {name: float64 array}) of a model folder, read with the

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import traces
-from helpers import CONFIGS, random_tokens, read_folder
+from helpers import CONFIGS, ODD_CONFIGS, random_tokens, read_folder, sharpen_folder
 from plain import qwen3_plain as plain
 
 pytestmark = pytest.mark.gpu
@@ -122,6 +122,26 @@ def test_engine_matches_plain(model_folders, name, sharp, page_size, dtype, mode
     err, where = worst(got, want)
     print(f"\n[{name} sharp={sharp} P={page_size} {dtype} {mode}] max |engine - plain| = {err:.3e} at {where}"
           f" (allowed {tol:.3e})")
+    assert err < tol, (err, tol, where)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(ODD_CONFIGS))
+def test_shapes_at_the_edges_match_plain(tmp_path_factory, name, dtype):
+    """Head sizes 16, 80, 112 and 256, one and seventeen heads a group, a window on every layer, widths that are
+    multiples of 8 only: mixed steps in a tight pool (which kernels serve such a shape differs; the logits do not)."""
+    from tinyinfer_amd.weights import write_model_folder
+    cfg = ODD_CONFIGS[name]
+    folder = str(tmp_path_factory.mktemp("odd"))
+    write_model_folder(folder, cfg, seed=99, dtype="bfloat16")
+    sharpen_folder(folder)
+    requests = make_requests(cfg["vocab_size"])
+    want, tol = plain_logits(folder, requests, dtype)
+    trace = make_trace("mixed", requests)
+    engine = build_engine(folder, dtype, traces.max_pages(trace, 16) * 16, 16)
+    got = replay(engine, trace)
+    assert not engine.cache.live_requests()
+    err, where = worst(got, want)
     assert err < tol, (err, tol, where)
 
 
