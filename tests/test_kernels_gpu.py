@@ -1380,6 +1380,63 @@ def test_attention_bf16_portions_and_mixed(ops, nh, nkv, hd, P, window, variant)
     assert (got - want).abs().max() < 2e-2
 
 
+def test_attention_bf16_far_into_long_contexts(ops):
+    """Rows of single tokens behind 20,000 and 32,767 cached tokens (a block table wider than the 1,024 entries
+    the decode kernel can hold in LDS, contexts cut into many runs) and portions of prompts deep inside a
+    context (300 tokens behind 20,000, 70 behind 9,000: tiles that walk hundreds of pages, the keys in runs),
+    against the softmax in float64 of just these rows.  In every request the key at position 7 is made to
+    stand out for the last query of head 0, so that a page dropped far back would show."""
+    if not ops.use_fast_attention:
+        pytest.skip("bfloat16 attention kernels are switched off")
+    from tinyinfer_amd.ops import attention_bf16
+    nh, nkv, hd, P = 4, 2, 128, 16
+    entries = [(1, 20000), (300, 20000), (1, 32767), (70, 9000), (1, 5)]
+    g = torch.Generator().manual_seed(21)
+    lens = [s + n for n, s in entries]
+    n_pages_each = [-(-L // P) for L in lens]
+    pages = sum(n_pages_each) + 5
+    perm = torch.randperm(pages, generator=g)
+    pool = (torch.randn(pages, 2, nkv, P, hd, generator=g) * 30).to(torch.bfloat16)
+    vt = pool[:, 1].reshape(pages, nkv, hd, P)
+    table = torch.full((len(lens), max(n_pages_each) + 1), -1, dtype=torch.int32)
+    qs, refs = [], []
+    used = 0
+    scale = 1.0 / math.sqrt(hd)
+    for e, ((n, start), L) in enumerate(zip(entries, lens)):
+        q = (torch.randn(n, nh, hd, generator=g) * 2.0).to(torch.bfloat16)
+        k = torch.randn(L, nkv, hd, generator=g).to(torch.bfloat16)
+        v = torch.randn(L, nkv, hd, generator=g).to(torch.bfloat16)
+        if L > 7:
+            k[7, 0] = (q[-1, 0].float() * 0.5).to(torch.bfloat16)          # score ~ 0.5 |q|^2 / sqrt(hd): far above the rest
+        mine = perm[used:used + n_pages_each[e]]
+        used += n_pages_each[e]
+        table[e, :len(mine)] = mine.to(torch.int32)
+        full = (L // P) * P
+        pool[mine[:L // P], 0] = k[:full].reshape(L // P, P, nkv, hd).permute(0, 2, 1, 3)
+        vt[mine[:L // P]] = v[:full].reshape(L // P, P, nkv, hd).permute(0, 2, 3, 1)
+        for t in range(full, L):
+            pool[mine[t // P], 0, :, t % P] = k[t]
+            vt[mine[t // P], :, :, t % P] = v[t]
+        ref = torch.zeros(n, nh, hd, dtype=torch.float64)
+        for h in range(nh):
+            sc = (f64(q[:, h]) @ f64(k[:, h // (nh // nkv)]).T) * scale           # [n, L]
+            key = torch.arange(L)[None, :]
+            sc = sc.masked_fill(key > (start + torch.arange(n))[:, None], float("-inf"))
+            ref[:, h] = torch.softmax(sc, -1) @ f64(v[:, h // (nh // nkv)])
+        if L > 7:
+            w7 = torch.softmax((f64(q[-1, 0]) @ f64(k[:, 0]).T) * scale, -1)[7]
+            assert w7 > 0.5                                                       # the far key carries the row
+        qs.append(q)
+        refs.append(ref)
+    qd = dev(torch.cat(qs).reshape(-1, nh * hd))
+    out = torch.zeros_like(qd)
+    ctx = FakeCtx(entries)
+    assert attention_bf16.run(ops, ctx, View(dev(table)), qd, dev(pool), out, nh, nkv, hd, scale, None)
+    got, want = f64(out), torch.cat(refs).reshape(-1, nh * hd)
+    assert torch.isfinite(got).all()
+    assert (got - want).abs().max() < 2e-2
+
+
 def test_attention_bf16_paired_tiles_of_one_long_prompt(ops):
     """A prompt of 1,100 tokens in one step (an odd number of 64-row tiles, the last one short):
     the kernel that pairs the tile of the most keys with the one of the fewest, against the
@@ -1437,10 +1494,19 @@ def test_attention_bf16_decode_from_projections(ops, nh, nkv, hd, P, window, nor
     value, against the two kernels it stands for, at context lengths around page edges and
     split over the context: the same bits in the cache; the same output up to the last
     bfloat16 bit (the row's own key enters the softmax last instead of in its block)."""
+    decode_from_projections_case(ops, nh, nkv, hd, P, window, norm, rope, (0, 1, 15, 16, 17, 31, 32, 100, 511, 512, 777, 1500))
+
+
+def test_attention_bf16_decode_from_projections_behind_long_contexts(ops):
+    """The same behind 4,097, 20,000 and 32,767 cached tokens: block-table rows wider than the 1,024 entries the
+    kernel can hold in LDS (the page ids are then looked up in memory), contexts cut into dozens of runs."""
+    decode_from_projections_case(ops, 16, 8, 128, 16, None, True, "table", (9, 4097, 20000, 32767))
+
+
+def decode_from_projections_case(ops, nh, nkv, hd, P, window, norm, rope, starts):
     if not ops.use_fast_attention:
         pytest.skip("bfloat16 attention kernels are switched off")
     g = torch.Generator().manual_seed(nh * 31 + hd)
-    starts = (0, 1, 15, 16, 17, 31, 32, 100, 511, 512, 777, 1500)
     entries = [(1, s) for s in starts]
     n_pages_each = [-(-(s + 1) // P) for s in starts]
     pages = sum(n_pages_each) + 5
