@@ -40,6 +40,16 @@ def bf16_sites(sites: Sequence[str]) -> Rounder:
     return rnd
 
 
+def float32_angles(rnd: Rounder = no_rounding) -> Rounder:
+    """`rnd`, and the rotation's frequencies and angles rounded to 32-bit floats as well (their sine and cosine
+    stay exact): what an engine that keeps to "angles in 32-bit" computes (src/cuda/rope.cu:20)."""
+    def both(site: str, a: np.ndarray) -> np.ndarray:
+        if site in ("rope_inv_freq", "rope_angle"):
+            return np.asarray(a, dtype=np.float32).astype(np.float64)
+        return rnd(site, a)
+    return both
+
+
 # The places where the reference drops to bfloat16: the operand of every matrix
 # product (src/inference.cu:40,53,59,63; src/cuda/lm_head.cu:8) and the cached
 # keys and values (src/cuda/attention.cu:83-84).
@@ -64,17 +74,20 @@ def linear(x: np.ndarray, w: np.ndarray) -> np.ndarray:
     return np.asarray(x, dtype=np.float64) @ np.asarray(w, dtype=np.float64).T
 
 
-def rope_neox(x: np.ndarray, positions: Sequence[int], theta: float) -> np.ndarray:
+def rope_neox(x: np.ndarray, positions: Sequence[int], theta: float, rnd: Rounder = no_rounding) -> np.ndarray:
     """Half-split rotation over the whole head: for k < hd/2 the angle is
     pos * theta^(-2k/hd); (x[k], x[k+hd/2]) -> (x[k] c - x[k+hd/2] s,
     x[k] s + x[k+hd/2] c).  x: [T, heads, hd].
-    src/cuda/attention.cu:38,64-74; src/cuda/rope.cu:20-28."""
+    src/cuda/attention.cu:38,64-74; src/cuda/rope.cu:20-28.  The reference has the frequency and
+    the angle in 32-bit (rope.cu:20); `rnd` may round them at the sites "rope_inv_freq" and
+    "rope_angle" (see `float32_angles`): thousands of tokens in, that is what limits the agreement
+    of a 32-bit engine with this model."""
     x = np.asarray(x, dtype=np.float64)
     hd = x.shape[-1]
     half = hd // 2
     k = np.arange(half, dtype=np.float64)
-    inv = theta ** (-2.0 * k / hd)
-    ang = np.asarray(positions, dtype=np.float64)[:, None] * inv[None, :]   # [T, half]
+    inv = rnd("rope_inv_freq", theta ** (-2.0 * k / hd))
+    ang = rnd("rope_angle", np.asarray(positions, dtype=np.float64)[:, None] * inv[None, :])   # [T, half]
     c = np.cos(ang)[:, None, :]
     s = np.sin(ang)[:, None, :]
     lo, hi = x[..., :half], x[..., half:]
@@ -131,8 +144,8 @@ def attention_block(h: np.ndarray, w: Dict[str, np.ndarray], prefix: str, cfg: d
     q = linear(hb, w[prefix + ".q_proj.weight"]).reshape(T, nh, hd)
     k = linear(hb, w[prefix + ".k_proj.weight"]).reshape(T, nkv, hd)
     v = linear(hb, w[prefix + ".v_proj.weight"]).reshape(T, nkv, hd)
-    q = rope_neox(qk_norm(q, w[prefix + ".q_norm.weight"], eps), positions, theta)
-    k = rope_neox(qk_norm(k, w[prefix + ".k_norm.weight"], eps), positions, theta)
+    q = rope_neox(qk_norm(q, w[prefix + ".q_norm.weight"], eps), positions, theta, rnd)
+    k = rope_neox(qk_norm(k, w[prefix + ".k_norm.weight"], eps), positions, theta, rnd)
     q = rnd("q", q)
     k = rnd("kv_cache", k)
     v = rnd("kv_cache", v)

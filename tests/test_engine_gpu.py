@@ -38,13 +38,16 @@ def make_requests(vocab, seed=7):
 _plain_cache = {}
 
 
-def plain_logits(folder, requests, dtype):
-    """({request: logits [T, V]}, tolerance) of the plain model for this dtype."""
-    key = (folder, tuple((r, tuple(t)) for r, t in sorted(requests.items())))
+def plain_logits(folder, requests, dtype, angles32=False):
+    """({request: logits [T, V]}, tolerance) of the plain model for this dtype.  angles32: the plain model has
+    the rotation's frequencies and angles in 32-bit like the engine (for contexts of thousands of tokens)."""
+    key = (folder, angles32, tuple((r, tuple(t)) for r, t in sorted(requests.items())))
     for d in ("float32", "bfloat16"):
         if key + (d,) not in _plain_cache:
             cfg, w = read_folder(folder)
             rnd = ROUNDED if d == "bfloat16" else plain.no_rounding
+            if angles32:
+                rnd = plain.float32_angles(rnd)
             _plain_cache[key + (d,)] = {r: plain.forward(w, cfg, t, rnd) for r, t in requests.items()}
     want = _plain_cache[key + (dtype,)]
     if dtype == "float32":
@@ -143,6 +146,37 @@ def test_shapes_at_the_edges_match_plain(tmp_path_factory, name, dtype):
     assert not engine.cache.live_requests()
     err, where = worst(got, want)
     assert err < tol, (err, tol, where)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prompt_of_5000_tokens_in_portions_then_decoding(tmp_path_factory, dtype):
+    """Beyond every other test's contexts: 5,000 tokens fed as portions of 2,048, 2,048 and 884 (the later ones
+    attend through thousands of cached keys, in runs), then 20 tokens one by one behind them (block-table rows
+    of 300 and more pages), beside a second short request; config D's shapes (a head of 64, windows of 37 on two
+    layers, full attention on one).  The last rows of every portion and every decoded row are the plain model's."""
+    from tinyinfer_amd.weights import write_model_folder
+    cfg = dict(CONFIGS["D"], max_position_embeddings=8192)
+    folder = str(tmp_path_factory.mktemp("long"))
+    write_model_folder(folder, cfg, seed=5, dtype="bfloat16")
+    sharpen_folder(folder)
+    requests = {"a": random_tokens(5020, cfg["vocab_size"], 70), "b": random_tokens(40, cfg["vocab_size"], 71)}
+    # thousands of tokens in, a 32-bit angle is some 1e-4 off its exact value: the plain model rounds where the engine does
+    want, tol = plain_logits(folder, requests, dtype, angles32=True)
+    a, b = requests["a"], requests["b"]
+    trace = [{"entries": [("a", a[:2048], [0, 2047])], "end": []},
+             {"entries": [("a", a[2048:4096], [0, 1000, 2047]), ("b", b[:20], [19])], "end": []},
+             {"entries": [("a", a[4096:5000], [0, 500, 903]), ("b", b[20:21], [0])], "end": []}]
+    for k in range(19):
+        trace.append({"entries": [("b", b[21 + k:22 + k], [0]), ("a", a[5000 + k:5001 + k], [0])], "end": []})
+    trace.append({"entries": [("a", a[5019:5020], [0])], "end": ["a", "b"]})
+    engine = build_engine(folder, dtype, 5120 + 64)
+    got = replay(engine, trace)
+    places = {"a": [0, 2047, 2048, 3048, 4095, 4096, 4596, 4999] + list(range(5000, 5020)), "b": [19] + list(range(20, 40))}
+    worst_err = 0.0
+    for r, at in places.items():
+        assert got[r].shape[0] == len(at), (r, got[r].shape)
+        worst_err = max(worst_err, float(np.abs(got[r] - want[r][at]).max()))
+    assert worst_err < tol, (worst_err, tol)
 
 
 @pytest.mark.parametrize("seed", [1, 2, 3])

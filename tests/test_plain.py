@@ -54,6 +54,23 @@ def test_rope_reference_vector():
     assert np.abs(plain.rope_neox(x, [0, 5], 1e6) - want).max() < 1e-12
 
 
+def test_rope_with_angles_in_32_bit():
+    """The reference has the angle in 32-bit (src/cuda/rope.cu:20): five tokens in that changes nothing one could
+    see, 5,000 tokens in the angle is up to 5000 * 2^-23 = 6e-4 off, and so are the rotated values."""
+    r = rng(6)
+    x = r.normal(size=(1, 2, 64))
+    rounded = plain.float32_angles()
+    assert np.abs(plain.rope_neox(x, [5], 1e4, rounded) - plain.rope_neox(x, [5], 1e4)).max() < 2e-6
+    far = np.abs(plain.rope_neox(x, [5000], 1e4, rounded) - plain.rope_neox(x, [5000], 1e4)).max()
+    assert 1e-6 < far < 6e-4 * np.abs(x).max() * 2
+    # it leaves the other sites to the rounder it wraps
+    seen = []
+    both = plain.float32_angles(lambda site, a: (seen.append(site), a)[1])
+    both("gemm_in", x)
+    both("rope_angle", x)
+    assert seen == ["gemm_in"]
+
+
 def test_rope_invariants():
     r = rng(4)
     q, k = r.normal(size=(1, 1, 32)), r.normal(size=(1, 1, 32))
