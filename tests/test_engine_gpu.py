@@ -160,8 +160,9 @@ def test_a_prompt_of_5000_tokens_in_portions_then_decoding(tmp_path_factory, dty
     write_model_folder(folder, cfg, seed=5, dtype="bfloat16")
     sharpen_folder(folder)
     requests = {"a": random_tokens(5020, cfg["vocab_size"], 70), "b": random_tokens(40, cfg["vocab_size"], 71)}
-    # thousands of tokens in, a 32-bit angle is some 1e-4 off its exact value: the plain model rounds where the engine does
-    want, tol = plain_logits(folder, requests, dtype, angles32=True)
+    # thousands of tokens in, an angle computed in 32-bit is some 1e-4 off (the plain model with
+    # `float32_angles` shows it): the engine's table of cosines and sines comes from angles in double precision
+    want, tol = plain_logits(folder, requests, dtype)
     a, b = requests["a"], requests["b"]
     trace = [{"entries": [("a", a[:2048], [0, 2047])], "end": []},
              {"entries": [("a", a[2048:4096], [0, 1000, 2047]), ("b", b[:20], [19])], "end": []},

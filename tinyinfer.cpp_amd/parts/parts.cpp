@@ -211,9 +211,13 @@ class RMSNorm final : public NormPart {
   Tensor weight;
 };
 
-// The inverse frequencies are built once on the host in double precision and rounded to float;
-// the angle pos * inv_freq[k] and its sine and cosine are 32-bit on the device.  `prepare(n)`
-// tabulates them for positions below n.  Parts with the same head size and base share one table.
+// The inverse frequencies are built once on the host in double precision and rounded to float.
+// `prepare(n)` tabulates cosine and sine for positions below n, on the host, from the angle in double
+// precision (rounded to float only at the end): a 32-bit angle pos * inv_freq[k] is pos * 2^-23 off, 6e-4
+// five thousand tokens in, and differently at every position, so that not only distances would count.
+// Positions beyond the table (none that an engine serves) have the angle and its sine and cosine in
+// 32-bit on the device, as /root/reference/src/cuda/rope.cu:20-22 has them everywhere.  Parts with the
+// same head size and base share one table.
 struct RopeTable {
   int head_dim = 0;
   double theta = 0;
@@ -255,8 +259,17 @@ class RotaryNeox final : public PositionPart {
     if (shared->table_len >= max_seq) return;
     const int half = head_dim / 2;
     DeviceBuffer fresh((size_t)max_seq * half * 2 * 4);
-    ops.rope_table(Tensor(shared->inv_freq.data(), DType::F32, {half}), Tensor(fresh.data(), DType::F32, {max_seq, half, 2}));
+    std::vector<double> inv(half);
+    for (int k = 0; k < half; ++k) inv[k] = std::pow(theta, -2.0 * k / head_dim);
+    std::vector<float> host((size_t)max_seq * half * 2);
+    for (int p = 0; p < max_seq; ++p)
+      for (int k = 0; k < half; ++k) {
+        const double angle = (double)p * inv[k];
+        host[((size_t)p * half + k) * 2] = (float)std::cos(angle);
+        host[((size_t)p * half + k) * 2 + 1] = (float)std::sin(angle);
+      }
     synchronize_device();          // the old table may still be read by a step in flight
+    upload(fresh.data(), host.data(), host.size() * 4);
     shared->table = std::move(fresh);
     shared->table_len = max_seq;
   }
