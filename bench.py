@@ -55,27 +55,44 @@ def say(msg):
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
 
-def model_numbers(c):
-    H, L, V = c["hidden_size"], c["num_hidden_layers"], c["vocab_size"]
-    nq = c["num_attention_heads"] * c["head_dim"]
-    nk = c["num_key_value_heads"] * c["head_dim"]
-    F = c["intermediate_size"]
-    layer_params = (nq + 2 * nk) * H + H * nq + 3 * H * F
-    norm_params = 2 * H + 2 * c["head_dim"]
-    head_params = V * H
-    # a decode step reads every layer, the head's matrix (the embedding itself when tied) and one
-    # embedding row per token
-    weight_bytes = L * (layer_params * 2 + norm_params * 4) + head_params * 2 + H * 4
-    kv_bytes_per_token = 2 * nk * L * 2
-    return dict(layer_params=layer_params, head_params=head_params, weight_bytes=weight_bytes,
-                kv_bytes_per_token=kv_bytes_per_token)
+def model_numbers(model):
+    """What a step must read and compute, from what the model's parts declare (their tensors with roles, their
+    cache needs), not from a formula of one architecture.  A decode step reads every matrix and vector of the
+    layers and the head once (a head tied to the embedding reads the embedding's matrix) and one embedding row
+    per token; per cached token it reads the keys and values of every cache layer."""
+    seen = set()
+    layer_params = head_params = vector_params = embed_row = 0
+    attn = []                     # (heads, head_dim, window) of every mixer that attends over cached keys
+    for part in model.parts():
+        for name, need in part.tensors().items():
+            n = 1
+            for d in need.shape:
+                n *= d
+            if part.family == "embedding":
+                embed_row = need.shape[-1]            # a row per token; the matrix counts where a head reads all of it
+                continue
+            if need.optional or name in seen:
+                continue
+            seen.add(name)
+            if need.role != "matrix":
+                vector_params += n
+            elif part.family == "head":
+                head_params += n
+            else:
+                layer_params += n
+        need = part.cache_need()
+        if need is not None and hasattr(need, "kv_heads") and "heads" in getattr(part, "params", {}):
+            attn.append((part.params["heads"], need.head_dim, need.window))
+    weight_bytes = (layer_params + head_params) * 2 + vector_params * 4 + embed_row * 2
+    kv_bytes = lambda context: sum(2 * need.kv_heads * need.head_dim * 2 * n * min(context, need.window or context)      # noqa: E731
+                                   for need, n in model.cache_groups if hasattr(need, "kv_heads"))
+    return dict(layer_params=layer_params, head_params=head_params, weight_bytes=weight_bytes, kv_bytes=kv_bytes, attention=attn)
 
 
-def prefill_flops(c, T):
-    n = model_numbers(c)
-    L, nh, hd = c["num_hidden_layers"], c["num_attention_heads"], c["head_dim"]
-    gemm = 2.0 * n["layer_params"] * L * T + 2.0 * n["head_params"]          # the head runs on one row
-    attn = 2.0 * hd * T * (T + 1) * nh * L                                    # QK^T and PV over the causal half
+def prefill_flops(model, T):
+    n = model_numbers(model)
+    gemm = 2.0 * n["layer_params"] * T + 2.0 * n["head_params"]              # the head runs on one row
+    attn = sum(2.0 * hd * T * (T + 1) * heads for heads, hd, _ in n["attention"])   # QK^T and PV over the causal half
     return gemm + attn
 
 
@@ -288,7 +305,7 @@ def main() -> int:
                                 max_tokens=biggest * (context + 512) + prefill_tokens + args.cached + args.portion,
                                 max_requests=biggest + 1, max_seq=max_seq)
     sampler = Sampler(engine.ops, engine.device)
-    nums = model_numbers(cfg)
+    nums = model_numbers(engine.model)
 
     if args.only == "mixed":
         say(f"a step of {args.batch} decoded tokens beside a portion of {args.portion} (after {args.cached} cached) ...")
@@ -322,7 +339,7 @@ def main() -> int:
                                                           f"p{b}_", draw=draw)[0], 1)
 
     ctx_mean = context + args.warmup + args.steps / 2.0
-    step_bytes = nums["weight_bytes"] + args.batch * ctx_mean * nums["kv_bytes_per_token"]
+    step_bytes = nums["weight_bytes"] + args.batch * nums["kv_bytes"](ctx_mean)
     achieved = step_bytes / (ms * 1e-3) if ms else None
     roofline = prefill = None
     if achieved is not None:
@@ -331,7 +348,7 @@ def main() -> int:
         if peaks:
             roofline.update(measured_read=round(peaks[0] / 1e9, 1), frac_of_measured=round(achieved / peaks[0], 4))
     if p_s is not None:
-        flops = prefill_flops(cfg, prefill_tokens)
+        flops = prefill_flops(engine.model, prefill_tokens)
         prefill = {"value": round(prefill_tokens / p_s, 1), "tokens": prefill_tokens, "ms": round(p_s * 1e3, 3),
                    "frac": round(flops / p_s / PEAK_BF16, 4)}
         if peaks:

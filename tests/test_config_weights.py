@@ -51,6 +51,9 @@ def test_config_defaults_and_windows():
     (dict(hidden_size=0), "hidden_size"),
     (dict(num_attention_heads=5), "num_key_value_heads"),
     (dict(head_dim=15), "head_dim"),
+    (dict(head_dim=24), "head_dim"),          # even, but no attention kernel takes it: said before any weight is read
+    (dict(head_dim=40), "steps of 16"),
+    (dict(head_dim=512), "up to 256"),
     (dict(attention_bias=True), "attention_bias"),
     (dict(hidden_act="gelu"), "hidden_act"),
     (dict(rope_scaling={"rope_type": "yarn", "factor": 4.0}), "rope_scaling"),
@@ -65,6 +68,15 @@ def test_config_errors_name_the_key(change, needle):
     with pytest.raises(ti.ConfigError) as e:
         Qwen3Config.from_dict(d)
     assert needle in str(e.value)
+
+
+def test_an_attention_part_refuses_a_head_size_no_kernel_takes():
+    """Not only through config.json: whoever builds the part (another architecture's spec) hears it at once."""
+    for hd in (8, 24, 272):
+        with pytest.raises((ti.ConfigError, ValueError)) as e:
+            ti.build_part("mixer", ti.PartSpec("attention", dict(hidden=64, heads=2, kv_heads=1, head_dim=hd)), "layer")
+        assert "head_dim" in str(e.value) and str(hd) in str(e.value)
+    ti.build_part("mixer", ti.PartSpec("attention", dict(hidden=64, heads=2, kv_heads=1, head_dim=48)), "layer")
 
 
 def test_registry_picks_by_name_and_lists_what_it_has():

@@ -304,6 +304,55 @@ def test_command_line(model_folders, tmp_path):
     assert bad.returncode == 1 and "usage:" in bad.stderr
 
 
+def test_command_line_options(tmp_path):
+    """`--random-weights --seed` from a folder with config.json alone, `--num-pages`, `--cuda-graph`, `-t`, `--top-k`,
+    `--verbose`: the tokens are the plain model's on the weights `write_model_folder` writes for that seed, drawn with
+    the same temperature, cut and seed; --verbose prints the first five and the five largest logits behind each prompt
+    (/root/reference/src/main.cpp:136-158,233-249)."""
+    import json
+    import tinyinfer_amd as ti
+    cfg = CONFIGS["A"]
+    bare = tmp_path / "bare"
+    bare.mkdir()
+    (bare / "config.json").write_text(json.dumps(cfg))
+    full = str(tmp_path / "full")
+    ti.write_model_folder(full, cfg, seed=9, dtype="float32")
+    _, w = read_folder(full)
+    p1, p2 = random_tokens(7, 256, 11), random_tokens(21, 256, 12)
+    exe = [sys.executable, os.path.join(ROOT, "bin", "tinyinfer")]
+    common = ["-m", str(bare), "--random-weights", "--seed", "9", "--dtype", "float32", "--max-seq", "48", "--num-pages", "6",
+              "-p", " ".join(map(str, p1)), "-p", " ".join(map(str, p2))]
+    greedy = subprocess.run(exe + common + ["-n", "8", "--cuda-graph", "--verbose"], capture_output=True, text=True, timeout=300)
+    assert greedy.returncode == 0, greedy.stderr
+    lines = greedy.stdout.strip().split("\n")
+    assert lines[2] == "[output] " + " ".join(map(str, plain_generate(cfg, w, p1, 8)))
+    assert lines[5] == "[output] " + " ".join(map(str, plain_generate(cfg, w, p2, 8)))
+    assert "[hip-graph: on]" in greedy.stderr
+    for s, p in enumerate((p1, p2)):
+        row = plain.forward(w, cfg, p)[-1]
+        shown = [ln for ln in greedy.stderr.split("\n") if ln.startswith(f"prefill logits seq {s} (first 5, top 5):")]
+        assert len(shown) == 1, greedy.stderr
+        first, top = shown[0].split(":", 1)[1].split(" | top5:")
+        assert np.allclose([float(v) for v in first.split()], row[:5], atol=2e-3)
+        ids = [int(t.split("(")[0]) for t in top.split()]
+        assert ids == [int(i) for i in np.lexsort((np.arange(row.size), -row))[:5]], (ids, shown)
+    # two pages of 16 tokens instead of six, for requests of 15 and 29 tokens: they cannot both be live; the tokens stay
+    tight = subprocess.run(exe + ["-m", str(bare), "--random-weights", "--seed", "9", "--dtype", "float32", "--max-seq", "48",
+                                  "--num-pages", "2", "-n", "8", "-p", " ".join(map(str, p1)), "-p", " ".join(map(str, p2))],
+                           capture_output=True, text=True, timeout=300)
+    assert tight.returncode == 0 and tight.stdout == greedy.stdout, tight.stderr
+    drawn = subprocess.run(exe + common + ["-n", "6", "-t", "0.8", "--top-k", "4", "--top-p", "0.9"], capture_output=True, text=True,
+                           timeout=300)
+    assert drawn.returncode == 0, drawn.stderr
+    lines = drawn.stdout.strip().split("\n")
+    for s, p in enumerate((p1, p2)):
+        want = plain_generate(cfg, w, p, 6, number=s, temperature=0.8, top_k=4, top_p=0.9, seed=9)
+        assert lines[3 * s + 2] == "[output] " + " ".join(map(str, want))
+    none = subprocess.run(exe + ["-m", str(bare), "-n", "2", "-p", "1 2 3", "--dtype", "float32"], capture_output=True, text=True,
+                          timeout=300)
+    assert none.returncode == 1 and "safetensors" in none.stderr          # no weights and no --random-weights
+
+
 def test_smoke_entry():
     sys.path.insert(0, ROOT)
     import __graft_entry__

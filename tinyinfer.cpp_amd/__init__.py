@@ -13,8 +13,10 @@ from .engine import Engine, StepEntry, token_from_feedback
 from .engine.scheduler import Scheduler, Request
 from .sampling import SamplingParams
 from .api import LLM, generate_ids, GenerationStats
+from .weights import write_model_folder
+from .native import load_plugin
 
 __all__ = ["ConfigError", "read_config_json", "Qwen3Config", "register_architecture",
            "registered_architectures", "config_and_spec", "register_part", "build_part",
            "Model", "ModelSpec", "LayerSpec", "PartSpec", "Engine", "StepEntry", "token_from_feedback", "Scheduler", "Request",
-           "SamplingParams", "LLM", "generate_ids", "GenerationStats"]
+           "SamplingParams", "LLM", "generate_ids", "GenerationStats", "write_model_folder", "load_plugin"]

@@ -35,12 +35,14 @@ class GenerationStats:
 
 def run_requests(engine: Engine, scheduler: Scheduler, sampler: Optional[Sampler] = None,
                  stats: Optional[GenerationStats] = None, on_token=None, use_graph: bool = False,
-                 run_ahead: bool = True) -> None:
+                 run_ahead: bool = True, on_prompt_logits=None) -> None:
     """Run until the scheduler has no work.  `on_token(request, token)` is called for every
     generated token.  When a step fails, every request the scheduler still holds is given back
     to the cache before the error is raised.  `run_ahead`: while every running request decodes
     and nobody waits, the next step is launched before the last one's ids are read (it takes
-    them from the device); the tokens are the same, `on_token` hears them a step later."""
+    them from the device); the tokens are the same, `on_token` hears them a step later.
+    `on_prompt_logits(request, logits)`: called with the 32-bit logits (a numpy array) behind the last token of
+    each request's prompt, before its first token is drawn."""
     native.ensure_kernels(["sampling"])
     raised = []
 
@@ -52,10 +54,20 @@ def run_requests(engine: Engine, scheduler: Scheduler, sampler: Optional[Sampler
             raised.append(e)
             return 1
 
+    def relay_logits(number, row, vocab):
+        try:
+            import numpy as np
+            on_prompt_logits(scheduler._requests[number], np.ctypeslib.as_array(row, shape=(vocab,)).copy())
+            return 0
+        except BaseException as e:  # noqa: BLE001
+            raised.append(e)
+            return 1
+
     callback = native.ON_TOKEN(relay) if on_token else ctypes_null(native.ON_TOKEN)
+    logits_callback = native.ON_LOGITS(relay_logits) if on_prompt_logits else ctypes_null(native.ON_LOGITS)
     try:
         out = native.text("ti_run_requests", engine._ptr, scheduler._ptr, sampler._ptr if sampler else None,
-                          int(use_graph), int(run_ahead), callback)
+                          int(use_graph), int(run_ahead), callback, logits_callback)
     except native.EngineError:
         if raised:
             raise raised[0] from None
@@ -82,14 +94,21 @@ def generate_ids(engine: Engine, prompts: Sequence[Sequence[int]], max_new_token
                  temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0, seed: int = 42,
                  eos_token_ids: Optional[Sequence[int]] = None, chunk_size: int = 512,
                  max_batched_tokens: int = 2048, use_graph: bool = False,
-                 stats: Optional[GenerationStats] = None, run_ahead: bool = True) -> List[List[int]]:
+                 stats: Optional[GenerationStats] = None, run_ahead: bool = True, on_prompt_logits=None) -> List[List[int]]:
     """Generated token ids for each prompt (the prompt itself is not repeated)."""
     if eos_token_ids is None:
         eos_token_ids = engine.model.spec.eos_token_ids
     scheduler = Scheduler(engine.cache, max_batched_tokens=max_batched_tokens, chunk_size=chunk_size)
     params = SamplingParams(float(temperature), int(top_k), float(top_p), int(seed))
     requests: List[Request] = [scheduler.add(p, max_new_tokens, params, eos_token_ids) for p in prompts]
-    run_requests(engine, scheduler, stats=stats, use_graph=use_graph, run_ahead=run_ahead)
+    relay = None
+    if on_prompt_logits:
+        index = {}          # request number -> index of its prompt
+        relay = lambda request, logits: on_prompt_logits(index[request.number], logits)     # noqa: E731
+    for i, r in enumerate(requests):
+        if relay:
+            index[r.number] = i
+    run_requests(engine, scheduler, stats=stats, use_graph=use_graph, run_ahead=run_ahead, on_prompt_logits=relay)
     return [list(r.generated) for r in requests]
 
 
@@ -117,7 +136,9 @@ class LLM:
 
     def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 128, temperature: float = 0.0,
                  top_k: int = 0, top_p: float = 1.0, seed: int = 42,
-                 eos_token_ids: Optional[Sequence[int]] = None) -> List[List[int]]:
+                 eos_token_ids: Optional[Sequence[int]] = None, on_prompt_logits=None) -> List[List[int]]:
+        """`on_prompt_logits(i, logits)`: the 32-bit logits behind the last token of prompt i, before its first token is drawn."""
         self.last_stats = GenerationStats()
         return generate_ids(self.engine, prompts, max_new_tokens, temperature, top_k, top_p, seed, eos_token_ids,
-                            self.chunk_size, self.max_batched_tokens, self.use_graph, self.last_stats)
+                            self.chunk_size, self.max_batched_tokens, self.use_graph, self.last_stats,
+                            on_prompt_logits=on_prompt_logits)

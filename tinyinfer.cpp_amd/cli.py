@@ -160,9 +160,20 @@ def main(argv: Optional[List[str]] = None) -> int:
     if verbose:
         for s, t in enumerate(ids):
             sys.stderr.write(f"prompt {s} tokens: {len(t)}\n")
+
+    def show_logits(s, row):
+        # the first five logits and the five largest behind each prompt, as the reference's --verbose prints them
+        # (/root/reference/src/main.cpp:233-249)
+        import numpy as np
+        top = np.lexsort((np.arange(row.shape[0]), -row))[:5]            # descending, the lowest id first among equals
+        piece = (lambda t: tokenizer.id_to_token(int(t)) or "") if tokenizer is not None else (lambda t: "")
+        sys.stderr.write(f"prefill logits seq {s} (first 5, top 5):" + "".join(f" {v:.3f}" for v in row[:5]) + " | top5:" +
+                         "".join(f" {int(t)}({piece(t)}):{row[t]:.3f}" for t in top) + "\n")
+
     t0 = time.perf_counter()
     try:
-        outs = llm.generate(ids, max_new_tokens=n_predict, temperature=temp, top_k=top_k, top_p=top_p, seed=seed)
+        outs = llm.generate(ids, max_new_tokens=n_predict, temperature=temp, top_k=top_k, top_p=top_p, seed=seed,
+                            on_prompt_logits=show_logits if verbose else None)
     except RuntimeError as e:
         sys.stderr.write(f"main: {e}\n")
         return 1

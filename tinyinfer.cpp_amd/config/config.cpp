@@ -161,6 +161,11 @@ void Qwen3Config::validate() const {
   if (head_dim % 2)
     throw ConfigError("config.json: 'head_dim' (" + std::to_string(head_dim) +
                       ") must be even (rotation pairs k with k + head_dim/2)");
+  // what the attention kernels take (the reference refuses a head size at the launch:
+  // /root/reference/src/cuda/attention.cu:321-324); said here, before any weight is read
+  if (head_dim % 16 || head_dim > 256)
+    throw ConfigError("config.json: 'head_dim' = " + std::to_string(head_dim) +
+                      " is not served: the attention kernels take head sizes in steps of 16 up to 256");
   if (!(rms_norm_eps > 0.0)) throw ConfigError("config.json: 'rms_norm_eps' must be positive");
   if (!(rope_theta > 0.0)) throw ConfigError("config.json: 'rope_theta' must be positive");
   if (sliding_window < 0) throw ConfigError("config.json: 'sliding_window' must be positive");
@@ -309,8 +314,13 @@ ModelSpec ModelSpec::from_json(const Json& j) {
 // ---------------------------------------------------------------------------------- registry
 namespace {
 std::mutex g_arch_mutex;
-std::vector<std::pair<std::string, SpecBuilder>>& architectures() {
-  static std::vector<std::pair<std::string, SpecBuilder>> table;
+struct Architecture {
+  std::string name;
+  SpecBuilder builder;
+  ConfigReader typed;
+};
+std::vector<Architecture>& architectures() {
+  static std::vector<Architecture> table;
   return table;
 }
 
@@ -379,8 +389,9 @@ void ensure_builtin_architectures() {
   static std::once_flag once;
   std::call_once(once, [] {
     std::lock_guard<std::mutex> lock(g_arch_mutex);
-    architectures().emplace_back("Qwen3ForCausalLM", build_qwen3_spec);
-    architectures().emplace_back("qwen3", build_qwen3_spec);
+    const ConfigReader typed = [](const Json& config) { return Qwen3Config::from_json(config).to_json(); };
+    architectures().push_back({"Qwen3ForCausalLM", build_qwen3_spec, typed});
+    architectures().push_back({"qwen3", build_qwen3_spec, typed});
   });
 }
 
@@ -402,17 +413,18 @@ std::string list_of(const std::vector<std::string>& v) {
 }
 }  // namespace
 
-void register_architecture(const std::vector<std::string>& names, SpecBuilder builder) {
+void register_architecture(const std::vector<std::string>& names, SpecBuilder builder, ConfigReader typed) {
   ensure_builtin_architectures();
   std::lock_guard<std::mutex> lock(g_arch_mutex);
   for (const auto& n : names) {
     bool found = false;
-    for (auto& kv : architectures())
-      if (kv.first == n) {
-        kv.second = builder;
+    for (auto& a : architectures())
+      if (a.name == n) {
+        a.builder = builder;
+        a.typed = typed;
         found = true;
       }
-    if (!found) architectures().emplace_back(n, builder);
+    if (!found) architectures().push_back({n, builder, typed});
   }
 }
 
@@ -420,7 +432,7 @@ std::vector<std::string> registered_architectures() {
   ensure_builtin_architectures();
   std::lock_guard<std::mutex> lock(g_arch_mutex);
   std::vector<std::string> names;
-  for (const auto& kv : architectures()) names.push_back(kv.first);
+  for (const auto& a : architectures()) names.push_back(a.name);
   std::sort(names.begin(), names.end());
   return names;
 }
@@ -429,33 +441,37 @@ bool architecture_registered(const Json& config) {
   ensure_builtin_architectures();
   std::lock_guard<std::mutex> lock(g_arch_mutex);
   for (const auto& c : candidates(config))
-    for (const auto& kv : architectures())
-      if (kv.first == c) return true;
+    for (const auto& a : architectures())
+      if (a.name == c) return true;
   return false;
 }
 
-ModelSpec spec_from_config(const Json& config) {
+namespace {
+Architecture architecture_of(const Json& config) {
   ensure_builtin_architectures();
   const auto cand = candidates(config);
   if (cand.empty())
     throw ConfigError("config.json: neither 'architectures' nor 'model_type' names the model; registered: " +
                       list_of(registered_architectures()));
-  SpecBuilder builder;
   {
     std::lock_guard<std::mutex> lock(g_arch_mutex);
-    for (const auto& c : cand) {
-      for (const auto& kv : architectures())
-        if (kv.first == c) {
-          builder = kv.second;
-          break;
-        }
-      if (builder) break;
-    }
+    for (const auto& c : cand)
+      for (const auto& a : architectures())
+        if (a.name == c) return a;
   }
-  if (!builder)
-    throw ConfigError("config.json: architecture " + list_of(cand) + " is not registered; registered: " +
-                      list_of(registered_architectures()));
-  return builder(config);
+  throw ConfigError("config.json: architecture " + list_of(cand) + " is not registered; registered: " +
+                    list_of(registered_architectures()));
+}
+}  // namespace
+
+ModelSpec spec_from_config(const Json& config) { return architecture_of(config).builder(config); }
+
+Json typed_config(const Json& config) {
+  const Architecture a = architecture_of(config);
+  Json j = Json::object();
+  j.set("architecture", a.name);
+  j.set("config", a.typed ? a.typed(config) : config);
+  return j;
 }
 
 }  // namespace tinyinfer

@@ -42,7 +42,11 @@ class Qwen3Config:
     @classmethod
     def from_dict(cls, d: Mapping[str, Any]) -> "Qwen3Config":
         """Read and validate; an error names the key."""
-        n = json.loads(native.text("ti_qwen3_config", json.dumps(dict(d)).encode()))
+        return cls.from_normalized(json.loads(native.text("ti_qwen3_config", json.dumps(dict(d)).encode())))
+
+    @classmethod
+    def from_normalized(cls, n: Mapping[str, Any]) -> "Qwen3Config":
+        """From the keys as the library writes them back (validated, defaults filled in)."""
         eos = n.get("eos_token_id")
         return cls(
             vocab_size=n["vocab_size"], hidden_size=n["hidden_size"], intermediate_size=n["intermediate_size"],

@@ -38,16 +38,21 @@ EXTRA_FLAGS: Dict[str, List[str]] = {
     "attention_bf16": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
 }
 
-# library name -> source file
-SOURCES: Dict[str, str] = {
-    "core": "core.hip",
-    "gemm_generic": "gemm_generic.hip",
-    "attention_generic": "attention_generic.hip",
-    "sampling": "sampling.hip",
-    "gemm_bf16": "gemm_bf16.hip",
-    "attention_bf16": "attention_bf16.hip",
-    "measure": "measure.hip",
-}
+def _discover() -> Dict[str, str]:
+    """library name -> source file: every `*.hip` in this folder is a kernel library of its own, named for
+    the file.  A new kernel file needs no entry anywhere."""
+    return {f[:-4]: f for f in sorted(os.listdir(HERE)) if f.endswith(".hip")}
+
+
+SOURCES: Dict[str, str] = _discover()
+# libraries no model needs (measurement helpers): built with everything else, never on a model's behalf
+ON_DEMAND = ("measure",)
+
+
+def libraries_for(dtype: str) -> List[str]:
+    """The kernel libraries a model of this dtype needs: every one except those whose name ends in `_bf16`
+    when the engine runs in float32 (what a first call compiles)."""
+    return [n for n in SOURCES if n not in ON_DEMAND and (dtype == "bfloat16" or not n.endswith("_bf16"))]
 
 
 # the host library (configuration, weights, parts, cache manager, step function, scheduler, sampler
@@ -276,6 +281,50 @@ def ensure_host(force: bool = False) -> str:
     return final
 
 
+# programs beside the libraries: name -> source (C++17, linked with the host library)
+TOOLS: Dict[str, str] = {"trace_run": "engine/trace_run.cpp"}
+
+
+def tool_name(name: str) -> str:
+    h = hashlib.sha256()
+    with open(os.path.join(PKG, TOOLS[name]), "rb") as fh:
+        h.update(fh.read())
+    h.update(_host_digest().encode())
+    return f"tinyinfer_{name}.{h.hexdigest()[:12]}"
+
+
+def ensure_tool(name: str, force: bool = False) -> str:
+    """Path of the program `name`, compiled and linked with the host library if it is not there."""
+    fn = tool_name(name)
+    if not force:
+        for d in _lib_dirs():
+            if os.path.isfile(os.path.join(d, fn)):
+                return os.path.join(d, fn)
+    host = ensure_host()
+    cxx = shutil.which("g++") or shutil.which("c++") or os.path.join(ROCM, "llvm", "bin", "clang++")
+    out_dir = os.path.dirname(host)
+    final = os.path.join(out_dir, fn)
+    part = final + f".{os.getpid()}.part"
+    t0 = time.time()
+    _say(f"compiling {TOOLS[name]} ...")
+    proc = subprocess.run([cxx, "-std=c++17", "-O2", "-D__HIP_PLATFORM_AMD__", os.path.join(PKG, TOOLS[name]), "-o", part, host,
+                           "-Wl,-rpath," + out_dir, "-Wl,-rpath," + os.path.join(ROCM, "lib")],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        if os.path.exists(part):
+            os.remove(part)
+        raise BuildError(f"{TOOLS[name]} does not compile:\n{proc.stdout}")
+    os.replace(part, final)
+    for f in os.listdir(out_dir):
+        if f.startswith(f"tinyinfer_{name}.") and f != fn and not f.endswith(".part"):
+            try:
+                os.remove(os.path.join(out_dir, f))
+            except OSError:
+                pass
+    _say(f"compiled {TOOLS[name]} in {time.time() - t0:.1f} s")
+    return final
+
+
 def write_manifest() -> None:
     """kernels.manifest beside the libraries: `name file` a line, for programs that use the host library
     without this package (it looks the kernel libraries up there)."""
@@ -296,6 +345,8 @@ def write_manifest() -> None:
 def build_all(force: bool = True) -> Dict[str, str]:
     paths = ensure([n for n, s in SOURCES.items() if os.path.isfile(os.path.join(HERE, s))], force=force)
     paths["host"] = ensure_host(force=force)
+    for tool in TOOLS:
+        paths[tool] = ensure_tool(tool, force=force)
     write_manifest()
     return paths
 

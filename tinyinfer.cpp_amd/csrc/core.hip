@@ -590,7 +590,10 @@ extern "C" int ti_fill_zero(void* p, long bytes, hipStream_t stream) {
 
 // Random weights on the device.  Element i of a tensor is a pure function of (seed, i): two
 // 24-bit uniforms from splitmix64's output function, then Box-Muller for a normal.  The host's
-// generator (the one that writes model folders) is the same function.
+// generator (the one that writes model folders) is the same function.  The logarithm, root and
+// cosine are taken in double precision and the value is rounded to 32-bit once at the end: the two
+// libraries' double results differ far below a 32-bit step, so the device draws the bits the host
+// draws (32-bit logf/cosf of two libraries differ in the last bit for a third of the values).
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {
   z += 0x9E3779B97F4A7C15ull;
   z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
@@ -602,11 +605,11 @@ template <typename T>
 __global__ void fill_random_kernel(T* __restrict__ p, long n, int kind, float a, float b, uint64_t seed) {
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
     const uint64_t z = mix64(mix64(seed) ^ (uint64_t)i);
-    const float u1 = ((float)((z >> 40) & 0xffffffu) + 1.0f) * (1.0f / 16777216.0f);   // (0, 1]
-    const float u2 = (float)((z >> 16) & 0xffffffu) * (1.0f / 16777216.0f);            // [0, 1)
+    const double u1 = ((double)((z >> 40) & 0xffffffu) + 1.0) * (1.0 / 16777216.0);   // (0, 1]
+    const double u2 = (double)((z >> 16) & 0xffffffu) * (1.0 / 16777216.0);            // [0, 1)
     float v;
-    if (kind == 0) v = a + b * (sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2));
-    else if (kind == 1) v = a + (b - a) * u2;
+    if (kind == 0) v = (float)((double)a + (double)b * (sqrt(-2.0 * log(u1)) * cos(6.28318530717958647692 * u2)));
+    else if (kind == 1) v = (float)((double)a + ((double)b - (double)a) * u2);
     else v = a;
     st<T>(p + i, v);
   }

@@ -134,8 +134,8 @@ int ti_argmax(const float* logits, int* out, void* scratch, int n_rows, int V, h
 // harnesses that forbid hipMalloc): the same two-stage kernels with their partial results in a
 // device array of the library itself (128 KiB on each GPU it runs on, kept until the process ends)
 // instead of a workspace argument.  At most 256 rows, else an error.  It calls no hipMalloc, hipFree or
-// allocating routine; calls that overlap on one GPU share the array and race.  The reference has no
-// counterpart (its argmax needs no scratch: /root/reference/src/cuda/sample.cu:13-54).
+// allocating routine; calls that overlap on one GPU share the array and race.  It has no counterpart in
+// the reference: it is there for callers that cannot allocate.
 int ti_argmax_static(const float* logits, int* out, int n_rows, int V, hipStream_t stream);
 // temperature, top-k (0: all), top-p and one uniform number per row.  scratch: ti_sample_scratch_bytes(n_rows)
 // bytes, zero before the first call and touched by nothing else since (the kernels leave them at zero; calls

@@ -180,6 +180,11 @@ int ti_kernels_register(const char* name, const char* path) {
   register_kernel_library(name, path);
   TI_END
 }
+int ti_load_plugin(const char* path) {
+  TI_BEGIN
+  load_plugin(path);
+  TI_END
+}
 int ti_set_allocator(void* (*alloc)(void*, size_t), void (*release)(void*, void*), void* user) {
   TI_BEGIN
   Allocator a;
@@ -205,6 +210,11 @@ int ti_qwen3_config(const char* config_json, const char** out_json) {
   const Qwen3Config c = Qwen3Config::from_json(Json::parse(config_json));
   Json j = c.to_json();
   return give(out_json, j.dump());
+  TI_END
+}
+int ti_typed_config(const char* config_json, const char** out) {
+  TI_BEGIN
+  return give(out, typed_config(Json::parse(config_json)).dump());
   TI_END
 }
 int ti_spec_from_config(const char* config_json, const char** out) {
@@ -256,7 +266,53 @@ int ti_part_create_foreign(const char* family, uint64_t id, const char* prefix, 
                                                      children_of(n_children, child_slots, children)));
   TI_END
 }
+namespace {
+int (*g_foreign_make)(const char*, const char*, const char*, const char*, int, const char* const*, void* const*, void**) = nullptr;
+}
+int ti_set_foreign_factory(int (*make)(const char*, const char*, const char*, const char*, int, const char* const*, void* const*,
+                                       void**)) {
+  TI_BEGIN
+  g_foreign_make = make;
+  TI_END
+}
+int ti_register_foreign_kind(const char* family_, const char* kind_, const char* slots_json) {
+  TI_BEGIN
+  const std::string family = family_, kind = kind_;
+  std::vector<std::pair<std::string, std::string>> slots;
+  if (slots_json && *slots_json) {
+    const Json parsed = Json::parse(slots_json);
+    for (const auto& kv : parsed.members()) slots.emplace_back(kv.first, kv.second.as_string());
+  }
+  register_part(family, kind, [family, kind](const std::string& prefix, const Json& params, const PartChildren& children) {
+    if (!g_foreign_make) throw ConfigError("the " + family + " part '" + kind + "' is implemented outside the library, which is gone");
+    // the children cross as handles that the other side owns from here on
+    std::vector<const char*> names;
+    std::vector<void*> handles;
+    for (const auto& c : children) {
+      names.push_back(c.first.c_str());
+      handles.push_back(new std::shared_ptr<Part>(c.second));
+    }
+    void* made = nullptr;
+    const std::string text = params.dump();
+    const int rc = g_foreign_make(family.c_str(), kind.c_str(), prefix.c_str(), text.c_str(), (int)children.size(), names.data(),
+                                  handles.data(), &made);
+    // (the handles to the children are the maker's now: it releases each with ti_part_release)
+    if (rc != 0 || !made) {
+      const std::string why = take_foreign_error();
+      throw ConfigError("building the " + family + " part '" + kind + "' outside the library failed" + (why.empty() ? "" : ": " + why));
+    }
+    return *static_cast<std::shared_ptr<Part>*>(made);       // a reference of our own; the handle stays the maker's
+  }, slots);
+  TI_END
+}
 void ti_part_release(void* part) { delete static_cast<std::shared_ptr<Part>*>(part); }
+int ti_part_child(void* part, int index, void** out) {
+  TI_BEGIN
+  const auto kids = P(part)->children();
+  if (index < 0 || index >= (int)kids.size()) throw Error("ti_part_child: the part has no child " + std::to_string(index));
+  *out = new std::shared_ptr<Part>(kids[index]);
+  TI_END
+}
 int ti_part_tensors(void* part, const char** out) {
   TI_BEGIN
   return give(out, needs_json(P(part)->tensors()).dump());
@@ -281,6 +337,12 @@ int ti_part_info(void* part, const char** out) {
   if (auto* n = dynamic_cast<NormPart*>(&p)) lazy_out = n->can_be_lazy();
   j.set("takes_lazy_norm", lazy_in);
   j.set("can_be_lazy", lazy_out);
+  j.set("built_kind", p.built_kind);
+  j.set("params", p.built_from.type() == Json::Object ? p.built_from : Json::object());
+  j.set("foreign_id", (int64_t)p.foreign_id);
+  Json slots = Json::array();
+  for (const auto& n : p.child_slots()) slots.push(n);
+  j.set("slots", slots);
   return give(out, j.dump());
   TI_END
 }
@@ -497,6 +559,28 @@ int ti_ctx_ops(void* ctx_, void** out) {
 }
 
 // -------------------------------------------------------------------------------------- model
+int ti_model_from_spec(const char* spec_json, void** out) {
+  TI_BEGIN
+  *out = new std::shared_ptr<Model>(new Model(ModelSpec::from_json(Json::parse(spec_json))));
+  TI_END
+}
+int ti_model_part(void* model, const char* which_, int index, void** out) {
+  TI_BEGIN
+  Model& m = *M(model);
+  const std::string which = which_;
+  std::shared_ptr<Part> p;
+  if (which == "embedding") p = m.embedding;
+  else if (which == "final_norm") p = m.final_norm;
+  else if (which == "head") p = m.head;
+  else if (which == "block") {
+    if (index < 0 || index >= (int)m.blocks.size()) throw Error("ti_model_part: the model has no layer " + std::to_string(index));
+    p = m.blocks[index];
+  } else {
+    throw Error("ti_model_part: unknown part '" + which + "'");
+  }
+  *out = new std::shared_ptr<Part>(p);
+  TI_END
+}
 int ti_model_create(const char* meta_json, void* embedding, int n_blocks, void* const* blocks, void* final_norm, void* head,
                     void** out) {
   TI_BEGIN
@@ -955,7 +1039,7 @@ int ti_scheduler_request(void* scheduler, int64_t number, const char** out) {
   TI_END
 }
 int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph, int run_ahead, int (*on_token)(int64_t, int),
-                    const char** out_stats) {
+                    int (*on_logits)(int64_t, const float*, int64_t), const char** out_stats) {
   TI_BEGIN
   SchedulerHandle& h = *static_cast<SchedulerHandle*>(scheduler);
   GenerationStats st;
@@ -964,7 +1048,12 @@ int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph,
     cb = [on_token](const Request& r, int tok) {
       if (on_token(r.number, tok) != 0) throw EngineError("the token callback stopped the run");
     };
-  run_requests(*static_cast<Engine*>(engine), *h.s, static_cast<Sampler*>(sampler), &st, cb, use_graph != 0, run_ahead != 0);
+  PromptLogits lcb;
+  if (on_logits)
+    lcb = [on_logits](const Request& r, const float* row, int64_t vocab) {
+      if (on_logits(r.number, row, vocab) != 0) throw EngineError("the logits callback stopped the run");
+    };
+  run_requests(*static_cast<Engine*>(engine), *h.s, static_cast<Sampler*>(sampler), &st, cb, use_graph != 0, run_ahead != 0, lcb);
   Json j = Json::object();
   j.set("prefill_ms", st.prefill_ms);
   j.set("prefill_tokens", st.prefill_tokens);
@@ -1147,6 +1236,8 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     answer(ops.compute_units());
   } else if (op == "fill_random") {
     ops.fill_random(arg(0), text ? text : "normal", num(0), num(1), (uint64_t)num(2));
+  } else if (op == "count_calls") {
+    ops.count_calls(num(0) != 0);
   } else if (op == "fill_zero") {
     ops.fill_zero(arg(0).data, arg(0).bytes());
   } else {

@@ -212,6 +212,22 @@ struct Engine::Impl {
       p->requests.push_back(en.request);
       p->n_tokens.push_back((int)en.tokens.size());
     }
+    // the pages are taken: whatever fails from here on (a part's plan, a buffer that cannot be had)
+    // gives them back before the error leaves
+    try {
+      fill(*p, entries, starts, M, n_want, graph, capturing);
+    } catch (...) {
+      undo(*p);
+      throw;
+    }
+    return p;
+  }
+
+  void fill(Prepared& prepared, const std::vector<StepEntry>& entries, const std::vector<int>& starts, int64_t M, int64_t n_want,
+            Graph* graph, bool capturing) {
+    Prepared* p = &prepared;
+    CacheManager& c = *e.cache;
+    const size_t R = entries.size();
     clear_slots();
 
     Workspace& work = graph ? graph->ws : ws;
@@ -311,7 +327,6 @@ struct Engine::Impl {
       ctx.views[g].page_size = e.page_size;
       ++gi;
     }
-    return p;
   }
 
   // The model over the step's tokens: embedding, the layers in run order, then final norm and

@@ -225,7 +225,8 @@ void Scheduler::abort_all() {
 
 // The loop of /root/reference/src/main.cpp:210-297 with admission, portions and preemption added.
 void run_requests(Engine& engine, Scheduler& scheduler, Sampler* sampler, GenerationStats* stats,
-                  const std::function<void(const Request&, int)>& on_token, bool use_graph, bool run_ahead) {
+                  const std::function<void(const Request&, int)>& on_token, bool use_graph, bool run_ahead,
+                  const PromptLogits& on_prompt_logits) {
   std::unique_ptr<Sampler> own;
   if (!sampler) {
     own.reset(new Sampler(engine.ops));
@@ -267,6 +268,18 @@ void run_requests(Engine& engine, Scheduler& scheduler, Sampler* sampler, Genera
       if (e.sample) f->asked.push_back(e.request);
     }
     Tensor logits = use_graph ? engine.step_graph(entries) : engine.step(entries);
+    if (on_prompt_logits && !before && logits.defined()) {
+      // rows of requests whose prompt this step finishes
+      std::vector<float> host;
+      for (size_t i = 0; i < f->asked.size(); ++i) {
+        if (!f->asked[i]->generated.empty()) continue;
+        if (host.empty()) {
+          host.resize((size_t)logits.numel());
+          engine.logits_to_host(logits, host.data());
+        }
+        on_prompt_logits(*f->asked[i], host.data() + i * (size_t)logits.shape[1], logits.shape[1]);
+      }
+    }
     if (!f->asked.empty()) {
       std::vector<SamplingParams> params;
       std::vector<int64_t> numbers, counters;

@@ -156,7 +156,13 @@ struct ModelSpec {
 // An architecture: config.json -> ModelSpec.  The reference gates on one string
 // (/root/reference/src/model.cpp:26-30); here that compare is a table.
 using SpecBuilder = std::function<ModelSpec(const Json& config)>;
-void register_architecture(const std::vector<std::string>& names, SpecBuilder builder);
+// The architecture's typed configuration: config.json read, validated and written back with its defaults
+// filled in (what a model folder's config.json says after a round trip).  Optional.
+using ConfigReader = std::function<Json(const Json& config)>;
+void register_architecture(const std::vector<std::string>& names, SpecBuilder builder, ConfigReader typed = nullptr);
+// {"architecture": the registered name that matched, "config": the typed configuration (the input itself if
+// the architecture registered no reader)}; ConfigError as spec_from_config
+Json typed_config(const Json& config);
 std::vector<std::string> registered_architectures();
 bool architecture_registered(const Json& config);
 ModelSpec spec_from_config(const Json& config);   // by architectures[0], else model_type; ConfigError lists what is registered
@@ -247,6 +253,14 @@ struct CacheNeed {
 // names are looked up in kernels.manifest beside this library or in $TINYINFER_KERNEL_DIR.
 void register_kernel_library(const std::string& name, const std::string& path);
 bool kernel_library_available(const std::string& name);
+// A function of a kernel library by name; the library is opened at the first call.  A part that lives
+// outside this library and brings kernels of its own registers their library and calls into it through
+// this (KernelError if the library or the function is not there).
+void* kernel_symbol(const std::string& library, const std::string& name);
+// Opens a shared library whose static initialisers (or its `extern "C" void tinyinfer_plugin_init()`)
+// register parts, architectures or kernel libraries: a model made of parts this library does not
+// know then builds, loads and steps like any other.  The plugin links with this library.
+void load_plugin(const std::string& path);
 
 class Workspace;       // named scratch buffers of a step
 struct Rows;           // activation rows, maybe a norm not computed yet
@@ -308,6 +322,10 @@ class Ops {
   // /root/reference/src/selftest.cpp:404-424): while on, every call records an event before and
   // after what it launches; the report waits for them and gives (name with sizes, calls, microseconds).
   void timing(bool on);
+  // the same list of calls without the times: nothing is recorded on the stream and no sum is added early, so
+  // the step runs exactly as it does unobserved; a name ends in what the call took ("[mfma]", "[generic]",
+  // "[fused]", ...).  For tests that check which kernel served a shape.
+  void count_calls(bool on);
   struct Timed { std::string name; int calls = 0; double us = 0; };
   std::vector<Timed> timing_report();
 
@@ -326,6 +344,7 @@ class Ops {
 
  private:
   void* launch_stream();
+  void took(const char* what);       // the call under way names the kernel it took (seen in the list of calls)
   void* stream_ = nullptr;
   int units_ = 0;
   DeviceBuffer partials_;
@@ -487,9 +506,13 @@ class Part {
   // the part reads the residual stream only through ctx.ops (so a product before it may leave
   // partial sums for the next norm); parts that do not say so find the residual complete
   virtual bool reads_through_ops() const { return false; }
+  // names of children(), in their order ("norm1", "mixer", ...; default "0", "1", ...)
+  virtual std::vector<std::string> child_slots() const;
   void walk(const std::function<void(Part&)>& fn);
   std::string prefix;
   uint64_t foreign_id = 0;     // non-zero: the part is implemented outside this library (see ForeignCalls)
+  std::string built_kind;      // what build_part made it from
+  Json built_from;
 };
 class EmbeddingPart : public Part { public: using Part::Part; const char* family() const override { return "embedding"; }
   virtual void forward(StepContext& ctx, const Tensor& x) = 0; };
@@ -534,6 +557,7 @@ struct ForeignCalls {
 };
 void set_foreign_calls(const ForeignCalls&);
 void set_foreign_error(const std::string& message);
+std::string take_foreign_error();      // the message left last on this thread; it is cleared
 // description: {"tensors": {name: {shape, role, init, a, b, optional}}, "cache_need": {...} | null, "fused": false}
 std::shared_ptr<Part> make_foreign_part(const std::string& family, uint64_t id, const std::string& prefix,
                                         const Json& description, const PartChildren& children);
@@ -843,9 +867,13 @@ struct GenerationStats {
 // `run_ahead`: while every running request decodes and nobody waits, the next step is launched
 // before the ids of the last one are read (it takes them from the device), so the device does
 // not wait for the host between steps; tokens are the same, `on_token` hears them one step later.
+// `on_prompt_logits`: called with the 32-bit logits (host memory, `vocab` of them) behind the last token of a
+// request's prompt, before its first token is drawn (what the reference's --verbose prints:
+// /root/reference/src/main.cpp:233-249); it costs a copy and a wait per such step.
+using PromptLogits = std::function<void(const Request&, const float* logits, int64_t vocab)>;
 void run_requests(Engine& engine, Scheduler& scheduler, Sampler* sampler = nullptr, GenerationStats* stats = nullptr,
                   const std::function<void(const Request&, int token)>& on_token = nullptr, bool use_graph = false,
-                  bool run_ahead = true);
+                  bool run_ahead = true, const PromptLogits& on_prompt_logits = nullptr);
 struct GenerateOptions {
   int max_new_tokens = 128;
   SamplingParams sampling;
@@ -871,6 +899,7 @@ const char* ti_error_message();
 typedef struct ti_tensor { void* data; int dtype; int ndim; int64_t shape[4]; int64_t stride[4]; } ti_tensor;
 
 int ti_kernels_register(const char* name, const char* path);
+int ti_load_plugin(const char* path);
 int ti_set_allocator(void* (*alloc)(void*, size_t), void (*release)(void*, void*), void* user);
 void ti_detach_allocator();
 int ti_set_foreign_calls(int (*call)(uint64_t, const char*, void*, const ti_tensor*, int, const char*, ti_tensor*));
@@ -878,6 +907,7 @@ void ti_set_foreign_error(const char* message);
 
 // configuration and registries
 int ti_qwen3_config(const char* config_json, const char** out_json);       // the typed configuration, validated
+int ti_typed_config(const char* config_json, const char** out_json);       // {"architecture", "config"} of whatever architecture config.json names
 int ti_spec_from_config(const char* config_json, const char** out_spec_json);
 int ti_architecture_registered(const char* config_json, int* out);
 int ti_registered_architectures(const char** out_json);
@@ -889,7 +919,14 @@ int ti_part_create(const char* family, const char* kind, const char* prefix, con
                    const char* const* child_slots, void* const* children, void** out);
 int ti_part_create_foreign(const char* family, uint64_t id, const char* prefix, const char* description_json,
                            int n_children, const char* const* child_slots, void* const* children, void** out);
+// kinds implemented outside this library: `make` builds one and returns a handle the caller owns (the library
+// takes a reference of its own); `ti_register_foreign_kind` enters the kind into the table of parts, so that a
+// spec that names it builds like any other (slots_json: for a block arrangement, {slot: family})
+int ti_set_foreign_factory(int (*make)(const char* family, const char* kind, const char* prefix, const char* params_json,
+                                       int n_children, const char* const* child_slots, void* const* children, void** out));
+int ti_register_foreign_kind(const char* family, const char* kind, const char* slots_json);
 void ti_part_release(void* part);
+int ti_part_child(void* part, int index, void** out);                  // a new handle to the index-th of the part's children
 int ti_part_tensors(void* part, const char** out_json);
 int ti_part_cache_need(void* part, const char** out_json);
 int ti_part_info(void* part, const char** out_json);
@@ -913,6 +950,9 @@ int ti_ctx_buf(void* ctx, const char* name, int dtype, int ndim, const int64_t* 
 int ti_ctx_ops(void* ctx, void** out_ops);
 
 // model
+int ti_model_from_spec(const char* spec_json, void** out);              // every part through the table of parts
+// a new handle to a part of the model: which = "embedding" | "block" (index) | "final_norm" | "head"
+int ti_model_part(void* model, const char* which, int index, void** out);
 int ti_model_create(const char* meta_json, void* embedding, int n_blocks, void* const* blocks, void* final_norm,
                     void* head, void** out);
 void ti_model_release(void* model);
@@ -978,8 +1018,10 @@ int ti_scheduler_set_next_number(void* scheduler, int64_t number);
 int ti_scheduler_state(void* scheduler, const char** out_json);
 int ti_scheduler_request(void* scheduler, int64_t number, const char** out_json);
 // on_token returns 0; anything else stops the run (the requests still held are given back, and the call fails)
+// on_logits (or null): the logits behind the last token of a request's prompt, as run_requests' on_prompt_logits
 int ti_run_requests(void* engine, void* scheduler, void* sampler, int use_graph, int run_ahead,
-                    int (*on_token)(int64_t number, int token), const char** out_stats_json);
+                    int (*on_token)(int64_t number, int token), int (*on_logits)(int64_t number, const float* row, int64_t vocab),
+                    const char** out_stats_json);
 
 // the kernels through an Ops object (what the kernel tests and foreign parts call)
 int ti_ops_create(void* stream, void** out);

@@ -235,13 +235,8 @@ void Model::write_random_folder(const std::string& dir, const Json& config_out, 
 
 void Model::write_folder(const std::string& dir, const Json& config, uint64_t seed, const std::string& store_dtype) {
   Model model(spec_from_config(config));
-  Json out = config;
   // a typed configuration writes itself back with its defaults filled in
-  bool qwen = false;
-  if (const Json* mt = config.find("model_type")) qwen = mt->type() == Json::String && mt->as_string() == "qwen3";
-  if (const Json* a = config.find("architectures"))
-    if (a->type() == Json::Array && a->size() && (*a)[0].type() == Json::String) qwen = qwen || (*a)[0].as_string() == "Qwen3ForCausalLM";
-  if (qwen) out = Qwen3Config::from_json(config).to_json();
+  const Json out = typed_config(config).at("config");
   model.write_random_folder(dir, out, seed, store_dtype);
 }
 

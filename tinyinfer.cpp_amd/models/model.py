@@ -1,6 +1,6 @@
-"""A model put together from a `ModelSpec`: parts built through the part
-registry, handed to the host library, which gathers their cache needs into
-groups and keeps the run order (models/model.cpp)."""
+"""A model put together from a `ModelSpec` by the host library (models/model.cpp):
+its parts are built through the one table of parts, their cache needs gathered
+into groups, the run order kept as a list.  This class names the result."""
 from __future__ import annotations
 
 import ctypes
@@ -8,8 +8,8 @@ import json
 from typing import Dict, List, Tuple
 
 from .. import native
-from ..parts.base import join, part_handle
-from ..parts.registry import _PARTS, build_part
+from ..parts.base import part_handle
+from ..parts.builtin import adopt
 from ..spec import ModelSpec, TensorNeed, cache_need_from_dict
 
 
@@ -18,39 +18,18 @@ class Model:
         self.spec = spec
         self.vocab_size = spec.vocab_size
         self.hidden_size = spec.hidden_size
-        self.embedding = build_part("embedding", spec.embedding, spec.embedding.name)
-        self.blocks = []
-        for ls in spec.layers:
-            key = ("block", ls.block.kind)
-            if key not in _PARTS:
-                raise KeyError(f"no block arrangement of kind {ls.block.kind!r}")
-            slots = getattr(_PARTS[key], "slots", None)
-            if slots is None:
-                raise TypeError(f"block arrangement {ls.block.kind!r} declares no `slots`")
-            built = {}
-            for slot, family in slots.items():
-                if slot not in ls.parts:
-                    raise KeyError(f"layer '{ls.prefix}': block '{ls.block.kind}' needs a '{slot}' part")
-                ps = ls.parts[slot]
-                built[slot] = build_part(family, ps, join(ls.prefix, ps.name))
-            self.blocks.append(_PARTS[key](prefix=ls.prefix, **built, **ls.block.params))
-        self.final_norm = build_part("norm", spec.final_norm, spec.final_norm.name)
-        self.head = build_part("head", spec.lm_head, spec.lm_head.name)
         self.run_order = spec.run_order()
-        for i in self.run_order:
-            if not 0 <= i < len(self.blocks):
-                raise ValueError(f"schedule names layer {i}, but there are {len(self.blocks)}")
-        meta = {"architecture": spec.architecture, "vocab_size": spec.vocab_size, "hidden_size": spec.hidden_size,
-                "schedule": spec.schedule, "eos_token_ids": list(spec.eos_token_ids),
-                "max_position_embeddings": spec.max_position_embeddings,
-                "cache_from": [ls.cache_from for ls in spec.layers]}
-        handles = (ctypes.c_void_p * max(1, len(self.blocks)))(*[part_handle(b).ptr for b in self.blocks])
+        # the library builds every part through its table of parts (kinds registered from Python are made
+        # by their Python classes on the way); what stands here afterwards are views of its parts
         try:
-            self._ptr = native.pointer("ti_model_create", json.dumps(meta).encode(), part_handle(self.embedding).ptr,
-                                       len(self.blocks), handles, part_handle(self.final_norm).ptr,
-                                       part_handle(self.head).ptr)
+            self._ptr = native.pointer("ti_model_from_spec", json.dumps(spec.to_dict()).encode())
         except native.ConfigError as e:
             raise ValueError(str(e)) from None
+        part = lambda which, i=0: adopt(native.pointer("ti_model_part", self._ptr, which, i))      # noqa: E731
+        self.embedding = part(b"embedding")
+        self.blocks = [part(b"block", i) for i in range(len(spec.layers))]
+        self.final_norm = part(b"final_norm")
+        self.head = part(b"head")
         # groups of cache layers with the same need, and per run: id(part) -> (group, cache layer)
         groups = json.loads(native.text("ti_model_cache_groups", self._ptr))
         self.cache_groups: List[Tuple[object, int]] = [(cache_need_from_dict(g["need"]), g["layers"]) for g in groups]

@@ -77,16 +77,25 @@ _ERRORS = {"ConfigError": ConfigError, "CacheError": CacheError, "OutOfPages": O
 FOREIGN_CALL = ctypes.CFUNCTYPE(c_int, c_u64, c_char_p, c_void_p, P(ti_tensor), c_int, c_char_p, P(ti_tensor))
 ALLOC = ctypes.CFUNCTYPE(c_void_p, c_void_p, c_size_t)
 RELEASE = ctypes.CFUNCTYPE(None, c_void_p, c_void_p)
+FOREIGN_MAKE = ctypes.CFUNCTYPE(c_int, c_char_p, c_char_p, c_char_p, c_char_p, c_int, P(c_char_p), P(c_void_p), P(c_void_p))
 ON_TOKEN = ctypes.CFUNCTYPE(c_int, c_i64, c_int)
+ON_LOGITS = ctypes.CFUNCTYPE(c_int, c_i64, P(c_float), c_i64)
 
 _OUT_TEXT = P(c_char_p)
 _OUT_PTR = P(c_void_p)
 _TT = P(ti_tensor)
 _SIGNATURES = {
     "ti_kernels_register": [c_char_p, c_char_p],
+    "ti_load_plugin": [c_char_p],
     "ti_set_allocator": [ALLOC, RELEASE, c_void_p],
     "ti_set_foreign_calls": [FOREIGN_CALL],
     "ti_qwen3_config": [c_char_p, _OUT_TEXT],
+    "ti_typed_config": [c_char_p, _OUT_TEXT],
+    "ti_set_foreign_factory": [FOREIGN_MAKE],
+    "ti_register_foreign_kind": [c_char_p, c_char_p, c_char_p],
+    "ti_part_child": [c_void_p, c_int, _OUT_PTR],
+    "ti_model_from_spec": [c_char_p, _OUT_PTR],
+    "ti_model_part": [c_void_p, c_char_p, c_int, _OUT_PTR],
     "ti_spec_from_config": [c_char_p, _OUT_TEXT],
     "ti_architecture_registered": [c_char_p, P(c_int)],
     "ti_registered_architectures": [_OUT_TEXT],
@@ -151,7 +160,7 @@ _SIGNATURES = {
     "ti_scheduler_set_next_number": [c_void_p, c_i64],
     "ti_scheduler_state": [c_void_p, _OUT_TEXT],
     "ti_scheduler_request": [c_void_p, c_i64, _OUT_TEXT],
-    "ti_run_requests": [c_void_p, c_void_p, c_void_p, c_int, c_int, ON_TOKEN, _OUT_TEXT],
+    "ti_run_requests": [c_void_p, c_void_p, c_void_p, c_int, c_int, ON_TOKEN, ON_LOGITS, _OUT_TEXT],
     "ti_ops_create": [c_void_p, _OUT_PTR],
     "ti_ops_switch": [c_void_p, c_char_p, c_int, P(c_int)],
     "ti_ops_timing_report": [c_void_p, _OUT_TEXT],
@@ -196,6 +205,7 @@ def lib() -> ctypes.CDLL:
         handle.ti_portion_launch.argtypes = [c_int] * 5 + [P(c_int)]
         handle.ti_detach_allocator.restype = None
         handle.ti_set_foreign_calls(_foreign_trampoline)
+        handle.ti_set_foreign_factory(_foreign_make_trampoline)
         _lib = handle
         # kernel libraries that are built already are made known; the others when they are asked for
         for name in _build.SOURCES:
@@ -207,6 +217,12 @@ def lib() -> ctypes.CDLL:
 
 
 _registered = set()
+
+
+def load_plugin(path: str) -> None:
+    """Open a shared library that registers parts, architectures or kernel libraries with the host library
+    (`tinyinfer::load_plugin`): a model made of them then builds, loads and steps like any other."""
+    call("ti_load_plugin", path.encode())
 
 
 def ensure_kernels(names: Sequence[str]) -> None:
@@ -402,6 +418,11 @@ def register_foreign(part) -> int:
     return i
 
 
+def foreign_object(part_id: int):
+    """The Python part behind a part of the library that is implemented here."""
+    return _foreign_parts[part_id]
+
+
 def forget_contexts() -> None:
     """The step is over: what its Python-side contexts kept alive may go."""
     _contexts.clear()
@@ -454,6 +475,22 @@ def _dispatch(part, op: str, ctx_ptr, args, n_args: int, names: Optional[bytes],
 def _foreign_trampoline(part_id, op, ctx_ptr, args, n_args, names, result):
     try:
         _dispatch(_foreign_parts[part_id], op.decode(), ctx_ptr, args, n_args, names, result)
+        return 0
+    except BaseException as e:  # noqa: BLE001  (an exception must not unwind through the library)
+        _lib.ti_set_foreign_error(f"{type(e).__name__}: {e}\n{traceback.format_exc()}".encode())
+        return 1
+
+
+@FOREIGN_MAKE
+def _foreign_make_trampoline(family, kind, prefix, params_json, n_children, slots, children, out):
+    """The library builds a model and comes to a kind that was registered from Python: make the part here and
+    hand back the library's part behind it."""
+    try:
+        from .parts.base import part_handle
+        from .parts.registry import make_registered
+        kids = [(slots[i].decode(), children[i]) for i in range(n_children)]
+        part = make_registered(family.decode(), kind.decode(), prefix.decode(), json.loads(params_json.decode()), kids)
+        out[0] = part_handle(part).ptr
         return 0
     except BaseException as e:  # noqa: BLE001  (an exception must not unwind through the library)
         _lib.ti_set_foreign_error(f"{type(e).__name__}: {e}\n{traceback.format_exc()}".encode())

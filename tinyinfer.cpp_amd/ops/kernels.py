@@ -25,10 +25,7 @@ _C_TYPES = {"int": ctypes.c_int, "long": ctypes.c_long, "float": ctypes.c_float,
 
 def required_libraries(dtype: str):
     """The kernel libraries a model of this dtype needs (what a first call compiles)."""
-    libs = ["core", "gemm_generic", "attention_generic", "sampling"]
-    if dtype == "bfloat16":
-        libs += [n for n in ("gemm_bf16", "attention_bf16") if os.path.isfile(os.path.join(_build.HERE, _build.SOURCES[n]))]
-    return libs
+    return _build.libraries_for(dtype)
 
 
 def header_signatures(text: str) -> Dict[str, tuple]:
@@ -201,6 +198,11 @@ class Ops:
     def timing(self, on: bool) -> None:
         """Switch per-call timing with events on or off (see `Ops::timing`)."""
         self._call("timing", [], [int(bool(on))], libs=["core"])
+
+    def count_calls(self, on: bool) -> None:
+        """List the calls without timing them (see `Ops::count_calls`): a step runs exactly as it does unobserved;
+        `timing_report()` then gives the names, each ending in what the call took ("[mfma]", "[generic]", "[fused]")."""
+        self._call("count_calls", [], [int(bool(on))], libs=["core"])
 
     def timing_report(self):
         """[{"name", "calls", "us"}] of the calls since timing was switched on (or last reported)."""

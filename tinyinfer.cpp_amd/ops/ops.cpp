@@ -255,6 +255,18 @@ void register_kernel_library(const std::string& name, const std::string& path) {
   lib_paths()[name] = path;
 }
 
+void* kernel_symbol(const std::string& lib, const std::string& name) {
+  void* s = dlsym(library(lib), name.c_str());
+  if (!s) throw KernelError("kernel library '" + lib + "' does not export " + name);
+  return s;
+}
+
+void load_plugin(const std::string& path) {
+  void* handle = dlopen(path.c_str(), RTLD_NOW | RTLD_GLOBAL);
+  if (!handle) throw FileError("cannot load the plugin " + path + ": " + dlerror());
+  if (void* init = dlsym(handle, "tinyinfer_plugin_init")) ((void (*)())init)();
+}
+
 bool kernel_library_available(const std::string& name) {
   try {
     library(name);
@@ -272,14 +284,17 @@ struct Ops::Timing {
   struct Rec { std::string name; hipEvent_t a, b; };
   std::vector<Rec> recs;
   int depth = 0;
+  bool names_only = false;      // calls are listed, not timed: nothing is recorded on the stream, nothing is flushed
+  std::string tag;              // what the call under way says about the kernel it took
 };
 Ops::Ops(void* stream) : stream_(stream) {}
 Ops::~Ops() {
   if (timing_)
-    for (auto& r : timing_->recs) {
-      (void)hipEventDestroy(r.a);
-      (void)hipEventDestroy(r.b);
-    }
+    for (auto& r : timing_->recs)
+      if (r.a) {
+        (void)hipEventDestroy(r.a);
+        (void)hipEventDestroy(r.b);
+      }
 }
 
 void Ops::timing(bool on) {
@@ -291,14 +306,27 @@ void Ops::timing(bool on) {
   }
 }
 
+void Ops::count_calls(bool on) {
+  if (timing_ && !timing_->names_only) timing(false);
+  if (on && !timing_) {
+    timing_.reset(new Timing());
+    timing_->names_only = true;
+  }
+  if (!on) timing_.reset();
+}
+
+void Ops::took(const char* what) {
+  if (timing_ && timing_->depth == 1) timing_->tag = what;
+}
+
 std::vector<Ops::Timed> Ops::timing_report() {
   std::vector<Timed> out;
   if (!timing_) return out;
-  hip_check(hipStreamSynchronize((hipStream_t)stream_), "hipStreamSynchronize");
+  if (!timing_->names_only) hip_check(hipStreamSynchronize((hipStream_t)stream_), "hipStreamSynchronize");
   std::map<std::string, size_t> index;
   for (auto& r : timing_->recs) {
     float ms = 0.f;
-    (void)hipEventElapsedTime(&ms, r.a, r.b);
+    if (r.a) (void)hipEventElapsedTime(&ms, r.a, r.b);
     auto it = index.find(r.name);
     if (it == index.end()) {
       it = index.emplace(r.name, out.size()).first;
@@ -306,8 +334,10 @@ std::vector<Ops::Timed> Ops::timing_report() {
     }
     out[it->second].calls += 1;
     out[it->second].us += ms * 1e3;
-    (void)hipEventDestroy(r.a);
-    (void)hipEventDestroy(r.b);
+    if (r.a) {
+      (void)hipEventDestroy(r.a);
+      (void)hipEventDestroy(r.b);
+    }
   }
   timing_->recs.clear();
   return out;
@@ -321,11 +351,15 @@ struct TimedScope {
   template <class F> TimedScope(Ops& o, F&& name) : ops(o) {
     if (!ops.timing_) return;
     if (ops.timing_->depth++ > 0) return;
-    if (ops.pending_.out) ops.flush();          // the sums of the call before are not this call's time
     Ops::Timing::Rec r;
     r.name = name();
-    if (hipEventCreate(&r.a) != hipSuccess || hipEventCreate(&r.b) != hipSuccess) return;
-    (void)hipEventRecord(r.a, (hipStream_t)ops.stream_);
+    r.a = r.b = nullptr;
+    ops.timing_->tag.clear();
+    if (!ops.timing_->names_only) {
+      if (ops.pending_.out) ops.flush();          // the sums of the call before are not this call's time
+      if (hipEventCreate(&r.a) != hipSuccess || hipEventCreate(&r.b) != hipSuccess) return;
+      (void)hipEventRecord(r.a, (hipStream_t)ops.stream_);
+    }
     index = ops.timing_->recs.size();
     ops.timing_->recs.push_back(r);
     active = true;
@@ -333,7 +367,10 @@ struct TimedScope {
   ~TimedScope() {
     if (!ops.timing_) return;
     --ops.timing_->depth;
-    if (active) (void)hipEventRecord(ops.timing_->recs[index].b, (hipStream_t)ops.stream_);
+    if (!active) return;
+    Ops::Timing::Rec& r = ops.timing_->recs[index];
+    if (!ops.timing_->tag.empty()) r.name += " " + ops.timing_->tag;
+    if (r.b) (void)hipEventRecord(r.b, (hipStream_t)ops.stream_);
   }
 };
 static std::string dims(const Tensor& t) {
@@ -506,6 +543,7 @@ bool Ops::linear_with_norm(const Rows& a, const Tensor& w, const Tensor& out, Ep
                                                     (hipStream_t)launch_stream());
   if (rc == 3) return false;
   check("gemm_bf16", rc, "linear(normed)");
+  took("[fused]");
   return true;
 }
 
@@ -551,6 +589,7 @@ void Ops::linear(const Tensor& a, const Tensor& w, const Tensor& out, Epilogue e
           pending_.count = out.numel();
           pending_.splits = splits;
         }
+        took(splits ? "[mfma, K split, sums left]" : "[mfma]");
         return;
       }
       if (rc != 3) check("gemm_bf16", rc, "linear(bf16, split K)");
@@ -560,14 +599,21 @@ void Ops::linear(const Tensor& a, const Tensor& w, const Tensor& out, Epilogue e
       if (!partials_.data()) partials_ = DeviceBuffer(PARTIALS_BYTES);
       int rc = KERNEL("gemm_bf16", ti_gemm_bf16_store_split)(a.data, w.data, out.data, (int)M, (int)N, (int)K, lda,
                                                              partials_.data(), (long)PARTIALS_BYTES, (hipStream_t)stream);
-      if (rc == 0) return;
+      if (rc == 0) {
+        took("[mfma, K split]");
+        return;
+      }
       if (rc != 3) check("gemm_bf16", rc, "linear(bf16, split K, stored)");
     }
     int rc = KERNEL("gemm_bf16", ti_gemm_bf16)(a.data, w.data, out.data, (int)M, (int)N, (int)K, lda, (int)epi,
                                                (hipStream_t)launch_stream());
-    if (rc == 0) return;
+    if (rc == 0) {
+      took("[mfma]");
+      return;
+    }
     if (rc != 3) check("gemm_bf16", rc, "linear(bf16)");     // 3: shape not served, the generic kernel takes it
   }
+  took("[generic]");
   int rc = KERNEL("gemm_generic", ti_gemm_generic)(dt, a.data, w.data, out.data, (int)M, (int)N, (int)K, lda, (int)epi,
                                                    (hipStream_t)launch_stream());
   check("gemm_generic", rc, "linear");
@@ -598,6 +644,7 @@ bool Ops::qkv_prepared(const Rows& a, const Tensor& w, const float* q_w, const f
       (hipStream_t)launch_stream());
   if (rc == 3) return false;
   check("gemm_bf16", rc, "qkv_prepared");
+  took("[fused]");
   return true;
 }
 
@@ -706,6 +753,7 @@ bool Ops::attention_from_projections(const AttentionWork& work, Workspace& ws, c
       heads, kv_heads, head_dim, P, scale, window, S, (hipStream_t)launch_stream());
   if (rc == 3) return false;
   check("attention_bf16", rc, "attention(decode, prepared)");
+  took(S > 1 ? "[fused, runs]" : "[fused]");
   return true;
 }
 
@@ -768,6 +816,7 @@ void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& v
       }
     }
   }
+  took(done ? "[mfma]" : "[generic]");
   if (!done)
     attention_rows(q, pool, view, work.positions, work.slots, out, heads, kv_heads, head_dim, scale, window);
 }

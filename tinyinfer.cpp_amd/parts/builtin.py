@@ -1,21 +1,21 @@
-"""The built-in parts, named from Python.  Each class holds the sizes it was built
-with and a handle to the part of the host library that does the work
-(parts/parts.cpp, where the formulas and their places in the reference are
-given); `forward` hands torch tensors across.  Run inside a step, a part gets the
-step's own context; run on its own (a test of one part), it gets a context of
-its own made from the caller's `ctx.dtype` and `ctx.positions`.
+"""Parts of the host library, seen from Python.  A view holds a handle to the library's
+part (parts/parts.cpp, where the formulas and their places in the reference are given)
+and what the part was built from; `forward` hands torch tensors across.  Every family
+has a view class, so a kind that the library or a plugin registers is usable from
+Python without a line here; the built-in kinds have named views that add their
+defaults and conveniences.  Run inside a step, a part gets the step's own context;
+run on its own (a test of one part), it gets a context of its own made from the
+caller's `ctx.dtype` and `ctx.positions`.
 """
 from __future__ import annotations
 
 import ctypes
 import json
 import math
-from typing import Optional
 
 from .. import native
-from ..spec import PartSpec, TensorNeed, cache_need_from_dict
-from .base import Handle, Part, children_arrays, part_handle
-from .registry import build_part, register_part
+from ..spec import TensorNeed, cache_need_from_dict
+from .base import Handle, Part
 
 ti_tensor = native.ti_tensor
 
@@ -52,15 +52,35 @@ def native_context(ctx, n_rows: int = 0, tokens=None) -> int:
 
 
 class NativePart(Part):
-    """A part of the host library.  `kind` names it in its family; `params` is what it was built from."""
+    """A part of the host library.  `family` and `kind` name it; `params` is what it was built from (each
+    entry also reads as an attribute, and so does every tensor the part holds: `part.w_qkv`)."""
     kind = ""
 
-    def _create(self, params: dict, children=()):
-        children = list(children)
-        n, slots, handles = children_arrays(children)
-        self._children = [p for _, p in children]
-        self._ti_handle = Handle(native.pointer("ti_part_create", self.family.encode(), self.kind.encode(),
-                                                self.prefix.encode(), json.dumps(params).encode(), n, slots, handles))
+    def _adopted(self, handle: Handle, info: dict):
+        self.prefix = info["prefix"]
+        self.family, self.kind = info["family"], info["built_kind"] or info["kind"]
+        self.params = info["params"]
+        self._ti_handle = handle
+        self._slots = list(info["slots"])
+        self._children = []
+        for i, slot in enumerate(self._slots):
+            child = adopt(native.pointer("ti_part_child", handle.ptr, i))
+            self._children.append(child)
+            if not slot.isdigit():
+                self.__dict__[slot] = child
+        return self
+
+    def __getattr__(self, name):
+        if name.startswith("_"):
+            raise AttributeError(name)
+        params = self.__dict__.get("params") or {}
+        if name in params:
+            return params[name]
+        if "_ti_handle" in self.__dict__:
+            t = self.held(name)
+            if t is not None:
+                return t
+        raise AttributeError(f"{type(self).__name__} ({self.__dict__.get('kind')}) has no parameter, child or tensor {name!r}")
 
     def tensors(self):
         d = json.loads(native.text("ti_part_tensors", self._ti_handle.ptr))
@@ -71,6 +91,9 @@ class NativePart(Part):
 
     def cache_need(self):
         return cache_need_from_dict(json.loads(native.text("ti_part_cache_need", self._ti_handle.ptr)))
+
+    def info(self) -> dict:
+        return json.loads(native.text("ti_part_info", self._ti_handle.ptr))
 
     def load(self, tensors) -> None:
         """Copy `tensors` (by name; torch tensors already in the dtype their role asks for) into the
@@ -101,47 +124,18 @@ class NativePart(Part):
         return [native.wrap(res[i]) for i in range(n_results)]
 
 
-class Embedding(NativePart):
-    family, kind = "embedding", "table"
-
-    def __init__(self, prefix: str, vocab: int, dim: int):
-        super().__init__(prefix)
-        self.vocab, self.dim = int(vocab), int(dim)
-        self._create({"vocab": self.vocab, "dim": self.dim})
-
-    weight = property(lambda self: self.held("weight"))
-
+# ----------------------------------------------------------- one view per family
+class NativeEmbedding(NativePart):
     def forward(self, ctx, tokens, x):
         self._call("forward", native_context(ctx, tokens.shape[0], tokens), [x])
 
 
-class LMHead(NativePart):
-    """`tied`: True reads `tied_to`; False reads its own `weight`; None takes its own weight if the
-    checkpoint holds one and `tied_to` otherwise."""
-    family, kind = "head", "linear"
-
-    def __init__(self, prefix: str, vocab: int, dim: int, tied, tied_to: str):
-        super().__init__(prefix)
-        self.vocab, self.dim, self.tied, self.tied_to = int(vocab), int(dim), tied, tied_to
-        self._create({"vocab": self.vocab, "dim": self.dim, "tied": tied, "tied_to": tied_to})
-
-    weight = property(lambda self: self.held("weight"))
-
+class NativeHead(NativePart):
     def forward(self, ctx, h_rows):
         return self._call("forward", native_context(ctx, h_rows.shape[0]), [h_rows], n_results=1)[0]
 
 
-class RMSNorm(NativePart):
-    family, kind = "norm", "rmsnorm"
-    can_be_lazy = True
-
-    def __init__(self, prefix: str, dim: int, eps: float):
-        super().__init__(prefix)
-        self.dim, self.eps = int(dim), float(eps)
-        self._create({"dim": self.dim, "eps": self.eps})
-
-    weight = property(lambda self: self.held("weight"))
-
+class NativeNorm(NativePart):
     def forward(self, ctx, x, out=None, rows=None, lazy=False):
         """x: f32 [M, dim].  Returns the normed rows in the compute dtype; with `rows` (i32 [N]) only
         those rows of x are read, in that order."""
@@ -152,108 +146,93 @@ class RMSNorm(NativePart):
             return out
         return res
 
+    can_be_lazy = property(lambda self: self.info()["can_be_lazy"])
 
-class RotaryNeox(NativePart):
-    family, kind = "pos", "rope_neox"
 
-    def __init__(self, prefix: str, head_dim: int, theta: float):
-        super().__init__(prefix)
-        if head_dim % 2:
-            raise ValueError(f"rotary: head_dim {head_dim} must be even")
-        self.head_dim, self.theta = int(head_dim), float(theta)
-        self._create({"head_dim": self.head_dim, "theta": self.theta})
+class NativePos(NativePart):
+    def apply(self, ctx, q, k):
+        """In place on f32 [M, heads, hd] views (strided rows allowed)."""
+        self._call("apply", native_context(ctx, q.shape[0]), [q] + ([k] if k is not None else []))
 
+    def prepare(self, ops, max_positions: int):
+        """Whatever the part tabulates for positions [0, max_positions)."""
+        native.use_torch_allocator()
+        self._call("prepare", None, flags=int(max_positions))
+
+
+class NativeMixer(NativePart):
+    """Mixers and feed-forwards: `forward(ctx, h, x)` adds the part's output into x."""
+
+    def forward(self, ctx, h, x):
+        self._call("forward", native_context(ctx, h.shape[0]), [h, x])
+
+    takes_lazy_norm = property(lambda self: self.info()["takes_lazy_norm"])
+
+
+class NativeBlock(NativePart):
+    def forward(self, ctx, x):
+        self._call("forward", native_context(ctx, x.shape[0]), [x])
+
+
+FAMILY_VIEWS = {"embedding": NativeEmbedding, "head": NativeHead, "norm": NativeNorm, "pos": NativePos, "mixer": NativeMixer,
+                "ffn": NativeMixer, "block": NativeBlock}
+
+
+# ------------------------------------------------------- the built-in kinds, by name
+class Embedding(NativeEmbedding):
+    pass
+
+
+class LMHead(NativeHead):
+    """`tied`: True reads `tied_to`; False reads its own `weight`; None takes its own weight if the
+    checkpoint holds one and `tied_to` otherwise."""
+
+
+class RMSNorm(NativeNorm):
+    pass
+
+
+class RotaryNeox(NativePos):
     def to(self, device):
         native.use_torch_allocator()
         self._call("prepare", None, flags=0)
         return self
 
-    def prepare(self, ops, max_positions: int):
-        """Tabulate cos and sin for positions [0, max_positions)."""
-        native.use_torch_allocator()
-        self._call("prepare", None, flags=int(max_positions))
-
-    inv_freq = property(lambda self: self.held("inv_freq"))
-    table = property(lambda self: self.held("table"))
-
     def fused_rotation(self):
         """What the fused norm/rotate/cache-write kernels read."""
-        return {"inv_freq": self.inv_freq, "table": self.table}
-
-    def apply(self, ctx, q, k):
-        """In place on f32 [M, heads, hd] views (strided rows allowed)."""
-        self._call("apply", native_context(ctx, q.shape[0]), [q] + ([k] if k is not None else []))
+        return {"inv_freq": self.held("inv_freq"), "table": self.held("table")}
 
 
-class SwiGLU(NativePart):
-    family, kind = "ffn", "swiglu"
-    takes_lazy_norm = True
-
-    def __init__(self, prefix: str, hidden: int, intermediate: int):
-        super().__init__(prefix)
-        self.hidden, self.intermediate = int(hidden), int(intermediate)
-        self._create({"hidden": self.hidden, "intermediate": self.intermediate})
-
-    w_gate_up = property(lambda self: self.held("w_gate_up"))
-    w_down = property(lambda self: self.held("w_down"))
-
-    def forward(self, ctx, h, x):
-        self._call("forward", native_context(ctx, h.shape[0]), [h, x])
+class SwiGLU(NativeMixer):
+    pass
 
 
-class Attention(NativePart):
-    family, kind = "mixer", "attention"
-    takes_lazy_norm = True
-
-    def __init__(self, prefix: str, hidden: int, heads: int, kv_heads: int, head_dim: int, qk_norm: bool = True,
-                 eps: float = 1e-6, window: Optional[int] = None, scale: Optional[float] = None, pos=None,
-                 shares_kv: bool = False):
-        super().__init__(prefix)
-        if heads % kv_heads:
-            raise ValueError(f"attention: heads {heads} not a multiple of kv_heads {kv_heads}")
-        self.hidden, self.heads, self.kv_heads, self.head_dim = int(hidden), int(heads), int(kv_heads), int(head_dim)
-        self.qk_norm, self.eps = bool(qk_norm), float(eps)
-        self.window = None if window is None else int(window)
-        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
-        self.shares_kv = bool(shares_kv)
-        if isinstance(pos, dict):
-            pos = PartSpec.from_dict(pos)
-        self.pos = build_part("pos", pos, prefix) if pos is not None else None
-        self.nq = self.heads * self.head_dim
-        self.nk = 0 if self.shares_kv else self.kv_heads * self.head_dim
-        params = {"hidden": self.hidden, "heads": self.heads, "kv_heads": self.kv_heads, "head_dim": self.head_dim,
-                  "qk_norm": self.qk_norm, "eps": self.eps, "window": self.window, "scale": self.scale,
-                  "shares_kv": self.shares_kv}
-        self._create(params, [("pos", self.pos)] if self.pos is not None else [])
-
-    w_qkv = property(lambda self: self.held("w_qkv"))
-    w_o = property(lambda self: self.held("w_o"))
-    q_norm_w = property(lambda self: self.held("q_norm_w"))
-    k_norm_w = property(lambda self: self.held("k_norm_w"))
-
-    def forward(self, ctx, h, x):
-        self._call("forward", native_context(ctx, h.shape[0]), [h, x])
+class Attention(NativeMixer):
+    window = property(lambda self: self.params.get("window"))
+    qk_norm = property(lambda self: self.params.get("qk_norm", True))
+    shares_kv = property(lambda self: bool(self.params.get("shares_kv")))
+    scale = property(lambda self: self.params["scale"] if self.params.get("scale") is not None
+                     else 1.0 / math.sqrt(self.params["head_dim"]))
+    nq = property(lambda self: self.params["heads"] * self.params["head_dim"])
+    nk = property(lambda self: 0 if self.shares_kv else self.params["kv_heads"] * self.params["head_dim"])
+    pos = None            # (an attention without a position encoding has no such child)
 
 
-class PreNormBlock(NativePart):
+class PreNormBlock(NativeBlock):
     """x += mixer(norm1(x)); x += ffn(norm2(x))."""
-    family, kind = "block", "pre_norm"
-    # which family each named slot of this arrangement is built from
-    slots = {"norm1": "norm", "mixer": "mixer", "norm2": "norm", "ffn": "ffn"}
-
-    def __init__(self, prefix: str, norm1, mixer, norm2, ffn):
-        super().__init__(prefix)
-        self.norm1, self.mixer, self.norm2, self.ffn = norm1, mixer, norm2, ffn
-        self._create({}, [("norm1", norm1), ("mixer", mixer), ("norm2", norm2), ("ffn", ffn)])
-
-    def forward(self, ctx, x):
-        self._call("forward", native_context(ctx, x.shape[0]), [x])
 
 
-register_part("embedding", "table", Embedding)
-register_part("head", "linear", LMHead)
-register_part("norm", "rmsnorm", RMSNorm)
-register_part("pos", "rope_neox", RotaryNeox)
-register_part("ffn", "swiglu", SwiGLU)
-register_part("mixer", "attention", Attention)
-register_part("block", "pre_norm", PreNormBlock)
+KIND_VIEWS = {("embedding", "table"): Embedding, ("head", "linear"): LMHead, ("norm", "rmsnorm"): RMSNorm,
+              ("pos", "rope_neox"): RotaryNeox, ("ffn", "swiglu"): SwiGLU, ("mixer", "attention"): Attention,
+              ("block", "pre_norm"): PreNormBlock}
+
+
+def adopt(ptr: int):
+    """The Python object for a part of the library, given a handle that becomes this object's own: the
+    Python part itself if the part is implemented here, else a view of the library's part."""
+    handle = Handle(ptr)
+    info = json.loads(native.text("ti_part_info", ptr))
+    if info["foreign_id"]:
+        return native.foreign_object(info["foreign_id"])         # (the handle goes; the part keeps its own)
+    cls = KIND_VIEWS.get((info["family"], info["built_kind"] or info["kind"])) or FAMILY_VIEWS[info["family"]]
+    return cls.__new__(cls)._adopted(handle, info)

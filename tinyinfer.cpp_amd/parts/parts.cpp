@@ -26,6 +26,13 @@
 
 namespace tinyinfer {
 
+std::vector<std::string> Part::child_slots() const {
+  std::vector<std::string> names;
+  const size_t n = children().size();
+  for (size_t i = 0; i < n; ++i) names.push_back(std::to_string(i));
+  return names;
+}
+
 void Part::walk(const std::function<void(Part&)>& fn) {
   fn(*this);
   for (const auto& c : children()) c->walk(fn);
@@ -113,7 +120,15 @@ std::shared_ptr<Part> build_part(const std::string& family, const PartSpec& spec
     }
     factory = it->second.factory;
   }
-  return factory(prefix, spec.params, children);
+  std::shared_ptr<Part> part = factory(prefix, spec.params, children);
+  if (!part) throw ConfigError("the factory of " + family + " '" + spec.kind + "' returned no part");
+  if (family != part->family())
+    throw ConfigError("the factory of " + family + " '" + spec.kind + "' returned a part of family '" + part->family() + "'");
+  if (part->built_kind.empty()) {
+    part->built_kind = spec.kind;
+    part->built_from = spec.params;
+  }
+  return part;
 }
 
 // ------------------------------------------------------------------------------- built-in parts
@@ -216,8 +231,12 @@ class RMSNorm final : public NormPart {
 // precision (rounded to float only at the end): a 32-bit angle pos * inv_freq[k] is pos * 2^-23 off, 6e-4
 // five thousand tokens in, and differently at every position, so that not only distances would count.
 // Positions beyond the table (none that an engine serves) have the angle and its sine and cosine in
-// 32-bit on the device, as /root/reference/src/cuda/rope.cu:20-22 has them everywhere.  Parts with the
-// same head size and base share one table.
+// 32-bit on the device, as /root/reference/src/cuda/rope.cu:20-22 has them everywhere.
+//
+// A table never changes and is never freed while anything may read it: captured graphs hold its
+// address in their kernel arguments.  Parts with the same head size and base share the longest table
+// made so far; an engine that needs a longer one makes a new table, and every part keeps each table
+// it has ever handed out until the part itself goes (its model outlives the engines on it).
 struct RopeTable {
   int head_dim = 0;
   double theta = 0;
@@ -236,72 +255,74 @@ class RotaryNeox final : public PositionPart {
     if (head_dim % 2) throw ConfigError("rotary: head_dim " + std::to_string(head_dim) + " must be even");
   }
   const char* kind_name() const override { return "rope_neox"; }
-  void ensure_inv_freq(Ops& ops) {
-    if (shared) return;
+  // the table this part reads now (null before the first use)
+  std::shared_ptr<RopeTable> current() const {
     std::lock_guard<std::mutex> lock(g_rope_mutex);
+    return kept.empty() ? nullptr : kept.back();
+  }
+  // a table of at least `len` positions (0: the frequencies alone will do)
+  std::shared_ptr<RopeTable> table_for(int len) {
+    std::lock_guard<std::mutex> lock(g_rope_mutex);
+    if (!kept.empty() && kept.back()->table_len >= len) return kept.back();
     auto& slot = rope_tables()[{head_dim, theta}];
-    shared = slot.lock();
-    if (!shared) {
-      shared = std::make_shared<RopeTable>();
-      shared->head_dim = head_dim;
-      shared->theta = theta;
+    std::shared_ptr<RopeTable> t = slot.lock();
+    if (!t || t->table_len < len) {
+      t = std::make_shared<RopeTable>();
+      t->head_dim = head_dim;
+      t->theta = theta;
       const int half = head_dim / 2;
-      std::vector<float> host(half);
-      for (int k = 0; k < half; ++k) host[k] = (float)std::pow(theta, -2.0 * k / head_dim);
-      shared->inv_freq = DeviceBuffer((size_t)half * 4);
-      upload(shared->inv_freq.data(), host.data(), (size_t)half * 4);
-      slot = shared;
-    }
-  }
-  void prepare(Ops& ops, int max_seq) override {
-    ensure_inv_freq(ops);
-    std::lock_guard<std::mutex> lock(g_rope_mutex);
-    if (shared->table_len >= max_seq) return;
-    const int half = head_dim / 2;
-    DeviceBuffer fresh((size_t)max_seq * half * 2 * 4);
-    std::vector<double> inv(half);
-    for (int k = 0; k < half; ++k) inv[k] = std::pow(theta, -2.0 * k / head_dim);
-    std::vector<float> host((size_t)max_seq * half * 2);
-    for (int p = 0; p < max_seq; ++p)
+      std::vector<double> inv(half);
+      std::vector<float> inv32(half);
       for (int k = 0; k < half; ++k) {
-        const double angle = (double)p * inv[k];
-        host[((size_t)p * half + k) * 2] = (float)std::cos(angle);
-        host[((size_t)p * half + k) * 2 + 1] = (float)std::sin(angle);
+        inv[k] = std::pow(theta, -2.0 * k / head_dim);
+        inv32[k] = (float)inv[k];
       }
-    synchronize_device();          // the old table may still be read by a step in flight
-    upload(fresh.data(), host.data(), host.size() * 4);
-    shared->table = std::move(fresh);
-    shared->table_len = max_seq;
+      t->inv_freq = DeviceBuffer((size_t)half * 4);
+      upload(t->inv_freq.data(), inv32.data(), (size_t)half * 4);
+      if (len > 0) {
+        std::vector<float> host((size_t)len * half * 2);
+        for (int p = 0; p < len; ++p)
+          for (int k = 0; k < half; ++k) {
+            const double angle = (double)p * inv[k];
+            host[((size_t)p * half + k) * 2] = (float)std::cos(angle);
+            host[((size_t)p * half + k) * 2 + 1] = (float)std::sin(angle);
+          }
+        t->table = DeviceBuffer(host.size() * 4);
+        upload(t->table.data(), host.data(), host.size() * 4);
+        t->table_len = len;
+      }
+      slot = t;
+    }
+    kept.push_back(t);
+    return t;
   }
+  void prepare(Ops&, int max_seq) override { table_for(max_seq); }
   bool fused(Ops::Rotation& rot) const override {
-    if (!shared) return false;
-    rot.inv_freq = (const float*)shared->inv_freq.data();
-    rot.table = (const float*)shared->table.data();
-    rot.table_len = shared->table_len;
+    const std::shared_ptr<RopeTable> t = current();
+    if (!t) return false;
+    rot.inv_freq = (const float*)t->inv_freq.data();
+    rot.table = (const float*)t->table.data();
+    rot.table_len = t->table_len;
     return true;
   }
   void apply(StepContext& ctx, const Tensor& q, const Tensor& k) override {
-    ensure_inv_freq(ctx.ops);
-    const Tensor inv(shared->inv_freq.data(), DType::F32, {head_dim / 2});
+    const Tensor inv = inv_freq_tensor(ctx.ops);
     ctx.ops.rope_neox(q, ctx.positions, inv);
     if (k.defined()) ctx.ops.rope_neox(k, ctx.positions, inv);
   }
-  Tensor inv_freq_tensor(Ops& ops) {
-    ensure_inv_freq(ops);
-    return Tensor(shared->inv_freq.data(), DType::F32, {head_dim / 2});
-  }
+  Tensor inv_freq_tensor(Ops&) { return Tensor(table_for(0)->inv_freq.data(), DType::F32, {head_dim / 2}); }
   std::vector<std::pair<std::string, Tensor>> held() const override {
-    if (!shared) return {};
+    const std::shared_ptr<RopeTable> t = current();
+    if (!t) return {};
     const int half = head_dim / 2;
-    std::vector<std::pair<std::string, Tensor>> h = {{"inv_freq", Tensor(shared->inv_freq.data(), DType::F32, {half})}};
-    if (shared->table_len) h.emplace_back("table", Tensor(shared->table.data(), DType::F32, {shared->table_len, half, 2}));
+    std::vector<std::pair<std::string, Tensor>> h = {{"inv_freq", Tensor(t->inv_freq.data(), DType::F32, {half})}};
+    if (t->table_len) h.emplace_back("table", Tensor(t->table.data(), DType::F32, {t->table_len, half, 2}));
     return h;
   }
   static void upload(void* dst, const void* src, size_t bytes);
-  static void synchronize_device();
   int head_dim;
   double theta;
-  std::shared_ptr<RopeTable> shared;
+  std::vector<std::shared_ptr<RopeTable>> kept;     // oldest first; the last one is read
 };
 
 class SwiGLU final : public FeedForwardPart {
@@ -348,6 +369,10 @@ class Attention final : public MixerPart {
     head_dim = (int)param_int(p, "head_dim");
     if (heads <= 0 || kv_heads <= 0 || heads % kv_heads)
       throw ConfigError("attention: heads " + std::to_string(heads) + " not a multiple of kv_heads " + std::to_string(kv_heads));
+    // every attention kernel's range (float32 and bfloat16 alike): refused when the part is built, not at its first step
+    if (head_dim < 16 || head_dim % 16 || head_dim > 256)
+      throw ConfigError("attention: head_dim " + std::to_string(head_dim) +
+                        " is not served: the attention kernels take head sizes in steps of 16 up to 256");
     qk_norm = p.has("qk_norm") ? p.at("qk_norm").as_bool() : true;
     eps = (float)(p.has("eps") ? p.at("eps").as_double() : 1e-6);
     window = p.has("window") ? (int)p.at("window").as_int() : 0;
@@ -364,6 +389,10 @@ class Attention final : public MixerPart {
   bool reads_through_ops() const override { return true; }
   std::vector<std::shared_ptr<Part>> children() const override {
     if (pos) return {pos};
+    return {};
+  }
+  std::vector<std::string> child_slots() const override {
+    if (pos) return {"pos"};
     return {};
   }
   std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
@@ -575,6 +604,7 @@ class PreNormBlock final : public BlockPart {
   const char* kind_name() const override { return "pre_norm"; }
   bool reads_through_ops() const override { return true; }
   std::vector<std::shared_ptr<Part>> children() const override { return {norm1, mixer, norm2, ffn}; }
+  std::vector<std::string> child_slots() const override { return {"norm1", "mixer", "norm2", "ffn"}; }
   void forward(StepContext& ctx, const Tensor& x) override {
     if (!norm1->reads_through_ops()) ctx.ops.flush();
     Rows h = norm1->forward(ctx, x, nullptr, 0, mixer->takes_lazy_norm() && norm1->can_be_lazy());
@@ -677,8 +707,12 @@ template <class Base> class Foreign : public Base {
   Foreign(uint64_t id, const std::string& prefix, const Json& description, const PartChildren& c)
       : Base(prefix), info(read_description(description)) {
     this->foreign_id = id;
-    for (const auto& kv : c) kids.push_back(kv.second);
+    for (const auto& kv : c) {
+      kids.push_back(kv.second);
+      slots.push_back(kv.first);
+    }
   }
+  std::vector<std::string> child_slots() const override { return slots; }
   const char* kind_name() const override { return "foreign"; }
   std::vector<std::pair<std::string, TensorNeed>> tensors() const override { return info.tensors; }
   std::vector<std::shared_ptr<Part>> children() const override { return kids; }
@@ -700,6 +734,7 @@ template <class Base> class Foreign : public Base {
   }
   ForeignInfo info;
   std::vector<std::shared_ptr<Part>> kids;
+  std::vector<std::string> slots;
 };
 
 class ForeignEmbedding final : public Foreign<EmbeddingPart> {
@@ -759,6 +794,11 @@ class ForeignHead final : public Foreign<HeadPart> {
 
 void set_foreign_calls(const ForeignCalls& calls) { g_foreign = calls; }
 void set_foreign_error(const std::string& message) { g_foreign_error = message; }
+std::string take_foreign_error() {
+  std::string m;
+  m.swap(g_foreign_error);
+  return m;
+}
 
 std::shared_ptr<Part> make_foreign_part(const std::string& family, uint64_t id, const std::string& prefix,
                                         const Json& description, const PartChildren& children) {
@@ -782,6 +822,5 @@ namespace {
 void RotaryNeox::upload(void* dst, const void* src, size_t bytes) {
   if (hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice) != hipSuccess) throw KernelError("rotary: copying the inverse frequencies failed");
 }
-void RotaryNeox::synchronize_device() { (void)hipDeviceSynchronize(); }
 }  // namespace
 }  // namespace tinyinfer

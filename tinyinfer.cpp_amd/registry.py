@@ -52,12 +52,33 @@ def config_and_spec(config_dict: Mapping[str, Any]):
             read_config, build_spec = _ARCHITECTURES[c]
             cfg = read_config(config_dict)
             return cfg, build_spec(cfg)
-    # the library's own table; its error lists the names
+    # the library's table (its own architecture and whatever plugins registered); its error lists the names
     text = json.dumps(dict(config_dict)).encode()
     try:
         spec = ModelSpec.from_dict(json.loads(native.text("ti_spec_from_config", text)))
+        typed = json.loads(native.text("ti_typed_config", text))
     except ConfigError as e:
         if "registered:" in str(e) and _ARCHITECTURES:
             raise ConfigError(str(e).split("registered:")[0] + f"registered: {registered_architectures()}") from None
         raise
-    return Qwen3Config.from_dict(config_dict), spec
+    # the architecture's own typed configuration: a class of this package where there is one, else the
+    # validated keys as the library wrote them back
+    reader = _TYPED_CONFIGS.get(typed["architecture"], TypedConfig)
+    return reader(typed["config"]), spec
+
+
+class TypedConfig(dict):
+    """The typed configuration of an architecture that has no class of its own here: its validated
+    config.json keys, each also an attribute."""
+
+    def __getattr__(self, name):
+        try:
+            return self[name]
+        except KeyError:
+            raise AttributeError(name) from None
+
+    def to_dict(self) -> dict:
+        return dict(self)
+
+
+_TYPED_CONFIGS = {"Qwen3ForCausalLM": Qwen3Config.from_normalized, "qwen3": Qwen3Config.from_normalized}

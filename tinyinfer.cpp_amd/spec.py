@@ -69,6 +69,15 @@ class ModelSpec:
     def run_order(self) -> List[int]:
         return list(range(len(self.layers))) if self.schedule is None else list(self.schedule)
 
+    def to_dict(self) -> dict:
+        return {"architecture": self.architecture, "vocab_size": self.vocab_size, "hidden_size": self.hidden_size,
+                "embedding": self.embedding.to_dict(),
+                "layers": [{"prefix": l.prefix, "block": l.block.to_dict(), "parts": {k: v.to_dict() for k, v in l.parts.items()},
+                            "cache_from": l.cache_from} for l in self.layers],
+                "final_norm": self.final_norm.to_dict(), "lm_head": self.lm_head.to_dict(),
+                "schedule": None if self.schedule is None else list(self.schedule),
+                "eos_token_ids": list(self.eos_token_ids), "max_position_embeddings": self.max_position_embeddings}
+
     @classmethod
     def from_dict(cls, d) -> "ModelSpec":
         layers = [LayerSpec(l["prefix"], PartSpec.from_dict(l["block"]),

@@ -493,11 +493,14 @@ void host_random(const TensorNeed& need, uint64_t seed, DType dt, void* out) {
         ((int32_t*)out)[i] = a + (int)((z >> 11) % (uint64_t)(b > a ? b - a : 1));
         continue;
       }
-      const float u1 = ((float)((z >> 40) & 0xffffffu) + 1.0f) * (1.0f / 16777216.0f);
-      const float u2 = (float)((z >> 16) & 0xffffffu) * (1.0f / 16777216.0f);
+      // in double precision, rounded to 32-bit once at the end, with the parameters as the device gets them
+      // (32-bit): the same bits as csrc/core.hip's fill_random_kernel draws
+      const double u1 = ((double)((z >> 40) & 0xffffffu) + 1.0) * (1.0 / 16777216.0);
+      const double u2 = (double)((z >> 16) & 0xffffffu) * (1.0 / 16777216.0);
+      const double a = (double)(float)need.a, b = (double)(float)need.b;
       float v;
-      if (kind == 0) v = (float)need.a + (float)need.b * (std::sqrt(-2.0f * std::log(u1)) * std::cos(6.28318530717958647692f * u2));
-      else if (kind == 1) v = (float)need.a + (float)(need.b - need.a) * u2;
+      if (kind == 0) v = (float)(a + b * (std::sqrt(-2.0 * std::log(u1)) * std::cos(6.28318530717958647692 * u2)));
+      else if (kind == 1) v = (float)(a + (b - a) * u2);
       else v = (float)need.a;
       if (dt == DType::BF16) ((uint16_t*)out)[i] = f32_to_bf16(v);
       else ((float*)out)[i] = v;
