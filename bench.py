@@ -129,6 +129,60 @@ def measured_peaks():
     return read, mfma
 
 
+def decode_floor(engine, rids, last, nums, context, batch):
+    """ms of a captured graph of kernels that only read memory, one for every call of a decode step in the step's own
+    order, each reading as many bytes as that call has to (a product its weight, an attention the keys and values of
+    the batch in one cache layer; everything else next to nothing): what a chain of so many dependent kernels over so
+    many bytes takes on this GPU whatever the kernels compute.  The calls are the engine's own list for this step."""
+    import re
+    import torch
+    from tinyinfer_amd import native
+    from tinyinfer_amd.csrc import build
+    from tinyinfer_amd.engine import StepEntry
+    engine.ops.count_calls(True)
+    engine.step([StepEntry(r, [t], (0,)) for r, t in zip(rids, last)])
+    calls = engine.ops.timing_report()
+    engine.ops.count_calls(False)
+    layers = sum(n for need, n in engine.model.cache_groups if hasattr(need, "kv_heads"))
+    kv_layer = nums["kv_bytes"](context) * batch // max(1, layers)
+    sizes = []
+    for c in calls:
+        m = re.search(r"\* (\d+)x(\d+)", c["name"])
+        per_call = int(m.group(1)) * int(m.group(2)) * 2 if m else kv_layer if c["name"].startswith("attention") else 4096
+        sizes += [per_call] * c["calls"]
+        if c["name"].startswith("attention") and "runs" in c["name"]:
+            sizes += [4096] * c["calls"]              # the kernel that merges the runs of a context
+    native.ensure_kernels(["measure"])
+    lib = ctypes.CDLL(build.find("measure"))
+    lib.ti_measure_read.argtypes = [ctypes.c_void_p, ctypes.c_long, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+    total = sum(-(-b // 256) * 256 for b in sizes)
+    buf = torch.empty(total + (1 << 20), dtype=torch.uint8, device="cuda")
+    buf.fill_(1)
+    sink = torch.zeros(1 << 16, dtype=torch.int32, device="cuda")
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            off = 0
+            for b in sizes:
+                b = -(-b // 256) * 256
+                blocks = int(min(units * 8, max(1, b // 16384)))
+                assert lib.ti_measure_read(buf.data_ptr() + off, b, sink.data_ptr(), blocks, stream.cuda_stream) == 0
+                off += b
+    best = None
+    for _ in range(6):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        graph.replay()
+        b.record(stream)
+        b.synchronize()
+        best = a.elapsed_time(b) if best is None else min(best, a.elapsed_time(b))
+    del graph, buf
+    torch.cuda.empty_cache()
+    return best, len(sizes)
+
+
 def fill(engine, rids, context, rng, chunk=4096):
     """Give each request `context` cached tokens by real prefill steps."""
     import torch
@@ -143,7 +197,7 @@ def fill(engine, rids, context, rng, chunk=4096):
     torch.cuda.synchronize()
 
 
-def measure_decode(engine, sampler, batch, steps, warmup, context, rng, tag, kernel_times=False, draw=None):
+def measure_decode(engine, sampler, batch, steps, warmup, context, rng, tag, kernel_times=False, draw=None, floor=None):
     """tokens/s and ms/step of `steps` decode steps at `batch`, every request at `context` tokens.
     draw: (temperature, top_k, top_p) for the sampler, or None for the greedy choice."""
     import torch
@@ -185,6 +239,9 @@ def measure_decode(engine, sampler, batch, steps, warmup, context, rng, tag, ker
     last = sampler.collect(ticket)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    if floor is not None:
+        floor["ms"], floor["kernels"] = decode_floor(engine, rids, last, floor["nums"], context + warmup + steps, batch)
+        last = one_step(last)
     table = None
     if kernel_times:
         one_step(last, graph=False)
@@ -314,7 +371,7 @@ def main() -> int:
                                     "decoded": args.batch, "portion": args.portion, "cached": args.cached,
                                     "decode_context": context, "model": NAMES[args.model]}}), flush=True)
         return 0
-    p_s = tps = ms = None
+    p_s = tps = ms = floor = None
     draw = (args.temperature, args.top_k, args.top_p) if args.temperature > 0 else None
     if args.only != "decode":
         say(f"prefill of {prefill_tokens} tokens ...")
@@ -327,8 +384,9 @@ def main() -> int:
             print_table(table, f"a prefill step of {prefill_tokens} tokens, call by call:")
     if args.only != "prefill":
         say(f"decode at batch {args.batch} ...")
+        floor = None if args.no_peaks else {"nums": nums}
         tps, ms, table = measure_decode(engine, sampler, args.batch, args.steps, args.warmup, context, rng, "m",
-                                        args.kernel_times, draw)
+                                        args.kernel_times, draw, floor)
         if table:
             print_table(table, f"a decode step at batch {args.batch}, call by call (not from the graph):")
     points = {}
@@ -347,6 +405,10 @@ def main() -> int:
                     "frac": round(achieved / PEAK_HBM, 4)}
         if peaks:
             roofline.update(measured_read=round(peaks[0] / 1e9, 1), frac_of_measured=round(achieved / peaks[0], 4))
+        if floor and floor.get("ms"):
+            # a graph of as many kernels that only read as many bytes, in the step's order: the structure's own floor
+            roofline.update(read_only_chain_ms=round(floor["ms"], 4), chain_kernels=floor["kernels"],
+                            frac_of_read_only_chain=round(floor["ms"] / ms, 4))
     if p_s is not None:
         flops = prefill_flops(engine.model, prefill_tokens)
         prefill = {"value": round(prefill_tokens / p_s, 1), "tokens": prefill_tokens, "ms": round(p_s * 1e3, 3),

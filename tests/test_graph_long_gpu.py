@@ -67,7 +67,7 @@ def test_decode_graph_captured_for_long_sequences(model_folders, name, dtype):
     Every row is the plain model's; the same steps through `step` give the same bits in 32-bit and the same
     values within the bound in bfloat16 (the graph cuts the contexts into other runs than the eager step)."""
     import tinyinfer_amd as ti
-    from tinyinfer_amd.ops import attention_bf16
+    from tinyinfer_amd.ops import kernels as attention_bf16
     cfg = CONFIGS[name]
     folder = model_folders(name, "bfloat16", True)
     V = cfg["vocab_size"]

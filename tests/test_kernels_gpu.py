@@ -12,6 +12,14 @@ pytestmark = pytest.mark.gpu
 DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
 
+def run_attention(ops, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window):
+    """The step's rows through `Ops.attention`; whether the matrix-core kernels serve these sizes (else the rows
+    went through the generic kernel)."""
+    from tinyinfer_amd.ops import kernels
+    ops.attention(ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window)
+    return head_dim in kernels.SERVED_HEAD_DIMS and pool.shape[3] % 16 == 0
+
+
 @pytest.fixture(scope="module")
 def ops():
     import tinyinfer_amd  # noqa: F401
@@ -611,7 +619,7 @@ def test_linear_bf16_weight_row_per_wavefront(ops, M, N, K):
     results = {}
     try:
         for on in (1, 0):
-            lib.ti_gemm_bf16_row_per_wave(on)
+            lib.ti_tuning_set(b"row_per_wave", on)
             out = torch.full((M + 1, N), 7.0, device="cuda")     # a row beyond: must stay untouched
             ops.linear(a, w, out[:M], "store")
             assert (f64(out[:M]) - ref).abs().max() < tol
@@ -621,7 +629,7 @@ def test_linear_bf16_weight_row_per_wavefront(ops, M, N, K):
             assert (f64(acc) - (ref + f64(base))).abs().max() < tol
             results[on] = (out[:M].clone(), acc)
     finally:
-        lib.ti_gemm_bf16_row_per_wave(1)
+        lib.ti_tuning_set(b"row_per_wave", 1)
     assert (results[1][0] - results[0][0]).abs().max() < tol
     # a row's bits do not depend on the rows beside it
     if M > 1:
@@ -714,18 +722,18 @@ def test_linear_bf16_token_rows_in_pieces(ops, M, N, K, ks):
     run(a[M - 1:M], one, 0)
     assert torch.equal(one[0], out[M - 1])
     # the kernels that hold all of K at once: the same order of summation
-    lib.ti_gemm_bf16_pieces_on(0)
-    lib.ti_gemm_bf16_row_per_wave(0)
-    lib.ti_gemm_bf16_skinny_waves(4)
+    lib.ti_tuning_set(b"pieces", 0)
+    lib.ti_tuning_set(b"row_per_wave", 0)
+    lib.ti_tuning_set(b"skinny_waves", 4)
     try:
         old = torch.empty(M, N, device="cuda")
         rc = lib.ti_gemm_bf16(ptr(a), ptr(w), ptr(old), M, N, K, ctypes.c_long(a.stride(0)), 0, None)
         assert rc == 0, lib.ti_last_error()
         assert torch.equal(old, out[:M])
     finally:
-        lib.ti_gemm_bf16_pieces_on(1)
-        lib.ti_gemm_bf16_row_per_wave(1)
-        lib.ti_gemm_bf16_skinny_waves(0)
+        lib.ti_tuning_set(b"pieces", 1)
+        lib.ti_tuning_set(b"row_per_wave", 1)
+        lib.ti_tuning_set(b"skinny_waves", 0)
     base = torch.randn(M, N, generator=g)
     for splits in split_counts:
         acc = dev(base.clone())
@@ -808,7 +816,7 @@ def test_linear_bf16_large_weight_at_17_to_64_rows(ops, M, epilogue):
     outs = []
     try:
         for rule in (280 << 20, 1 << 60, 0):              # as shipped, never, always
-            lib.ti_gemm_bf16_tiled_from(rule)
+            lib.ti_tuning_set(b"tiled_from", rule)
             if epilogue == "swiglu":
                 out = torch.empty(M, N // 2, device="cuda", dtype=torch.bfloat16)
             elif epilogue == "store_act":
@@ -820,7 +828,7 @@ def test_linear_bf16_large_weight_at_17_to_64_rows(ops, M, epilogue):
             assert (f64(out) - want).abs().max() < bound
             outs.append(f64(out))
     finally:
-        lib.ti_gemm_bf16_tiled_from(280 << 20)
+        lib.ti_tuning_set(b"tiled_from", 280 << 20)
     assert (outs[1] - outs[2]).abs().max() < 2 * bound
     # 17 rows x 16 Mi lie under the rule, 33 and 64 over it
     same_as = outs[1] if M == 17 else outs[2]
@@ -848,14 +856,14 @@ def test_linear_bf16_large_weight_at_13_to_16_rows(ops):
         outs = []
         try:
             for rule in (280 << 20, 1 << 60):
-                lib.ti_gemm_bf16_tiled_from(rule)
+                lib.ti_tuning_set(b"tiled_from", rule)
                 h = torch.empty(M, K, device="cuda", dtype=torch.bfloat16)
                 out = torch.empty(M, N, device="cuda")
                 ops.linear(NormedRows(x, nw, 1e-6, h), w, out, "store")
                 assert (f64(out) - ref).abs().max() < 0.01 * ref.abs().max() + 2e-5 * K
                 outs.append(out)
         finally:
-            lib.ti_gemm_bf16_tiled_from(280 << 20)
+            lib.ti_tuning_set(b"tiled_from", 280 << 20)
         assert torch.equal(outs[0], outs[1]) == (M == 12), M
 
 
@@ -879,14 +887,14 @@ def test_linear_bf16_wide_weight_at_17_to_64_rows(ops, M, N, K):
     outs = {}
     try:
         for on in (1, 0):
-            lib.ti_gemm_bf16_wide_rows_on(on)
+            lib.ti_tuning_set(b"wide_rows", on)
             out = torch.full((M + 1, N), 7.0, device="cuda")
             ops.linear(a, w, out[:M], "store")
             assert (f64(out[:M]) - ref).abs().max() < tol
             assert bool((out[M] == 7.0).all())
             outs[on] = out[:M].clone()
     finally:
-        lib.ti_gemm_bf16_wide_rows_on(1)
+        lib.ti_tuning_set(b"wide_rows", 1)
     assert (outs[1] - outs[0]).abs().max() < tol
     fewer = torch.empty(17, N, device="cuda")
     ops.linear(a[M - 17:], w, fewer, "store")
@@ -994,7 +1002,7 @@ def test_linear_bf16_every_tile(ops, tile, M, N, K):
     w = (torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16)
     ref = ref_linear(a, w)
     tol = 2e-5 * K
-    lib.ti_gemm_bf16_force_tile(tile)
+    ops.tune("gemm_bf16", "force_tile", tile)        # this object's own override: set around each of its calls
     try:
         out = torch.empty(M, N, device="cuda")
         ops.linear(dev(a), dev(w), out, "store")
@@ -1012,8 +1020,11 @@ def test_linear_bf16_every_tile(ops, tile, M, N, K):
         gte, up = ref[:, :F], ref[:, F:]
         want = gte / (1 + torch.exp(-gte)) * up
         assert (f64(out) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
+        with pytest.raises(Exception, match="no shape rule"):
+            ops.tune("gemm_bf16", "no_such_rule", 1)
+            ops.linear(dev(a), dev(w), torch.empty(M, N, device="cuda"), "store")
     finally:
-        lib.ti_gemm_bf16_force_tile(0)
+        ops.tune()
 
 
 @pytest.mark.parametrize("M,N,K", [(2000, 5130, 192), (2048, 5120, 64), (1100, 9000, 128)])
@@ -1034,7 +1045,7 @@ def test_columns_split_between_two_tile_shapes(ops, M, N, K):
     ref = ref_linear(a, w)
     got = {}
     for split in (1, 0):
-        lib.ti_gemm_bf16_two_ranges(split)
+        lib.ti_tuning_set(b"two_ranges", split)
         try:
             out = torch.empty(M, N, device="cuda")
             ops.linear(dev(a), dev(w), out, "store")
@@ -1046,7 +1057,7 @@ def test_columns_split_between_two_tile_shapes(ops, M, N, K):
             ops.linear(dev(a), dev(w), paired, "swiglu")
             got[split] = (out, added, act, paired)
         finally:
-            lib.ti_gemm_bf16_two_ranges(1)
+            lib.ti_tuning_set(b"two_ranges", 1)
     for x, y in zip(got[1], got[0]):
         assert torch.equal(x, y)
     tol = 2e-5 * K
@@ -1074,7 +1085,7 @@ def test_widths_that_160_divides_take_tiles_of_160_columns(ops, M, N, K):
     ref = ref_linear(a, w)
     got = {}
     for on in (1, 0):
-        lib.ti_gemm_bf16_tiles_160(on)
+        lib.ti_tuning_set(b"tiles_160", on)
         try:
             out = torch.empty(M, N, device="cuda")
             ops.linear(dev(a), dev(w), out, "store")
@@ -1084,7 +1095,7 @@ def test_widths_that_160_divides_take_tiles_of_160_columns(ops, M, N, K):
             ops.linear(dev(a), dev(w), act, "store_act")
             got[on] = (out, added, act)
         finally:
-            lib.ti_gemm_bf16_tiles_160(1)
+            lib.ti_tuning_set(b"tiles_160", 1)
     for x, y in zip(got[1], got[0]):
         assert torch.equal(x, y)
     tol = 2e-5 * K
@@ -1109,13 +1120,13 @@ def test_swiglu_of_up_to_64_rows_under_a_wide_weight(ops, M):
     outs = []
     try:
         for tile in (0, 3):
-            lib.ti_gemm_bf16_force_tile(tile)
+            lib.ti_tuning_set(b"force_tile", tile)
             out = torch.empty(M, F, device="cuda", dtype=torch.bfloat16)
             ops.linear(a, w, out, "swiglu")
             assert (f64(out) - want).abs().max() < 0.005 * want.abs().max() + 2e-4 * K
             outs.append(out)
     finally:
-        lib.ti_gemm_bf16_force_tile(0)
+        lib.ti_tuning_set(b"force_tile", 0)
     assert torch.equal(outs[0], outs[1])
 
 
@@ -1303,7 +1314,7 @@ class FakeCtx:
 def fast_attention_case(ops, entries_tokens, nh, nkv, hd, P, window, seed, sharp=2.0):
     """Several requests with full contexts in a scattered pool; the step holds the
     last `n` tokens of each.  Returns (got, want) for the step's rows."""
-    from tinyinfer_amd.ops import attention_bf16
+    from tinyinfer_amd.ops import kernels as attention_bf16
     g = torch.Generator().manual_seed(seed)
     lens = [s + n for n, s in entries_tokens]
     n_pages_each = [-(-L // P) for L in lens]
@@ -1335,7 +1346,7 @@ def fast_attention_case(ops, entries_tokens, nh, nkv, hd, P, window, seed, sharp
     qd = dev(torch.cat(qs).reshape(-1, nh * hd))
     out = torch.zeros_like(qd)
     ctx = FakeCtx(entries_tokens)
-    ok = attention_bf16.run(ops, ctx, View(dev(table)), qd, dev(pool), out, nh, nkv, hd, 1.0 / math.sqrt(hd), window)
+    ok = run_attention(ops, ctx, View(dev(table)), qd, dev(pool), out, nh, nkv, hd, 1.0 / math.sqrt(hd), window)
     assert ok
     return f64(out), torch.cat(refs).reshape(-1, nh * hd)
 
@@ -1367,13 +1378,13 @@ def test_attention_bf16_portions_and_mixed(ops, nh, nkv, hd, P, window, variant)
     entries = [(2, 0), (7, 30), (1, 99), (16, 16), (17, 15), (64, 0), (65, 63), (130, 41), (1, 0), (3, 300), (200, 5),
                (333, 700)]
     lib = ops.lib("attention_bf16")
-    lib.ti_attention_prefill_groups({"one group": 1, "two groups": 2}.get(variant, 0))
+    lib.ti_tuning_set(b"prefill_groups", {"one group": 1, "two groups": 2}.get(variant, 0))
     ops.use_paired_prefill = variant in ("paired", "a tile each")
     ops.force_paired_tiles = variant == "paired"
     try:
         got, want = fast_attention_case(ops, entries, nh, nkv, hd, P, window, seed=nh * 10 + hd)
     finally:
-        lib.ti_attention_prefill_groups(0)
+        lib.ti_tuning_set(b"prefill_groups", 0)
         ops.use_paired_prefill = True
         ops.force_paired_tiles = None
     assert torch.isfinite(got).all()
@@ -1388,7 +1399,7 @@ def test_attention_bf16_far_into_long_contexts(ops):
     stand out for the last query of head 0, so that a page dropped far back would show."""
     if not ops.use_fast_attention:
         pytest.skip("bfloat16 attention kernels are switched off")
-    from tinyinfer_amd.ops import attention_bf16
+    from tinyinfer_amd.ops import kernels as attention_bf16
     nh, nkv, hd, P = 4, 2, 128, 16
     entries = [(1, 20000), (300, 20000), (1, 32767), (70, 9000), (1, 5)]
     g = torch.Generator().manual_seed(21)
@@ -1431,7 +1442,7 @@ def test_attention_bf16_far_into_long_contexts(ops):
     qd = dev(torch.cat(qs).reshape(-1, nh * hd))
     out = torch.zeros_like(qd)
     ctx = FakeCtx(entries)
-    assert attention_bf16.run(ops, ctx, View(dev(table)), qd, dev(pool), out, nh, nkv, hd, scale, None)
+    assert run_attention(ops, ctx, View(dev(table)), qd, dev(pool), out, nh, nkv, hd, scale, None)
     got, want = f64(out), torch.cat(refs).reshape(-1, nh * hd)
     assert torch.isfinite(got).all()
     assert (got - want).abs().max() < 2e-2
@@ -1466,7 +1477,7 @@ def test_attention_bf16_short_portions_against_a_long_context(ops, nh, nkv, hd, 
     and against the same launch with one run."""
     if not ops.use_fast_attention:
         pytest.skip("bfloat16 attention kernels are switched off")
-    from tinyinfer_amd.ops import attention_bf16
+    from tinyinfer_amd.ops import kernels as attention_bf16
     entries = [(70, 3000), (40, 0), (1, 2500), (130, 1000)]
     ctx = FakeCtx(entries)
     assert attention_bf16.portion_launch(ctx, nh, int(window or 0))[0] >= 3
@@ -1630,11 +1641,11 @@ def qkv_prepared_case(ops, tile_rows, M, nh, nkv, hd, K, P, norm, rope):
     ops.qk_norm_rope_kv_write(qkv, q_w, k_w, 1e-5, inv_freq, pos, slot, view, pool_a, q_a, nh, nkv, hd, tab)
     q_b = torch.zeros_like(q_a)
     lib = ops.lib("gemm_bf16")
-    lib.ti_gemm_bf16_qkv_prep_rows(tile_rows)
+    lib.ti_tuning_set(b"qkv_prep_rows", tile_rows)
     try:
         assert ops.qkv_prepared(a, w, q_w, k_w, 1e-5, inv_freq, tab, pos, slot, view, pool_b, q_b, nh, nkv, hd)
     finally:
-        lib.ti_gemm_bf16_qkv_prep_rows(0)
+        lib.ti_tuning_set(b"qkv_prep_rows", 0)
     if M > 64:
         assert torch.equal(q_a.view(torch.int16), q_b.view(torch.int16))
         assert torch.equal(pool_a.view(torch.int16), pool_b.view(torch.int16))
@@ -1654,7 +1665,7 @@ def test_attention_bf16_far_key(ops):
     """One key far back carries the weight, for a decode row and for a row inside a portion."""
     if not ops.use_fast_attention:
         pytest.skip("bfloat16 attention kernels are switched off")
-    from tinyinfer_amd.ops import attention_bf16
+    from tinyinfer_amd.ops import kernels as attention_bf16
     T, hd, P = 1000, 64, 16
     g = torch.Generator().manual_seed(21)
     k = (torch.randn(T, 1, hd, generator=g) * 0.1).to(torch.bfloat16)
@@ -1675,5 +1686,5 @@ def test_attention_bf16_far_key(ops):
         q[-1, 3] = 30.0
         out = torch.zeros(n, hd, dtype=torch.bfloat16, device="cuda")
         ctx = FakeCtx(entries)
-        assert attention_bf16.run(ops, ctx, View(dev(table)), dev(q), dev(pool), out, 1, 1, hd, 1.0 / 8, None)
+        assert run_attention(ops, ctx, View(dev(table)), dev(q), dev(pool), out, 1, 1, hd, 1.0 / 8, None)
         assert (f64(out[-1]) - f64(v[far, 0])).abs().max() < 2e-2

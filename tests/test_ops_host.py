@@ -40,7 +40,8 @@ def test_declarations_are_read_as_written():
     restype, args = sig["ti_gemm_bf16"]
     assert args[6] is ctypes.c_long and args[-1] is ctypes.c_void_p and len(args) == 9
     with open(os.path.join(build.HERE, "tinyinfer_kernels_tuning.h")) as f:
-        assert kernels.header_signatures(f.read())["ti_gemm_bf16_force_tile"] == (None, [ctypes.c_int])
+        tuning = kernels.header_signatures(f.read())
+    assert tuning["ti_tuning_set"] == (ctypes.c_int, [ctypes.c_void_p, ctypes.c_long]) and tuning["ti_tuning_reset"] == (None, [])
     assert sig["ti_fill_random"][1][6] is ctypes.c_ulong
     # what the call sites pass for such arguments is accepted
     assert ctypes.c_void_p.from_param(None) is None
@@ -60,7 +61,7 @@ def test_context_splits_of_the_decode_kernel(monkeypatch):
     """The number of runs the decode attention cuts the context into: bounded by the context the
     launch is sized for, chosen for the typical one, and never just beyond a whole round of the
     compute units when fewer runs fill one round (12 rows x 8 kv heads: 2 runs, not 3)."""
-    from tinyinfer_amd.ops import attention_bf16 as a
+    from tinyinfer_amd.ops import kernels as a
     monkeypatch.setattr(a, "compute_units", lambda: 256)
     assert a.decode_splits(8, 8, 16, 4096, 2112) == 4          # 256 workgroups
     assert a.decode_splits(12, 8, 16, 4096, 2112) == 2         # 192, not 288

@@ -22,6 +22,7 @@
 //            together and share them in the cache.
 // (The reference scans positions with 16-lane groups and FMA for both cases:
 // /root/reference/src/cuda/attention.cu:107-198.)
+#include <string>
 #include <type_traits>
 #include "common.h"
 #include "tinyinfer_kernels.h"
@@ -1168,7 +1169,6 @@ static int compute_units() {
 }
 // 1 (default): small decode launches from the projections let one wavefront prepare the query
 static int g_decode_shared_query = 1;
-extern "C" void ti_attention_decode_shared_query(int on) { g_decode_shared_query = on; }
 
 // Decode rows.  rows: which rows of the step (nullptr: rows 0..n_rows-1).  n_splits > 1 needs
 // part_o (float [n_rows, n_head, n_splits, hd]) and part_ml (float [n_rows, n_head, n_splits, 2]).
@@ -1265,11 +1265,9 @@ extern "C" int ti_attention_decode_prepared_bf16(const float* qkv, int row_width
 }
 
 static int g_prefill_groups = 0;   // for measurements: 1 or 2 wavefront groups per workgroup, 0 = by the launch
-extern "C" void ti_attention_prefill_groups(int groups) { g_prefill_groups = groups; }
 static int g_prefill_lds = 1;
 // 1: head sizes 64 and 128 take the kernel that shares keys and values through LDS
 // (default); 0: every head size takes the kernel that reads them per wavefront
-extern "C" void ti_attention_prefill_use_lds(int on) { g_prefill_lds = on; }
 
 // Portions of prompts.  tiles: int [n_tiles, 2] = (entry, first row), each tile 128 rows;
 // entries: int [n_entries, 4] = (row0, n_tokens, start_pos, -); table row e belongs to entry e.
@@ -1388,5 +1386,23 @@ extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool,
                                                                    n_splits);
   }
   TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------- tests and measurements
+// One entry for every choice above that a test or a measurement may want to force (names as in
+// tinyinfer_kernels_tuning.h); process-wide in the library, applied and reset around its calls by the
+// host library's Ops.  Returns 0, or 1 for an unknown name.
+extern "C" void ti_tuning_reset() {
+  g_decode_shared_query = 1;
+  g_prefill_groups = 0;
+  g_prefill_lds = 1;
+}
+extern "C" int ti_tuning_set(const char* name, long value) {
+  const std::string n = name ? name : "";
+  if (n == "decode_shared_query") g_decode_shared_query = (int)value;
+  else if (n == "prefill_groups") g_prefill_groups = (int)value;
+  else if (n == "prefill_use_lds") g_prefill_lds = (int)value;
+  else return 1;
   return 0;
 }

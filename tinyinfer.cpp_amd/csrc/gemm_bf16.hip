@@ -17,6 +17,7 @@
 // /root/reference/src/cuda/gemm.cu:37-85 and 152-261; it reads the weights once
 // per row of A for M <= 32.)
 #include <algorithm>
+#include <string>
 #include "common.h"
 #include "tinyinfer_kernels.h"
 #include "tinyinfer_kernels_tuning.h"
@@ -1137,13 +1138,9 @@ static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, 
 }
 
 static int g_tiles_160 = 1;      // a hook for measurements: 0 = no tiles of 160 columns
-extern "C" void ti_gemm_bf16_tiles_160(int on) { g_tiles_160 = on; }
 static int g_two_ranges = 1;     // a hook for measurements: 0 = never split the columns between two tile shapes
-extern "C" void ti_gemm_bf16_two_ranges(int on) { g_two_ranges = on; }
 static int g_qkv_rows = 0;       // hooks for measurements: 128 or 256 forces the tile's rows;
 static int g_qkv_min_rows = 17;  // the fewest rows served (fewer take the kernels with the norm in front)
-extern "C" void ti_gemm_bf16_qkv_prep_min_rows(int rows) { g_qkv_min_rows = rows; }
-extern "C" void ti_gemm_bf16_qkv_prep_rows(int rows) { g_qkv_rows = rows; }
 
 static int compute_units() {
   static int n = 0;
@@ -1234,7 +1231,6 @@ extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K,
 // for measurements: 0 = choose the tile by the shape, 1 = 256 x 128, 3 = 128 x 64, 5 = 64 x 128 (SwiGLU only), 6 = 64 x 64,
 // 8 = 128 x 160, 9 = 256 x 160 (neither for SwiGLU)
 static int g_force_tile = 0;
-extern "C" void ti_gemm_bf16_force_tile(int which) { g_force_tile = which; }
 
 // Three tiles.  256 x 128 with eight wavefronts does the most per byte it loads, one workgroup
 // to a compute unit: it is taken when its workgroups come in (nearly) whole rounds of the 256
@@ -1311,10 +1307,8 @@ static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M,
 // has few workgroups (one per 16 columns); more wavefronts in each, splitting K further, keep
 // more loads in flight.  0 = choose by the shape.
 static int g_skinny_waves = 0;
-extern "C" void ti_gemm_bf16_skinny_waves(int waves) { g_skinny_waves = waves; }
 // 1 (default): eight chunks of K in flight per wavefront where its share of K is more than four
 static int g_skinny_deep = 1;
-extern "C" void ti_gemm_bf16_skinny_deep(int on) { g_skinny_deep = on; }
 
 template <int EPI>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
@@ -1371,7 +1365,7 @@ static int g_use_pipelined = 1;
 // the norm a kernel of its own.  (At 9 to 12 rows that was measured as well, and loses.)
 static long g_tiled_from = 280L << 20;           // 17..64 rows x weight elements from which steps take the tiled kernels
 static long g_tiled_from_16 = 600L << 20;        // the same for 13..16 rows
-extern "C" void ti_gemm_bf16_tiled_from(long rows_times_elems) {
+static void set_tiled_from(long rows_times_elems) {
   g_tiled_from = rows_times_elems;
   g_tiled_from_16 = rows_times_elems >= (280L << 20) && rows_times_elems < (1L << 59) ? rows_times_elems / 280 * 600
                                                                                      : rows_times_elems;
@@ -1387,7 +1381,6 @@ static bool large_weight(int M, int N, int K, int epi) {
 #define GR_MMAX 8
 #define GR_ROWS_BELOW 4096
 static int g_row_per_wave = 1;
-extern "C" void ti_gemm_bf16_row_per_wave(int on) { g_row_per_wave = on; }
 // Every workgroup (four weight rows) copies all M token rows into LDS: M / 4 times the bytes of its
 // weight rows.  Up to four tokens that is no more than the weight itself; beyond, the kernel is taken
 // only while its workgroups are no more than the compute units (Qwen3-0.6B's o and down, 1,024 rows: 4.7
@@ -1455,7 +1448,6 @@ static int skinny_waves_for(int grid, int K) {
 static bool pieces_serves(int M, int N, int K, int epi);
 #define NORMED_WEIGHT_BELOW (40L << 20)   // weight elements from which the norm stays a kernel of its own
 static long g_normed_weight_below = NORMED_WEIGHT_BELOW;
-extern "C" void ti_gemm_bf16_normed_weight_below(long elements) { g_normed_weight_below = elements > 0 ? elements : NORMED_WEIGHT_BELOW; }
 // out = rmsnorm(x; nw, eps) W^T for M <= 16 (see gemm_skinny_staged_kernel).  Returns 3 for
 // sizes it does not serve (M > 16, K not a multiple of 64 or above 4096).
 extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, const void* W, void* out,
@@ -1515,7 +1507,6 @@ extern "C" int ti_gemm_bf16_normed(const float* x, const float* nw, float eps, c
 // 1 (default): up to 16 tokens with K a multiple of 64 up to 4096, the token rows are copied into
 // LDS once per workgroup (see CopyProducer); 0: every wavefront fetches its fragments from memory
 static int g_skinny_copy = 1;
-extern "C" void ti_gemm_bf16_skinny_copy(int on) { g_skinny_copy = on; }
 
 template <int EPI>
 static int launch_skinny_copied(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
@@ -1749,7 +1740,6 @@ gemm_wide_rows_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
 }
 
 static int g_wide_rows = 1;      // a hook for measurements: 0: the kernel above serves nothing
-extern "C" void ti_gemm_bf16_wide_rows_on(int on) { g_wide_rows = on; }
 #define WIDE_ROWS_MIN_N 16384
 
 // whether gemm_wide_rows_kernel takes the product (storing 32-bit results)
@@ -1806,7 +1796,6 @@ static int launch_pieces(const bf16_t* a, long lda, const bf16_t* w, void* out, 
 // 1 (default): up to 16 rows times a weight whose K is a multiple of 64 and at least two pieces long
 // take the kernel with the token rows in pieces; 0: the kernels above it (for comparison)
 static int g_pieces = 1;
-extern "C" void ti_gemm_bf16_pieces_on(int on) { g_pieces = on; }
 static bool pieces_serves(int M, int N, int K, int epi) {
   if (!g_pieces || M > 16 || K % 64 != 0 || K < 2 * SP_PIECE) return false;
   if (epi < TI_EPI_STORE_F32 || epi > TI_EPI_SWIGLU) return false;
@@ -1830,7 +1819,6 @@ static int pieces_splits(int N, int K, long partial_bytes) {
 }
 
 static int g_add_split = 1;        // a hook for measurements: 0: ti_gemm_bf16_add_split serves nothing
-extern "C" void ti_gemm_bf16_add_split_on(int on) { g_add_split = on; }
 
 template <int EPI>
 static void launch_mblocks(const bf16_t* a, const bf16_t* w, void* out, float* partial, int M, int N, int K,
@@ -2057,7 +2045,6 @@ extern "C" int ti_gemm_bf16_mblocks_any(const void* A, const void* W, void* out,
   return 0;
 }
 
-extern "C" void ti_gemm_bf16_use_pipelined(int on) { g_use_pipelined = on; }
 
 // N: output columns (SwiGLU: F, with W holding 2F rows).  Returns 3 for a shape
 // these kernels do not serve (the caller takes the generic kernel then).
@@ -2125,5 +2112,36 @@ extern "C" int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int 
   }
 #undef TI_GO
   TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------- tests and measurements
+// One entry for every shape rule above that a test or a measurement may want to force: `name` as in
+// tinyinfer_kernels_tuning.h, value 0 (or what the table says) restores the rule's own choice.
+// The rules are the library's, process-wide; the host library's Ops applies an object's own
+// overrides around its calls and resets them afterwards.  Returns 0, or 1 for an unknown name.
+extern "C" void ti_tuning_reset() {
+  g_tiles_160 = 1; g_two_ranges = 1; g_qkv_rows = 0; g_qkv_min_rows = 17; g_force_tile = 0; g_skinny_waves = 0;
+  g_skinny_deep = 1; g_use_pipelined = 1; set_tiled_from(280L << 20); g_row_per_wave = 1;
+  g_normed_weight_below = NORMED_WEIGHT_BELOW; g_skinny_copy = 1; g_wide_rows = 1; g_pieces = 1; g_add_split = 1;
+}
+extern "C" int ti_tuning_set(const char* name, long value) {
+  const std::string n = name ? name : "";
+  if (n == "force_tile") g_force_tile = (int)value;
+  else if (n == "normed_weight_below") g_normed_weight_below = value > 0 ? value : NORMED_WEIGHT_BELOW;
+  else if (n == "tiles_160") g_tiles_160 = (int)value;
+  else if (n == "two_ranges") g_two_ranges = (int)value;
+  else if (n == "skinny_waves") g_skinny_waves = (int)value;
+  else if (n == "qkv_prep_min_rows") g_qkv_min_rows = (int)value;
+  else if (n == "qkv_prep_rows") g_qkv_rows = (int)value;
+  else if (n == "wide_rows") g_wide_rows = (int)value;
+  else if (n == "tiled_from") set_tiled_from(value);
+  else if (n == "add_split") g_add_split = (int)value;
+  else if (n == "use_pipelined") g_use_pipelined = (int)value;
+  else if (n == "row_per_wave") g_row_per_wave = (int)value;
+  else if (n == "skinny_copy") g_skinny_copy = (int)value;
+  else if (n == "pieces") g_pieces = (int)value;
+  else if (n == "skinny_deep") g_skinny_deep = (int)value;
+  else return 1;
   return 0;
 }

@@ -1236,6 +1236,16 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     answer(ops.compute_units());
   } else if (op == "fill_random") {
     ops.fill_random(arg(0), text ? text : "normal", num(0), num(1), (uint64_t)num(2));
+  } else if (op == "tune") {
+    // text = "library name"; no text: every override of this object goes
+    if (!text || !*text) {
+      ops.untune();
+    } else {
+      const std::string t = text;
+      const size_t sp = t.find(' ');
+      if (sp == std::string::npos) throw Error("ti_ops_call: 'tune' takes \"library name\"");
+      ops.tune(t.substr(0, sp), t.substr(sp + 1), (long)num(0));
+    }
   } else if (op == "count_calls") {
     ops.count_calls(num(0) != 0);
   } else if (op == "fill_zero") {

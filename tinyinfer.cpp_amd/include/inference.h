@@ -338,6 +338,11 @@ class Ops {
     int force_paired_tiles = -1;    // 1 / 0: that kernel with / without pairs, whatever the launch
     int force_decode_splits = 0;    // > 0: the decode attention cuts every context into this many runs
   } use;
+  // A shape rule of a kernel library forced for this object's calls (tests and measurements; the names are listed
+  // in csrc/tinyinfer_kernels_tuning.h).  The rules are the libraries' own, process-wide: this object sets its
+  // overrides before each of its calls into that library and resets them afterwards.
+  void tune(const std::string& library, const std::string& name, long value);
+  void untune();
   static int decode_splits(int n_rows, int kv_heads, int heads, int context, int typical, int units, int head_dim = 128);
   // runs of keys for the prefill kernel with 64-row tiles, and whether it pairs a heavy with a light tile
   static int portion_launch(int n_tiles_small, int heads, int portion_context, int window, int units, bool* paired);
@@ -351,6 +356,8 @@ class Ops {
   DeviceBuffer argmax_scratch_;
   DeviceBuffer sample_scratch_;       // zero between calls
   struct { void* out = nullptr; int64_t count = 0; int splits = 0; } pending_;
+  std::map<std::string, std::map<std::string, long>> tuning_;
+  friend struct TunedScope;
   struct Timing;
   friend struct TimedScope;
   std::unique_ptr<Timing> timing_;

@@ -199,6 +199,14 @@ class Ops:
         """Switch per-call timing with events on or off (see `Ops::timing`)."""
         self._call("timing", [], [int(bool(on))], libs=["core"])
 
+    def tune(self, library: Optional[str] = None, name: str = "", value: int = 0) -> None:
+        """Force a shape rule of a kernel library for this object's calls (`Ops::tune`; the names are listed in
+        csrc/tinyinfer_kernels_tuning.h).  Without arguments: every override of this object goes."""
+        if library is None:
+            self._call("tune", [], [0], libs=["core"])
+        else:
+            self._call("tune", [], [int(value)], text=f"{library} {name}", libs=[library])
+
     def count_calls(self, on: bool) -> None:
         """List the calls without timing them (see `Ops::count_calls`): a step runs exactly as it does unobserved;
         `timing_report()` then gives the names, each ending in what the call took ("[mfma]", "[generic]", "[fused]")."""
@@ -319,6 +327,29 @@ class Ops:
             if x.dtype != dt or x.shape[0] < n:
                 raise KernelError("sample: per-row arguments must be float32/int32 [n]")
         self._call("sample", [logits, temperature, top_k, top_p, uniform, out])
+
+
+# ---------------------------------------------- how the host library hands rows to the attention kernels
+SERVED_HEAD_DIMS = (32, 64, 128)     # head sizes of the bfloat16 matrix-core attention kernels
+MAX_SPLITS = 64                      # the merge kernel's limit
+MIN_BLOCKS_PER_SPLIT = 16            # four 16-key blocks per wavefront at least
+
+
+def compute_units() -> int:
+    return int(get_ops()._call("compute_units", libs=["core"]))
+
+
+def decode_splits(n_rows: int, kv_heads: int, heads: int, context: int, typical: int = 0, head_dim: int = 128) -> int:
+    """Into how many runs the decode kernel splits the context (`Ops::decode_splits`, ops/ops.cpp)."""
+    return int(native.lib().ti_decode_splits(n_rows, kv_heads, heads, context, typical or context, compute_units(), head_dim))
+
+
+def portion_launch(ctx, heads: int, window: int):
+    """(runs of keys, paired) for the prefill kernel with 64-row tiles (`Ops::portion_launch`)."""
+    paired = ctypes.c_int()
+    runs = native.lib().ti_portion_launch(ctx.n_tiles_small, heads, getattr(ctx, "portion_context", 0), int(window or 0),
+                                          compute_units(), ctypes.byref(paired))
+    return int(runs), bool(paired.value)
 
 
 _OPS: Optional[Ops] = None

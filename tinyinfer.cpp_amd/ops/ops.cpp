@@ -277,6 +277,34 @@ bool kernel_library_available(const std::string& name) {
 }
 
 // ---------------------------------------------------------------------------------------- Ops
+// An object's overrides of a kernel library's shape rules, in force for the calls of one scope.
+static std::mutex g_tuning_mutex;
+struct TunedScope {
+  const char* lib = nullptr;
+  TunedScope(Ops& ops, const char* library) {
+    if (ops.tuning_.empty()) return;
+    auto it = ops.tuning_.find(library);
+    if (it == ops.tuning_.end() || it->second.empty()) return;
+    lib = library;
+    g_tuning_mutex.lock();
+    auto set = symbol<int (*)(const char*, long)>(library, "ti_tuning_set");
+    for (const auto& kv : it->second)
+      if (set(kv.first.c_str(), kv.second) != 0) {
+        symbol<void (*)()>(library, "ti_tuning_reset")();
+        g_tuning_mutex.unlock();
+        lib = nullptr;
+        throw KernelError(std::string("kernel library '") + library + "' has no shape rule '" + kv.first + "'");
+      }
+  }
+  ~TunedScope() {
+    if (!lib) return;
+    symbol<void (*)()>(lib, "ti_tuning_reset")();
+    g_tuning_mutex.unlock();
+  }
+};
+void Ops::tune(const std::string& library, const std::string& name, long value) { tuning_[library][name] = value; }
+void Ops::untune() { tuning_.clear(); }
+
 static const int64_t PARTIALS_BYTES = 32 << 20;
 static const int NORMED_MAX_ROWS = 16;
 
@@ -522,6 +550,7 @@ bool Ops::can_fuse_norm(int64_t n_rows, DType dtype) const {
 }
 
 bool Ops::linear_with_norm(const Rows& a, const Tensor& w, const Tensor& out, Epilogue epi) {
+  TunedScope tuned(*this, "gemm_bf16");
   static const char* EPI_NAMES[] = {"store", "add", "store_act", "swiglu"};
   TIMED(std::string("norm+linear.") + EPI_NAMES[epi] + " " + dims(a.t) + " * " + dims(w));
   const int64_t M = a.t.shape[0], K = a.t.shape[1];
@@ -556,6 +585,7 @@ void Ops::linear(const Rows& a, const Tensor& w, const Tensor& out, Epilogue epi
 }
 
 void Ops::linear(const Tensor& a, const Tensor& w, const Tensor& out, Epilogue epi, bool may_defer) {
+  TunedScope tuned(*this, "gemm_bf16");
   static const char* EPI_NAMES[] = {"store", "add", "store_act", "swiglu"};
   TIMED(std::string("linear.") + EPI_NAMES[epi] + " " + dims(a) + " * " + dims(w));
   require(a.ndim == 2 && w.ndim == 2, "linear: a and w must be matrices");
@@ -622,6 +652,7 @@ void Ops::linear(const Tensor& a, const Tensor& w, const Tensor& out, Epilogue e
 bool Ops::qkv_prepared(const Rows& a, const Tensor& w, const float* q_w, const float* k_w, float eps, const Rotation& rot,
                        const int* positions, const int* slots, const CacheView& view, const Tensor& pool,
                        const Tensor& q_out, int heads, int kv_heads, int head_dim) {
+  TunedScope tuned(*this, "gemm_bf16");
   TIMED("qkv_prepared " + dims(a.t) + " * " + dims(w));
   if (!(use.fused_qkv_prefill && use.fast_gemm) || a.lazy) return false;
   if (a.t.dtype != DType::BF16 || w.dtype != DType::BF16 || q_out.dtype != DType::BF16) return false;
@@ -723,6 +754,7 @@ bool Ops::attention_from_projections(const AttentionWork& work, Workspace& ws, c
                                      const float* q_w, const float* k_w, float eps, const Rotation& rot,
                                      const Tensor& pool, bool write_kv, const Tensor& out, int heads, int kv_heads,
                                      int head_dim, float scale, int window) {
+  TunedScope tuned(*this, "attention_bf16");
   TIMED("attention.decode_prepared rows=" + std::to_string(work.M) + " context<=" + std::to_string(work.max_context));
   if (!(use.fused_qk_decode && use.fast_attention && work.decode_only && pool.dtype == DType::BF16)) return false;
   if (!kernel_library_available("attention_bf16")) return false;
@@ -759,6 +791,7 @@ bool Ops::attention_from_projections(const AttentionWork& work, Workspace& ws, c
 
 void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& view, const Tensor& q, const Tensor& pool,
                     const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window) {
+  TunedScope tuned(*this, "attention_bf16");
   TIMED("attention rows=" + std::to_string(work.M) + (work.decode_only ? " decode" : " tiles=" + std::to_string(work.n_tiles) + " single=" + std::to_string(work.n_decode_rows)) + " context<=" + std::to_string(work.max_context));
   bool done = false;
   if (q.dtype == DType::BF16 && use.fast_attention && kernel_library_available("attention_bf16")) {
