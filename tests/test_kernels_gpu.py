@@ -628,8 +628,18 @@ def test_linear_bf16_weight_row_per_wavefront(ops, M, N, K):
             ops.linear(a, w, acc, "add")
             assert (f64(acc) - (ref + f64(base))).abs().max() < tol
             results[on] = (out[:M].clone(), acc)
+        # the token rows straight into registers (up to K = 3,072 at 8 tokens) or through LDS: the same bits
+        lib.ti_tuning_set(b"row_per_wave", 1)
+        lib.ti_tuning_set(b"rows_direct", 0)
+        through_lds = torch.empty(M, N, device="cuda")
+        ops.linear(a, w, through_lds, "store")
+        assert torch.equal(through_lds, results[1][0])
+        acc = dev(base.clone())
+        ops.linear(a, w, acc, "add")
+        assert torch.equal(acc, results[1][1])
     finally:
         lib.ti_tuning_set(b"row_per_wave", 1)
+        lib.ti_tuning_set(b"rows_direct", 1)
     assert (results[1][0] - results[0][0]).abs().max() < tol
     # a row's bits do not depend on the rows beside it
     if M > 1:

@@ -60,7 +60,7 @@ def test_config_b_workload_in_bfloat16(model_folders, top_k):
             exact = plain.forward(w, cfg, seq)[-1]
             want = plain.forward(w, cfg, seq, ENGINE_SITES)[-1]
             ref = plain.forward(w, cfg, seq, REFERENCE_SITES)[-1]
-            bound = 2.0 * max(float(np.abs(want - exact).max()), 1e-3)
+            bound = 1.0 * max(float(np.abs(want - exact).max()), 1e-3)
             err = float(np.abs(logits[row] - want).max())
             assert err < bound, (r.number, len(seq), err, bound)
             checked["worst"] = max(checked["worst"], err)

@@ -20,6 +20,7 @@
 //   skinny_copy          0: up to 16 tokens, fragments of the token rows straight from memory
 //   pieces               0: up to 16 rows never take the kernel with the token rows in pieces
 //   skinny_deep          0: four chunks of K in flight per wavefront also for a long K
+//   rows_direct          0: the kernel with a weight row per wavefront takes its token rows through LDS for every K
 // libti_attention_bf16:
 //   decode_shared_query  0: every wavefront of a decode workgroup prepares the query itself
 //   prefill_groups       1 or 2 groups of wavefronts per workgroup, 0: by the launch
