@@ -275,11 +275,12 @@ def measure_prefill(engine, rng, tokens, reps=5):
     return times[len(times) // 2]
 
 
-def measure_mixed(engine, batch, portion, cached, context, rng, reps=8):
+def measure_mixed(engine, batch, portion, cached, context, rng, reps=8, graph=False):
     """ms of a step that holds one decoded token of each of `batch` requests (`context` tokens each)
     beside `portion` tokens of a prompt of which `cached` tokens are in the cache already: what the
-    scheduler runs while a prompt arrives in portions.  Not a captured graph.  Also the ms after
-    which the host has handed the whole step to the GPU."""
+    scheduler runs while a prompt arrives in portions.  graph: through `step_graph`, which replays a
+    step's shape from a captured graph once it has come twice (generation with --cuda-graph).  Also
+    the ms after which the host has handed the whole step to the GPU."""
     import torch
     from tinyinfer_amd.engine import StepEntry
     V = engine.model.vocab_size
@@ -293,7 +294,7 @@ def measure_mixed(engine, batch, portion, cached, context, rng, reps=8):
         entries.append(StepEntry("long", rng.integers(0, V, size=portion).tolist(), (portion - 1,)))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        logits = engine.step(entries)
+        logits = (engine.step_graph if graph else engine.step)(entries)
         t1 = time.perf_counter()
         logits[0, :8].cpu()
         torch.cuda.synchronize()
@@ -369,7 +370,9 @@ def main() -> int:
     if args.only == "mixed":
         say(f"a step of {args.batch} decoded tokens beside a portion of {args.portion} (after {args.cached} cached) ...")
         ms, host_ms = measure_mixed(engine, args.batch, args.portion, args.cached, context, rng)
-        print(json.dumps({"mixed": {"ms_per_step": round(ms, 3), "host_ms": round(host_ms, 3), "tokens": args.batch + args.portion,
+        g_ms, g_host = measure_mixed(engine, args.batch, args.portion, args.cached, context, rng, graph=True)
+        print(json.dumps({"mixed": {"ms_per_step": round(ms, 3), "host_ms": round(host_ms, 3), "ms_from_graph": round(g_ms, 3),
+                                    "host_ms_from_graph": round(g_host, 3), "tokens": args.batch + args.portion,
                                     "decoded": args.batch, "portion": args.portion, "cached": args.cached,
                                     "decode_context": context, "model": NAMES[args.model]}}), flush=True)
         return 0

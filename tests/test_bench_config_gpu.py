@@ -144,8 +144,7 @@ def test_decode_attention_at_contexts_of_2048_to_4095():
     from tinyinfer_amd.ops.kernels import get_ops
     from test_kernels_gpu import fast_attention_case
     ops = get_ops()
-    if not ops.use_fast_attention:
-        pytest.skip("bfloat16 attention kernels are switched off")
+    assert ops.use_fast_attention, "the bfloat16 attention kernels are switched off or not built"
     entries = [(1, s) for s in (2047, 2048, 2049, 3000, 3583, 4094)]
     got, want = fast_attention_case(ops, entries, 16, 8, 128, 16, None, seed=4095)
     assert torch.isfinite(got).all()

@@ -51,3 +51,14 @@ def test_bench_line_keeps_the_contract(drawn):
     assert out["roofline"]["bound"] == "hbm" and out["roofline"]["peak"] == 8000.0 and out["roofline"]["unit"] == "GB/s"
     assert abs(out["roofline"]["frac"] - out["roofline"]["achieved"] / out["roofline"]["peak"]) < 1e-3
     assert set(out["points"]) == {"decode_b1", "decode_b64"} and all(v > 0 for v in out["points"].values())
+    # the figures behind the fractions, worked out here by hand for this configuration (one layer): every matrix of
+    # the layer and the tied head once, norm vectors in 32-bit, keys and values of 8 requests at their mean length
+    layer, head = (4096 + 2048 + 2 * 3 * 3072) * 1024, 151936 * 1024
+    weight_bytes = (layer + head) * 2 + (2 * 1024 + 2 * 128 + 1024) * 4
+    kv_bytes = 8 * (2048 + 2 + 6 / 2) * 2 * 8 * 128 * 2
+    achieved = (weight_bytes + kv_bytes) / (out["ms_per_step"] * 1e-3) / 1e9
+    assert abs(out["roofline"]["achieved"] - achieved) < 0.01 * achieved, (out["roofline"]["achieved"], achieved)
+    flops = 2.0 * layer * 2048 + 2.0 * head + 2.0 * 128 * 2048 * 2049 * 16
+    frac = flops / (out["prefill"]["ms"] * 1e-3) / 2.5e15
+    assert abs(out["prefill"]["frac"] - frac) < 0.01 * frac + 1e-4, (out["prefill"]["frac"], frac)
+    assert abs(out["prefill"]["value"] - 2048 / (out["prefill"]["ms"] * 1e-3)) < 0.01 * out["prefill"]["value"]

@@ -573,8 +573,7 @@ def test_linear_bf16_matrix_cores(ops, M, N, K):
     """The skinny (M <= 64) and tiled (M > 64) MFMA kernels against float64, every
     epilogue, at sizes that are no multiples of their tiles.  (5, 261, 1024) is the
     reference's own case, src/selftest.cpp:33-72."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     g = torch.Generator().manual_seed(M * 7 + N)
     a = (torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16)
     w = (torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16)
@@ -606,8 +605,7 @@ def test_linear_bf16_weight_row_per_wavefront(ops, M, N, K):
     wavefront, at the edges of what it serves (one row, one piece of K, the longest K, every
     template variant of M and K), with strided token rows, against float64 and against the
     kernels that take these sizes when it is switched off (same values up to rounding)."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     g = torch.Generator().manual_seed(M * 11 + N + K)
     wide = (torch.rand(M, K + 24, generator=g) * 2 - 1).to(torch.bfloat16)
     a = dev(wide)[:, 8:8 + K]                                    # rows 16 bytes into a wider matrix
@@ -656,8 +654,7 @@ def test_linear_bf16_mfma_fed_from_memory(ops, M, N, K, ks):
     do not fill a tile, K split over workgroups with the partial sums added afterwards, strided
     rows; against float64.  A row's bits do not depend on the rows beside it."""
     import ctypes
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     lib = ops.lib("gemm_bf16")
     g = torch.Generator().manual_seed(M * 7 + N + K + ks)
     wide = (torch.rand(M, K + 24, generator=g) * 2 - 1).to(torch.bfloat16)
@@ -706,8 +703,7 @@ def test_linear_bf16_token_rows_in_pieces(ops, M, N, K, ks):
     not depend on the rows beside it, and with K in one workgroup they are the bits of the kernels that take
     all of K into LDS at once."""
     import ctypes
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     lib = ops.lib("gemm_bf16")
     g = torch.Generator().manual_seed(M * 7 + N + K + ks)
     wide = (torch.rand(M, K + 24, generator=g) * 2 - 1).to(torch.bfloat16)
@@ -766,8 +762,7 @@ def test_linear_bf16_long_k_split_for_few_rows(ops, M):
     """Up to 16 rows added into a residual through a weight with a long K and few rows (the shape of a
     large model's down projection): K goes to several workgroups; their sums are left to the next norm,
     or added at once, with the same bits; a row's bits do not depend on the rows beside it."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     N, K = 2064, 17408
     g = torch.Generator().manual_seed(M)
     a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
@@ -805,8 +800,7 @@ def test_linear_bf16_large_weight_at_17_to_64_rows(ops, M, epilogue):
     kernels take the product (their tile partly empty), below that the kernels whose workgroups
     own 16 weight rows.  Both sides of the rule and the rule switched off agree with float64 and
     with one another up to rounding; the adding epilogue with its sums left to a later kernel too."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     N, K = 8192, 2048
     g = torch.Generator().manual_seed(M)
     a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
@@ -851,8 +845,7 @@ def test_linear_bf16_large_weight_at_13_to_16_rows(ops):
     these row counts (rows x elements of 600 Mi or more), so the tiled kernels take the product and
     a norm in front becomes a kernel of its own; 12 rows stay with the kernels that take the norm
     in.  Against float64, and the rule switched off."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     from tinyinfer_amd.ops.kernels import NormedRows
     N, K = 49152, 1024
     g = torch.Generator().manual_seed(3)
@@ -885,8 +878,7 @@ def test_linear_bf16_wide_weight_at_17_to_64_rows(ops, M, N, K):
     weight's tiles.  One to four k-blocks per wavefront, four and eight wavefronts, a last tile
     beyond the matrix, strided token rows; against float64 and against the kernels that take the
     product when this one is switched off; a row's bits do not depend on the rows beside it."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     g = torch.Generator().manual_seed(M + N + K)
     wide = (torch.rand(M, K + 24, generator=g) * 2 - 1).to(torch.bfloat16)
     a = dev(wide)[:, 8:8 + K]
@@ -921,8 +913,7 @@ def test_partial_sums_left_to_the_next_norm(ops, M, N, K):
     With `may_defer` its partial sums wait for whatever reads the residual next: the norm adds
     them on its way, any other launch (or `flush`) adds them with a kernel of their own.  All
     three give the bits of the product that adds them at once, and match float64."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     g = torch.Generator().manual_seed(M + N + K)
     a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
     w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
@@ -1004,8 +995,7 @@ def test_linear_bf16_every_tile(ops, tile, M, N, K):
     """Each tile of the pipelined kernel (256 x 128 with eight wavefronts, 128 x 64, 64 x 128 for the SwiGLU
     epilogue, 64 x 64, and 128 x 160 and 256 x 160 with four wavefronts, which the SwiGLU epilogue does not
     take), whatever the dispatch would have chosen for the shape, with every epilogue, against float64."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     lib = ops.lib("gemm_bf16")
     g = torch.Generator().manual_seed(M + N + tile)
     a = (torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16)
@@ -1042,8 +1032,7 @@ def test_columns_split_between_two_tile_shapes(ops, M, N, K):
     """256 x 128 tiles that fill the compute units once or more and leave a round mostly empty: the columns
     that make whole rounds take those tiles, the rest 128 x 64 tiles in a second launch.  Same bits as the
     smaller tile everywhere, and the values of float64, for every epilogue."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     lib = ops.lib("gemm_bf16")
     units = torch.cuda.get_device_properties(0).multi_processor_count
     big = -(-M // 256) * -(-N // 128)
@@ -1083,8 +1072,7 @@ def test_columns_split_between_two_tile_shapes(ops, M, N, K):
 def test_widths_that_160_divides_take_tiles_of_160_columns(ops, M, N, K):
     """Where tiles of 256 x 160 or 128 x 160 make whole rounds of the compute units the dispatch takes them
     (widths of 2,560 and 5,120).  Same bits as without them, and the values of float64."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     lib = ops.lib("gemm_bf16")
     units = torch.cuda.get_device_properties(0).multi_processor_count
     assert (-(-M // 256) * (N // 160)) % units == 0 or (-(-M // 128) * (N // 160)) % units == 0, "the shape does not take the rule"
@@ -1118,8 +1106,7 @@ def test_widths_that_160_divides_take_tiles_of_160_columns(ops, M, N, K):
 def test_swiglu_of_up_to_64_rows_under_a_wide_weight(ops, M):
     """17 to 64 rows times a stacked [gate; up] weight of 32,768 rows take 64 x 128 tiles (twice the weight
     under way per workgroup); the bits are those of the 128 x 64 tiles, and the values match float64."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     F, K = 16384, 1024
     g = torch.Generator().manual_seed(M)
     a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
@@ -1146,8 +1133,7 @@ def test_stored_product_of_17_to_64_rows_under_a_large_weight_splits_k(ops, M):
     32-bit: K goes to several workgroups a tile and a kernel of its own adds their sums.  Against float64,
     against the product with the split switched off (the same values up to the order of the sum), and a
     row's bits do not depend on the rows beside it."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     N, K = 6144, 4096
     g = torch.Generator().manual_seed(M)
     a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
@@ -1174,8 +1160,7 @@ def test_linear_bf16_rows_do_not_depend_on_the_batch(ops):
     """Within one family of kernels a row's bits do not depend on the other rows: the tiled
     kernels (more than 64 rows), the kernels whose workgroups own 16 weight rows (9 to 64 rows
     here), and the kernel with a weight row per wavefront (up to 8 rows, a weight of few rows)."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     g = torch.Generator().manual_seed(4)
     a = torch.randn(200, 264, generator=g).to(torch.bfloat16)
     w = torch.randn(150, 264, generator=g).to(torch.bfloat16)
@@ -1204,8 +1189,7 @@ def test_linear_bf16_few_columns_many_wavefronts(ops, M, N, K):
     """Few output columns and a long K: up to 8 rows take the kernel with a weight row per
     wavefront, more rows the kernel with eight wavefronts that split K.  Same result as float64,
     and a row has the bits it has in a larger batch of the same family."""
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     g = torch.Generator().manual_seed(M + N)
     a = (torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16)
     w = (torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16)
@@ -1230,8 +1214,7 @@ def test_linear_with_the_norm_inside(ops, M, N, K):
     tokens and a weight of fewer than 4,096 rows are left to the kernel with a weight row per
     wavefront, except for SwiGLU: see the next test.)"""
     from tinyinfer_amd.ops.kernels import NormedRows
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     g = torch.Generator().manual_seed(M * 3 + N)
     x = dev(torch.randn(M, K, generator=g) * 3.0)
     nw = dev(1 + 0.1 * torch.randn(K, generator=g))
@@ -1264,8 +1247,7 @@ def test_linear_with_the_norm_inside_refuses_what_it_does_not_serve(ops):
     of few rows (which another kernel takes): `linear` computes the norm first and the result
     is that of the norm kernel followed by the product."""
     from tinyinfer_amd.ops.kernels import NormedRows
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     g = torch.Generator().manual_seed(9)
     for M, N, K in ((17, 32, 128), (4, 32, 72), (4, 32, 128), (8, 1024, 2048)):
         x = dev(torch.randn(M, K, generator=g))
@@ -1366,8 +1348,7 @@ def fast_attention_case(ops, entries_tokens, nh, nkv, hd, P, window, seed, sharp
     (4, 4, 64, 16, 40), (20, 1, 32, 16, None), (8, 2, 128, 16, 300)])
 def test_attention_bf16_decode_rows(ops, nh, nkv, hd, P, window):
     """Single-token entries at many context lengths, page edges included, split over the context."""
-    if not ops.use_fast_attention:
-        pytest.skip("bfloat16 attention kernels are switched off")
+    assert ops.use_fast_attention, "the bfloat16 attention kernels are switched off or not built"
     entries = [(1, s) for s in (0, 1, 15, 16, 17, 31, 32, 100, 511, 512, 777, 1500)]
     got, want = fast_attention_case(ops, entries, nh, nkv, hd, P, window, seed=nh * 100 + hd)
     assert torch.isfinite(got).all()
@@ -1383,8 +1364,7 @@ def test_attention_bf16_portions_and_mixed(ops, nh, nkv, hd, P, window, variant)
     page, the start of a request), beside decode rows; with one and with two groups of
     wavefronts per workgroup, and with the kernel of 64-row tiles, giving a workgroup two
     tiles or one (the launch would choose by its size)."""
-    if not ops.use_fast_attention:
-        pytest.skip("bfloat16 attention kernels are switched off")
+    assert ops.use_fast_attention, "the bfloat16 attention kernels are switched off or not built"
     entries = [(2, 0), (7, 30), (1, 99), (16, 16), (17, 15), (64, 0), (65, 63), (130, 41), (1, 0), (3, 300), (200, 5),
                (333, 700)]
     lib = ops.lib("attention_bf16")
@@ -1407,8 +1387,7 @@ def test_attention_bf16_far_into_long_contexts(ops):
     context (300 tokens behind 20,000, 70 behind 9,000: tiles that walk hundreds of pages, the keys in runs),
     against the softmax in float64 of just these rows.  In every request the key at position 7 is made to
     stand out for the last query of head 0, so that a page dropped far back would show."""
-    if not ops.use_fast_attention:
-        pytest.skip("bfloat16 attention kernels are switched off")
+    assert ops.use_fast_attention, "the bfloat16 attention kernels are switched off or not built"
     from tinyinfer_amd.ops import kernels as attention_bf16
     nh, nkv, hd, P = 4, 2, 128, 16
     entries = [(1, 20000), (300, 20000), (1, 32767), (70, 9000), (1, 5)]
@@ -1462,8 +1441,7 @@ def test_attention_bf16_paired_tiles_of_one_long_prompt(ops):
     """A prompt of 1,100 tokens in one step (an odd number of 64-row tiles, the last one short):
     the kernel that pairs the tile of the most keys with the one of the fewest, against the
     kernel that takes one tile of 128 rows per workgroup and against the softmax in float64."""
-    if not ops.use_fast_attention:
-        pytest.skip("bfloat16 attention kernels are switched off")
+    assert ops.use_fast_attention, "the bfloat16 attention kernels are switched off or not built"
     outs = []
     try:
         for paired in (True, False):
@@ -1485,8 +1463,7 @@ def test_attention_bf16_short_portions_against_a_long_context(ops, nh, nkv, hd, 
     start of a request (its later runs are empty), one in between, and a single token (its
     row is written by the decode kernel after the merge has passed over it); against float64
     and against the same launch with one run."""
-    if not ops.use_fast_attention:
-        pytest.skip("bfloat16 attention kernels are switched off")
+    assert ops.use_fast_attention, "the bfloat16 attention kernels are switched off or not built"
     from tinyinfer_amd.ops import kernels as attention_bf16
     entries = [(70, 3000), (40, 0), (1, 2500), (130, 1000)]
     ctx = FakeCtx(entries)
@@ -1525,8 +1502,7 @@ def test_attention_bf16_decode_from_projections_behind_long_contexts(ops):
 
 
 def decode_from_projections_case(ops, nh, nkv, hd, P, window, norm, rope, starts):
-    if not ops.use_fast_attention:
-        pytest.skip("bfloat16 attention kernels are switched off")
+    assert ops.use_fast_attention, "the bfloat16 attention kernels are switched off or not built"
     g = torch.Generator().manual_seed(nh * 31 + hd)
     entries = [(1, s) for s in starts]
     n_pages_each = [-(-(s + 1) // P) for s in starts]
@@ -1619,8 +1595,7 @@ def test_qkv_product_with_prepared_heads_in_two_ranges(ops, M, nh, nkv, hd):
 
 
 def qkv_prepared_case(ops, tile_rows, M, nh, nkv, hd, K, P, norm, rope):
-    if not ops.use_fast_gemm:
-        pytest.skip("bfloat16 MFMA kernels are switched off")
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     g = torch.Generator().manual_seed(M + nh)
     N = (nh + 2 * nkv) * hd
     a = dev((torch.randn(M, K, generator=g)).to(torch.bfloat16))
@@ -1673,8 +1648,7 @@ def qkv_prepared_case(ops, tile_rows, M, nh, nkv, hd, K, P, norm, rope):
 
 def test_attention_bf16_far_key(ops):
     """One key far back carries the weight, for a decode row and for a row inside a portion."""
-    if not ops.use_fast_attention:
-        pytest.skip("bfloat16 attention kernels are switched off")
+    assert ops.use_fast_attention, "the bfloat16 attention kernels are switched off or not built"
     from tinyinfer_amd.ops import kernels as attention_bf16
     T, hd, P = 1000, 64, 16
     g = torch.Generator().manual_seed(21)

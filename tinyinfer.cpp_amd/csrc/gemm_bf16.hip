@@ -1812,8 +1812,9 @@ static int g_wide_rows = 1;      // a hook for measurements: 0: the kernel above
 #define WIDE_ROWS_MIN_N 16384
 
 // whether gemm_wide_rows_kernel takes the product (storing 32-bit results)
+static int g_wide_rows_min_n = WIDE_ROWS_MIN_N, g_wide_rows_grid = 0;     // hooks for measurements
 static bool wide_rows_serves(int M, int N, int K, int epi) {
-  return g_wide_rows && epi == TI_EPI_STORE_F32 && M > 16 && M <= 64 && N >= WIDE_ROWS_MIN_N && K % 64 == 0 &&
+  return g_wide_rows && epi == TI_EPI_STORE_F32 && M > 16 && M <= 64 && N >= g_wide_rows_min_n && K % 64 == 0 &&
          K / 64 <= 4 * 8;
 }
 
@@ -1828,7 +1829,7 @@ static void launch_wide_rows(const bf16_t* a, const bf16_t* w, float* out, int M
     if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) units = prop.multiProcessorCount;
     cached_units = units > 0 ? units : 256;
   }
-  const int grid = min(tiles, cached_units);
+  const int grid = g_wide_rows_grid > 0 ? min(tiles, g_wide_rows_grid) : min(tiles, cached_units);
 #define TI_GO(MBV)                                                                                   \
   if (eight) gemm_wide_rows_kernel<MBV, 8><<<grid, 512, 0, s>>>(a, w, out, M, N, K, lda);            \
   else gemm_wide_rows_kernel<MBV, 4><<<grid, 256, 0, s>>>(a, w, out, M, N, K, lda)
@@ -2194,6 +2195,8 @@ extern "C" void ti_tuning_reset() {
   g_skinny_deep = 1; g_use_pipelined = 1; set_tiled_from(280L << 20); g_row_per_wave = 1;
   g_normed_weight_below = NORMED_WEIGHT_BELOW; g_skinny_copy = 1; g_wide_rows = 1; g_pieces = 1; g_add_split = 1;
   g_rows_direct = 1;
+  g_wide_rows_min_n = WIDE_ROWS_MIN_N;
+  g_wide_rows_grid = 0;
 }
 extern "C" int ti_tuning_set(const char* name, long value) {
   const std::string n = name ? name : "";
@@ -2213,6 +2216,8 @@ extern "C" int ti_tuning_set(const char* name, long value) {
   else if (n == "pieces") g_pieces = (int)value;
   else if (n == "skinny_deep") g_skinny_deep = (int)value;
   else if (n == "rows_direct") g_rows_direct = (int)value;
+  else if (n == "wide_rows_min_n") g_wide_rows_min_n = value > 0 ? (int)value : WIDE_ROWS_MIN_N;
+  else if (n == "wide_rows_grid") g_wide_rows_grid = (int)value;
   else return 1;
   return 0;
 }

@@ -21,6 +21,8 @@
 //   pieces               0: up to 16 rows never take the kernel with the token rows in pieces
 //   skinny_deep          0: four chunks of K in flight per wavefront also for a long K
 //   rows_direct          0: the kernel with a weight row per wavefront takes its token rows through LDS for every K
+//   wide_rows_min_n      the fewest weight rows from which 17..64 rows take the kernel that keeps them in registers (16,384)
+//   wide_rows_grid       its number of workgroups (0: a tile of 16 weight rows each, at most one per compute unit)
 // libti_attention_bf16:
 //   decode_shared_query  0: every wavefront of a decode workgroup prepares the query itself
 //   prefill_groups       1 or 2 groups of wavefronts per workgroup, 0: by the launch
