@@ -53,7 +53,7 @@ def test_bench_line_keeps_the_contract(drawn):
     assert set(out["points"]) == {"decode_b1", "decode_b64"} and all(v > 0 for v in out["points"].values())
     # the figures behind the fractions, worked out here by hand for this configuration (one layer): every matrix of
     # the layer and the tied head once, norm vectors in 32-bit, keys and values of 8 requests at their mean length
-    layer, head = (4096 + 2048 + 2 * 3 * 3072) * 1024, 151936 * 1024
+    layer, head = (4096 + 2048 + 3 * 3072) * 1024, 151936 * 1024
     weight_bytes = (layer + head) * 2 + (2 * 1024 + 2 * 128 + 1024) * 4
     kv_bytes = 8 * (2048 + 2 + 6 / 2) * 2 * 8 * 128 * 2
     achieved = (weight_bytes + kv_bytes) / (out["ms_per_step"] * 1e-3) / 1e9
