@@ -24,6 +24,7 @@
 // /root/reference/src/cuda/attention.cu:107-198.)
 #include <string>
 #include <type_traits>
+#include <utility>
 #include "common.h"
 #include "tinyinfer_kernels.h"
 #include "tinyinfer_kernels_tuning.h"
@@ -750,6 +751,16 @@ __device__ __forceinline__ void vm_wait_turns(int k) {
 #undef TI_VM
 }
 
+// f(integral_constant<int, 0>), f(<1>), ... f(<N - 1>), until one returns false
+template <typename F, int... Is>
+__device__ __forceinline__ void unrolled_while_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (void)(f(std::integral_constant<int, Is>{}) && ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void unrolled_while(F&& f) {
+  unrolled_while_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 // NG groups of NW wavefronts in the workgroup.  A tile is 32 NW rows: a column block of 32
 // tokens per wavefront of a group, and every group takes all of the tile's rows.  With more
 // than one group the turns (32 keys) go to the groups in rotation (each group loads and walks
@@ -757,10 +768,13 @@ __device__ __forceinline__ void vm_wait_turns(int k) {
 // LDS at the end.  More groups put two wavefronts on every SIMD when a launch has only one
 // workgroup per compute unit, so that one's loads, LDS reads and vector work hide behind the
 // other's matrix products.
+// CB: column blocks of 32 tokens per wavefront.  (Two, for groups of one wavefront that need no barrier
+// and read every K fragment once for 64 tokens, do not fit the registers: the accumulators and the
+// queries alone are 192, and the compiler moves them through the other register file all the time.)
 // PAIRED: a workgroup takes two tiles, one after the other: tiles[blockIdx.x] and
 // tiles[n_tiles - 1 - blockIdx.x] of a list ordered from the most keys to the fewest, so that
 // under a causal mask every workgroup of a launch has about the same work.
-template <int HD, int NG, int NW = 4, int ST = PF_STAGES, bool PAIRED = false>
+template <int HD, int NG, int NW = 4, int ST = PF_STAGES, bool PAIRED = false, int CB = 1>
 __global__ void __launch_bounds__(64 * NW * NG)
 attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool,
                         const int* __restrict__ table, int table_stride, const int* __restrict__ tiles,
@@ -771,7 +785,6 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
   // run z and leaves its maxima, sums and unscaled outputs in part_ml [row][head][z] = (m, l) and
   // part_o [row][head][z][HD] for the kernel that merges them
   const int n_splits = gridDim.z, split = blockIdx.z;
-  constexpr int CB = 1;                               // column blocks (of 32 tokens) per wavefront
   constexpr int WROWS = 32 * CB;                      // tokens per wavefront
   constexpr int TROWS = NW * WROWS;                   // tokens per tile
   constexpr int NP = HD / 8;                          // 16-byte pieces per K row
@@ -798,7 +811,10 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     head = (xcd + 8 * (local / per_kv)) * (n_head / n_kv) + rest / gridDim.x;
     bx = rest % gridDim.x;
   }
-  const int grp = (threadIdx.x >> 6) / NW, wave = (threadIdx.x >> 6) % NW, lane = threadIdx.x & 63;
+  // the wavefront's number in scalar registers: what follows from it (which turns it loads, where they
+  // go, which rows are its own) is then worked out once per wavefront, not once per lane
+  const int wid = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int grp = wid / NW, wave = wid % NW, lane = threadIdx.x & 63;
   const int r32 = lane & 31, h = lane >> 5;
   const int kvh = head / (n_head / n_kv);
   const size_t page_elems = (size_t)2 * n_kv * P * HD;
@@ -813,31 +829,35 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
   //            holds piece c ^ (r & (NP - 1)) of key 16 (r / 16) + swap23(r % 16)
   //  V load g: dims 16 g .. 16 g + 15, 64 bytes each; lane i -> dim d = 16 g + i / 4, slot c = i % 4,
   //            holds piece c ^ ((d >> 2) & 3): keys 16 (piece / 2) + 8 (piece % 2) .. + 7
-  // packed per load: (element offset inside the page, without the row of the block's first
-  // key) * 2 + (which 16-key block of the turn).  Loads j < MY_K are K loads.
-  int ld_desc[MY_LOADS];
-#pragma unroll
-  for (int j = 0; j < MY_LOADS; ++j) {
-    if (j < MY_K) {
-      const int g = wave + NW * j;
-      const int r = K_ROWS * g + lane / NP, c = lane % NP;
-      const int r16 = r & 15;
-      const int key16 = ((r16 & 4) << 1) | ((r16 & 8) >> 1) | (r16 & 3);
-      ld_desc[j] = (key16 * HD + (c ^ (r & (NP - 1))) * 8) * 2 + (r >> 4);
-    } else {
-      const int gv = wave + NW * (j - MY_K);
-      const int d = 16 * gv + (lane >> 2), c = lane & 3;
-      const int piece = c ^ ((d >> 2) & 3);
-      ld_desc[j] = (d * P + (piece & 1) * 8) * 2 + (piece >> 1);
-    }
-  }
+  // In bytes from a block's first K row, K load g takes for lane i (lr = i / NP < K_ROWS, c = i % NP)
+  //   (k_lane ^ X(g)) + C(g),  k_lane = swap23(lr) * HD * 2 + (c ^ lr) * 16,
+  //   X(g) = ((K_ROWS g) & (NP - 1)) * 16,  C(g) = swap23((K_ROWS g) & 15) * HD * 2
+  // (the row number K_ROWS g + lr has g's bits and the lane's bits apart, and so have its pieces), from the
+  // first block of the turn if (K_ROWS g) & 16 is clear, else from the second; and V load g takes, from
+  // the V^T row of a block's first key, v_lane + 32 g P, v_lane = ((i / 4) P + 8 (piece & 1)) * 2, from the
+  // second block in the lanes whose piece is 2 or 3.  One register a kind instead of one a load.
+  static_assert(K_ROWS <= 16 && (K_ROWS & (K_ROWS - 1)) == 0, "rows of a K load lie in one block of 16");
+  auto swap23 = [](int r16) __attribute__((always_inline)) { return ((r16 & 4) << 1) | ((r16 & 8) >> 1) | (r16 & 3); };
+  const unsigned k_lane = (unsigned)(swap23(lane / NP) * HD * 2 + (((lane % NP) ^ (lane / NP)) << 4));
+  const int v_piece = (lane & 3) ^ ((lane >> 4) & 3);
+  const unsigned v_lane = (unsigned)((((lane >> 2) * P) + (v_piece & 1) * 8) * 2);
+  const bool v_second = (v_piece >> 1) != 0;
 
   const unsigned lds0 = (unsigned)(size_t)smem + grp * (ST * STAGE);   // this group's stages
-  // LDS addresses of this lane's fragments (without stage and k-step)
-  const unsigned k_row = lds0 + r32 * (HD * 2);                     // K row r32
-  const unsigned v_row = lds0 + K_BYTES + r32 * 64;                 // V^T row (dim) r32 of a 32-dim block
+  // the wavefronts of a group wait for each other at the workgroup's barrier (a handshake of a group's
+  // two wavefronts through a word of LDS, which lets the groups drift apart, was slower: 4.72 ms against
+  // 4.59 ms for a prompt of 2,048 tokens at Qwen3-0.6B's sizes)
+  auto group_sync = [&]() __attribute__((always_inline)) {
+    if constexpr (NW > 1) __builtin_amdgcn_s_barrier();
+  };
+  // LDS addresses of this lane's fragments; the stage, and the dim block of a V^T fragment, are
+  // constants in the read instructions
+  unsigned k_addr[KS], v_addr[2];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) k_addr[ks] = lds0 + r32 * (HD * 2) + (((ks * 2 + h) ^ (r32 & (NP - 1))) << 4);
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) v_addr[tt] = lds0 + K_BYTES + r32 * 64 + (((tt * 2 + h) ^ ((r32 >> 2) & 3)) << 4);
 
-  int turn_count = 0;                                               // turns so far: picks the stage
   for (int slot = 0; slot < (PAIRED ? 2 : 1); ++slot) {
   // ---- this slot's tile
   const int tile = (slot == 0) ? bx : n_tiles - 1 - bx;
@@ -857,6 +877,75 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
   const int g_rows = min(TROWS, row_end - first);
   const int g_pos_first = start + (first - row0), g_pos_last = g_pos_first + g_rows - 1;
   const int g_lo = (window > 0 && g_pos_first - window + 1 > 0) ? g_pos_first - window + 1 : 0;
+
+  int blk_lo = (g_lo / PF_KEYS) * 2, blk_hi = g_pos_last / 16;         // 16-key blocks, starting on a turn
+  const int v_limit = min(kv_last, blk_hi * 16 + 15);               // last key whose value row is real
+  if (n_splits > 1) {
+    const int per = (((blk_hi + 1 - blk_lo) + n_splits - 1) / n_splits + 1) & ~1;   // whole turns
+    blk_lo += split * per;
+    blk_hi = min(blk_hi, blk_lo + per - 1);                         // a run past the end is empty
+  }
+
+  // A run is up to 64 blocks.  Lane i keeps where block c0 + i starts in the pool (in elements: the V^T
+  // row of its first key; its first K row lies prow * (HD - 1) further) and the row of its first key in
+  // its page, so that the walk waits for the block table once per run and divides by the page size once
+  // per run.  Blocks past the end stand on page 0, and so do blocks whose page was given back (all their
+  // keys are masked).
+  long base = 0;
+  int prow = 0;
+  auto run_blocks = [&](int c0, int nblk) __attribute__((always_inline)) {
+    const int key = (c0 + lane) * 16, pidx = key / P;
+    prow = key - pidx * P;
+    int page = (lane < nblk) ? tab[pidx] : 0;
+    if (page < 0) page = 0;
+    base = (long)page * (long)page_elems + prow;
+  };
+  // The loads of this group's turn i of the run into a stage (stage_off: its offset, a constant where
+  // the loop is unrolled).  Which blocks, which pages and where in LDS is the same in every lane and
+  // worked out in scalar registers; a lane adds the offset of its piece.  (Asking for a turn in portions
+  // between the steps of the turn before, so that the unit that takes the addresses (64 bytes a cycle
+  // for the whole compute unit) works beside the matrix cores, gained nothing.)
+  auto issue = [&](int i, unsigned stage_off) __attribute__((always_inline)) {
+    const int t = i * NG + grp;
+    const int ja = min(2 * t, 63), jb = min(2 * t + 1, 63);
+    const unsigned lo_a = __builtin_amdgcn_readlane((int)(unsigned)base, ja), hi_a = __builtin_amdgcn_readlane((int)(base >> 32), ja);
+    const unsigned lo_b = __builtin_amdgcn_readlane((int)(unsigned)base, jb), hi_b = __builtin_amdgcn_readlane((int)(base >> 32), jb);
+    const long v_a = (long)(((unsigned long)hi_a << 32) | lo_a), v_b = (long)(((unsigned long)hi_b << 32) | lo_b);
+    const long k_a = v_a + (long)__builtin_amdgcn_readlane(prow, ja) * (HD - 1);
+    const long k_b = v_b + (long)__builtin_amdgcn_readlane(prow, jb) * (HD - 1);
+#pragma unroll
+    for (int j = 0; j < MY_LOADS; ++j) {
+      const char* src;
+      unsigned dst;
+      if (j < MY_K) {
+        const int g = wave + NW * j;                              // the same in every lane
+        const int rows = K_ROWS * g;
+        const char* from = reinterpret_cast<const char*>(kpool + ((rows & 16) ? k_b : k_a)) +
+                           swap23(rows & 15) * HD * 2;
+        src = from + (k_lane ^ (unsigned)((rows & (NP - 1)) << 4));
+        dst = g * 1024;
+      } else {
+        const int gv = wave + NW * (j - MY_K);
+        const char* from = reinterpret_cast<const char*>(vpool + (v_second ? v_b : v_a));
+        src = from + v_lane + (size_t)gv * 32 * P;
+        dst = K_BYTES + gv * 1024;
+      }
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(size_t)(lds0 + stage_off + dst), 16, 0, 0);
+    }
+  };
+  constexpr int AHEAD = ST - 1;
+  // the first run's blocks and first turns are asked for before the queries: those arrive meanwhile
+  // (a workgroup whose run of keys is empty walks nothing, and nothing may be on its way into LDS
+  // when it goes on to the merge)
+  if (blk_lo <= blk_hi) {
+    const int nblk = min(64, blk_hi + 1 - blk_lo);
+    run_blocks(blk_lo, nblk);
+    const int my_turns = ((nblk + 1) / 2 - grp + NG - 1) / NG;
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i)
+      if (i < my_turns) issue(i, i * STAGE);
+  }
 
   v4u qf[CB][KS];
   int my_pos[CB];
@@ -887,249 +976,273 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
       for (int i = 0; i < 16; ++i) o[cb][d][i] = 0.f;
   }
 
-  int blk_lo = (g_lo / PF_KEYS) * 2, blk_hi = g_pos_last / 16;         // 16-key blocks, starting on a turn
-  const int v_limit = min(kv_last, blk_hi * 16 + 15);               // last key whose value row is real
-  if (n_splits > 1) {
-    const int per = (((blk_hi + 1 - blk_lo) + n_splits - 1) / n_splits + 1) & ~1;   // whole turns
-    blk_lo += split * per;
-    blk_hi = min(blk_hi, blk_lo + per - 1);                         // a run past the end is empty
-  }
+  // One turn of 32 keys from a stage for this wavefront's columns, in two steps: the scores, then the
+  // softmax and the second product.  plain (the same in every lane): every key of the turn is visible
+  // to every column and written: no compare at all.
+  auto turn_scores = [&](auto stage_tag, floatx16* sc) __attribute__((always_inline)) {
+    constexpr unsigned SOFF = decltype(stage_tag)::value * STAGE;
+    // ---- the fragments: keys now, values right behind them
+    v4u kf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kf[ks]) : "v"(k_addr[ks]), "n"(SOFF));
+    // ---- S^T = K . Q^T
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sc[cb][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (cb == 0) {
+          lgkm_wait(KS - 1 - ks);        // the first ks + 1 of the KS reads have arrived
+          asm volatile("" : "+v"(kf[ks]));
+        }
+        sc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[ks]),
+                                                         __builtin_bit_cast(bf16x8, qf[cb][ks]), sc[cb], 0, 0, 0);
+      }
+    }
+  };
+  auto turn_rest = [&](auto stage_tag, int key0, bool plain, const floatx16* sc) __attribute__((always_inline)) {
+    constexpr unsigned SOFF = decltype(stage_tag)::value * STAGE;
+    // the value fragments are asked for now and waited for after the softmax
+    v4u vf[DB][2];
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(vf[d][tt]) : "v"(v_addr[tt]), "n"(SOFF + d * 32 * 64));
+
+    // ---- masks, the online softmax and O^T += V^T . P^T, column block by column block: the matrix
+    // core works on one block's second product while the next block's softmax runs.  The scores stay
+    // as the first product left them: the maximum is taken over them and scaled once (the scale is
+    // positive), and the scale goes into the multiply-add of the exponent.
+    // element i of a lane: key key0 + 16 (i / 8) + 8 h + 4 ((i / 4) % 2) + i % 4
+    // (the keys' numbers are worked out behind the branches that need them, not before the loop and kept
+    // in registers: the compiler takes `hm` for something the branch has made)
+    int hm = h;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+      float sv[16];
+      if (plain) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sv[i] = sc[cb][i];
+      } else {
+        asm volatile("" : "+v"(hm));
+        const int hi = col_ok[cb] ? my_pos[cb] : -1;
+        const int lo = (window > 0) ? my_pos[cb] - window + 1 : 0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = key0 + 16 * (i >> 3) + 8 * hm + 4 * ((i >> 2) & 1) + (i & 3);
+          const bool see = (key <= hi) & (key >= lo);      // bitwise on purpose: selects, no branches
+          sv[i] = see ? sc[cb][i] : -INFINITY;
+        }
+      }
+      float bm = sv[0];
+#pragma unroll
+      for (int i = 1; i < 16; ++i) bm = fmaxf(bm, sv[i]);
+      bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+      const float m_new = fmaxf(mx[cb], bm * scale2);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      float ps = 0.f;
+      float pv[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        pv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale2, -m_safe));
+        ps += pv[i];
+      }
+      v4u pf[2];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+        pf[tt] = v4u{pack_bf16x2(pv[8 * tt], pv[8 * tt + 1]), pack_bf16x2(pv[8 * tt + 2], pv[8 * tt + 3]),
+                     pack_bf16x2(pv[8 * tt + 4], pv[8 * tt + 5]), pack_bf16x2(pv[8 * tt + 6], pv[8 * tt + 7])};
+      // the running maximum settles after a few turns; then nothing needs rescaling
+      if (__builtin_amdgcn_ballot_w64(m_new != mx[cb]) != 0) {
+        const float alpha = __builtin_amdgcn_exp2f(mx[cb] - m_safe);
+        l[cb] *= alpha;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[cb][d][i] *= alpha;
+        mx[cb] = m_new;
+      }
+      l[cb] += ps;
+
+      if (cb == 0) {
+        // the value fragments have had the first block's softmax to arrive
+        lgkm_wait(0);
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt) asm volatile("" : "+v"(vf[d][tt]));
+        if (!plain) {
+          if (key0 + PF_KEYS - 1 > v_limit || key0 < g_lo) {
+            // rows never written, and the stand-in page read for a block that was given back or
+            // lies past the end, may hold anything, NaN included, and 0 * NaN is NaN
+            asm volatile("" : "+v"(hm));
+#pragma unroll
+            for (int d = 0; d < DB; ++d)
+#pragma unroll
+              for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                  const int key = key0 + 16 * tt + 8 * hm + e;
+                  const bool drop = (key > v_limit) | (key < g_lo);
+                  const unsigned keep = drop ? ((e & 1) ? 0x0000FFFFu : 0xFFFF0000u) : 0xFFFFFFFFu;
+                  vf[d][tt][e >> 1] &= keep;
+                }
+          }
+        }
+      }
+#pragma unroll
+      for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+          o[cb][d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[d][tt]),
+                                                             __builtin_bit_cast(bf16x8, pf[tt]), o[cb][d], 0, 0, 0);
+    }
+  };
+
   for (int c0 = blk_lo; c0 <= blk_hi; c0 += 64) {
     const int nblk = min(64, blk_hi + 1 - c0);
     const int n_turns = (nblk + 1) / 2;
-    // the page ids of this run's blocks, one per lane; blocks past the end repeat page 0
-    int ids = (lane < nblk) ? tab[((c0 + lane) * 16) / P] : 0;
-    if (ids < 0) ids = 0;                                           // given back: all its keys are masked
-    // this group's turns are turns grp, grp + NG, ... of the run; i counts them
+    // this group's turns are turns grp, grp + NG, ... of the run; i counts them, and turn i of a run
+    // goes through stage i % ST
     const int my_turns = (n_turns - grp + NG - 1) / NG;
     const int n_iter = (n_turns + NG - 1) / NG;                      // the first group's count: the most
-    auto issue = [&](int i) {
-      const int t = i * NG + grp;
-      const unsigned stage = lds0 + ((turn_count + i) % ST) * STAGE;
-      const int pa = __builtin_amdgcn_readlane(ids, min(2 * t, 63));
-      const int pb = __builtin_amdgcn_readlane(ids, min(2 * t + 1, 63));
-      const int key0 = (c0 + 2 * t) * 16;
-      // where the two blocks of the turn start, in elements from the pool's first: the same in
-      // every lane (scalar arithmetic); a lane adds the offset of its piece
-      const int prow_a = key0 % P, prow_b = (key0 + 16) % P;
-      const long k_a = (long)pa * (long)page_elems + (long)prow_a * HD, k_b = (long)pb * (long)page_elems + (long)prow_b * HD;
-      const long v_a = (long)pa * (long)page_elems + prow_a, v_b = (long)pb * (long)page_elems + prow_b;
+    if (c0 != blk_lo) {
+      run_blocks(c0, nblk);
 #pragma unroll
-      for (int j = 0; j < MY_LOADS; ++j) {
-        const bool second = ld_desc[j] & 1;
-        const int off = ld_desc[j] >> 1;
-        const bf16_t* src;
-        unsigned dst;
-        if (j < MY_K) {
-          src = kpool + (second ? k_b : k_a) + off;
-          dst = (wave + NW * j) * 1024;
-        } else {
-          src = vpool + (second ? v_b : v_a) + off;
-          dst = K_BYTES + (wave + NW * (j - MY_K)) * 1024;
-        }
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (__attribute__((address_space(3))) void*)(size_t)(stage + dst), 16, 0, 0);
-      }
-    };
-    constexpr int AHEAD = ST - 1;
-#pragma unroll
-    for (int i = 0; i < AHEAD; ++i)
-      if (i < my_turns) issue(i);
-    for (int i = 0; i < n_iter; ++i) {
-      // this group's turn i has landed: only its turns issued after it (at most AHEAD - 1) may be
-      // outstanding.  Both groups pass the barrier together, also the one that has run out of turns.
-      vm_wait_turns<MY_LOADS, ST>(max(0, min(AHEAD - 1, my_turns - 1 - i)));
-      __builtin_amdgcn_s_barrier();
-      if (i + AHEAD < my_turns) issue(i + AHEAD);                  // into the stage that turn i - 1 has left
-      if (i >= my_turns) continue;
-      const int key0 = (c0 + 2 * (i * NG + grp)) * 16;
-      // nothing of this turn is visible to this wavefront: it only helps loading
-      if (w_rows == 0 || key0 > w_pos_last || key0 + PF_KEYS - 1 < w_lo) continue;
-      const unsigned st = ((turn_count + i) % ST) * STAGE;
-
-      // ---- the fragments of both tiles: keys now, values right behind them
-      v4u kf[KS];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const unsigned a = k_row + st + (((ks * 2 + h) ^ (r32 & (NP - 1))) << 4);
-        asm volatile("ds_read_b128 %0, %1" : "=v"(kf[ks]) : "v"(a));
-      }
-      // ---- S^T = K . Q^T, one column block after the other, so that the softmax of a
-      //      block can run while the matrix core is busy with the next one
-      floatx16 sc[CB];
-#pragma unroll
-      for (int cb = 0; cb < CB; ++cb) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sc[cb][i] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          if (cb == 0) {
-            lgkm_wait(KS - 1 - ks);        // the first ks + 1 of the KS reads have arrived
-            asm volatile("" : "+v"(kf[ks]));
-          }
-          sc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[ks]),
-                                                           __builtin_bit_cast(bf16x8, qf[cb][ks]), sc[cb], 0, 0, 0);
-        }
-      }
-      // the value fragments are asked for now and waited for after the softmax
-      v4u vf[DB][2];
-#pragma unroll
-      for (int d = 0; d < DB; ++d)
-#pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
-          const unsigned a = v_row + st + d * 32 * 64 + (((tt * 2 + h) ^ ((r32 >> 2) & 3)) << 4);
-          asm volatile("ds_read_b128 %0, %1" : "=v"(vf[d][tt]) : "v"(a));
-        }
-
-      // ---- masks and the online softmax, per column block
-      // element i of a lane: key key0 + 16 (i / 8) + 8 h + 4 ((i / 4) % 2) + i % 4
-      const bool plain = (key0 + PF_KEYS - 1 <= w_pos_first) && (w_rows == WROWS) &&
-                         (window <= 0 || key0 >= w_pos_last - window + 1);
-      v4u pf[CB][2];
-#pragma unroll
-      for (int cb = 0; cb < CB; ++cb) {
-        float sv[16];
-        if (plain) {                       // the same in every lane: no compare at all
-#pragma unroll
-          for (int i = 0; i < 16; ++i) sv[i] = sc[cb][i] * scale2;
-        } else {
-          const int hi = col_ok[cb] ? my_pos[cb] : -1;
-          const int lo = (window > 0) ? my_pos[cb] - window + 1 : 0;
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int key = key0 + 16 * (i >> 3) + 8 * h + 4 * ((i >> 2) & 1) + (i & 3);
-            const bool see = (key <= hi) & (key >= lo);      // bitwise on purpose: selects, no branches
-            sv[i] = see ? sc[cb][i] * scale2 : -INFINITY;
-          }
-        }
-        float bm = sv[0];
-#pragma unroll
-        for (int i = 1; i < 16; ++i) bm = fmaxf(bm, sv[i]);
-        bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
-        const float m_new = fmaxf(mx[cb], bm);
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        float ps = 0.f;
-        float pv[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          pv[i] = __builtin_amdgcn_exp2f(sv[i] - m_safe);
-          ps += pv[i];
-        }
-#pragma unroll
-        for (int tt = 0; tt < 2; ++tt)
-          pf[cb][tt] = v4u{pack_bf16x2(pv[8 * tt], pv[8 * tt + 1]), pack_bf16x2(pv[8 * tt + 2], pv[8 * tt + 3]),
-                           pack_bf16x2(pv[8 * tt + 4], pv[8 * tt + 5]), pack_bf16x2(pv[8 * tt + 6], pv[8 * tt + 7])};
-        // the running maximum settles after a few turns; then nothing needs rescaling
-        if (__builtin_amdgcn_ballot_w64(m_new != mx[cb]) != 0) {
-          const float alpha = __builtin_amdgcn_exp2f(mx[cb] - m_safe);
-          l[cb] *= alpha;
-#pragma unroll
-          for (int d = 0; d < DB; ++d)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o[cb][d][i] *= alpha;
-          mx[cb] = m_new;
-        }
-        l[cb] += ps;
-      }
-
-      // ---- O^T += V^T . P^T
-      lgkm_wait(0);
-#pragma unroll
-      for (int d = 0; d < DB; ++d)
-#pragma unroll
-        for (int tt = 0; tt < 2; ++tt) asm volatile("" : "+v"(vf[d][tt]));
-      if (key0 + PF_KEYS - 1 > v_limit || key0 < g_lo) {
-        // rows never written, and the stand-in page read for a block that was given back or
-        // lies past the end, may hold anything, NaN included, and 0 * NaN is NaN
-#pragma unroll
-        for (int d = 0; d < DB; ++d)
-#pragma unroll
-          for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-              const int key = key0 + 16 * tt + 8 * h + e;
-              const bool drop = (key > v_limit) | (key < g_lo);
-              const unsigned keep = drop ? ((e & 1) ? 0x0000FFFFu : 0xFFFF0000u) : 0xFFFFFFFFu;
-              vf[d][tt][e >> 1] &= keep;
-            }
-      }
-#pragma unroll
-      for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-        for (int d = 0; d < DB; ++d)
-#pragma unroll
-          for (int tt = 0; tt < 2; ++tt)
-            o[cb][d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[d][tt]),
-                                                               __builtin_bit_cast(bf16x8, pf[cb][tt]), o[cb][d],
-                                                               0, 0, 0);
+      for (int i = 0; i < AHEAD; ++i)
+        if (i < my_turns) issue(i, i * STAGE);
     }
-    turn_count += n_iter;
-    // every wavefront is done with this run's stages before the next run refills them
-    __builtin_amdgcn_s_barrier();
+    for (int i0 = 0; i0 < n_iter; i0 += ST) {
+      // ST turns, each with its stage as a constant; ends with the run
+      unrolled_while<ST>([&](auto si_tag) __attribute__((always_inline)) {
+        constexpr int si = decltype(si_tag)::value;
+        const int i = i0 + si;
+        if (i >= n_iter) return false;
+        // this wavefront's part of the group's turn i has landed: only its turns issued after it (at
+        // most AHEAD - 1) may be outstanding.  Then the group's wavefronts wait for each other: the
+        // whole turn has landed, and everyone is done with the turn before, whose stage turn
+        // i + AHEAD goes into.
+        vm_wait_turns<MY_LOADS, ST>(max(0, min(AHEAD - 1, my_turns - 1 - i)));
+        group_sync();
+        // turn i + AHEAD goes into the stage that turn i - 1 has left
+        if (i + AHEAD < my_turns) issue(i + AHEAD, ((si + AHEAD) % ST) * STAGE);
+        if (i >= my_turns) return true;
+        const int key0 = (c0 + 2 * (i * NG + grp)) * 16;
+        // nothing of this turn is visible to this wavefront: it only helps loading
+        if (w_rows == 0 || key0 > w_pos_last || key0 + PF_KEYS - 1 < w_lo) return true;
+        const bool plain = (key0 + PF_KEYS - 1 <= w_pos_first) && (w_rows == WROWS) &&
+                           (window <= 0 || key0 >= w_pos_last - window + 1);
+        floatx16 sc[CB];
+        turn_scores(si_tag, sc);
+        turn_rest(si_tag, key0, plain, sc);
+        return true;
+      });
+    }
+    // every wavefront of the group is done with this run's stages before the next run (or the merge)
+    // writes into them
+    group_sync();
   }
 
-  if constexpr (NG > 1) {
-    // The other groups hand their maxima, sums and outputs to the first through LDS (the stages
-    // are free now): lane for lane, all hold the same columns and dims.
-    constexpr int NVAL = DB * 16 + 2;
-    static_assert((NG - 1) * NW * NVAL * 64 * 4 <= NG * ST * STAGE, "the partial results fit into the stages");
-    if (grp > 0) {
-      float* xm = reinterpret_cast<float*>(smem) + (size_t)((grp - 1) * NW + wave) * NVAL * 64 + lane;
+  // ---- the result: o[cb][d][i] is dim 32 d + 8 (i / 4) + 4 h + i % 4 of token (column) r32 of block cb.
+  // `first_val`, `count_tag`: which of a lane's DB * 16 values of a block (value v = 16 d + i) these are; a
+  // lane's values come in fours of consecutive dims.
+  auto write_out = [&](int cb, const float* val, int first_val, auto count_tag, float m_all, float lt) __attribute__((always_inline)) {
+    constexpr int n_val = decltype(count_tag)::value;
+    if (!col_ok[cb]) return;
+    const int row = w_first + cb * 32 + r32;
+    if (n_splits > 1) {
+      const size_t at = ((size_t)row * n_head + head) * n_splits + split;
+      float* po = part_o + at * HD;
 #pragma unroll
-      for (int d = 0; d < DB; ++d)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) xm[(d * 16 + i) * 64] = o[0][d][i];
-      xm[(DB * 16) * 64] = mx[0];
-      xm[(DB * 16 + 1) * 64] = l[0];
-    }
-    __syncthreads();
-    if (grp == 0) {
-#pragma unroll
-      for (int g = 1; g < NG; ++g) {
-        const float* xm = reinterpret_cast<const float*>(smem) + (size_t)((g - 1) * NW + wave) * NVAL * 64 + lane;
-        const float m1 = xm[(DB * 16) * 64], l1 = xm[(DB * 16 + 1) * 64];
-        const float m_new = fmaxf(mx[0], m1);
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float a0 = __builtin_amdgcn_exp2f(mx[0] - m_safe), a1 = __builtin_amdgcn_exp2f(m1 - m_safe);
-        l[0] = l[0] * a0 + l1 * a1;
-#pragma unroll
-        for (int d = 0; d < DB; ++d)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o[0][d][i] = o[0][d][i] * a0 + xm[(d * 16 + i) * 64] * a1;
-        mx[0] = m_new;
+      for (int j = 0; j < n_val; j += 4) {
+        const int v = first_val + j;
+        *reinterpret_cast<float4*>(po + 32 * (v >> 4) + 8 * ((v & 15) >> 2) + 4 * h) =
+            make_float4(val[j], val[j + 1], val[j + 2], val[j + 3]);
       }
+      if (h == 0 && first_val == 0) reinterpret_cast<float2*>(part_ml)[at] = make_float2(m_all, lt);
+      return;
     }
-  }
-
-  // o[cb][d][i]: dim 32 d + 8 (i / 4) + 4 h + i % 4 of token (column) r32 of block cb
-  if (grp == 0) {
+    const float inv = 1.0f / lt;
+    bf16_t* dst = out + ((size_t)row * n_head + head) * HD;
+#pragma unroll
+    for (int j = 0; j < n_val; j += 4) {
+      const int v = first_val + j;
+      *reinterpret_cast<uint2*>(dst + 32 * (v >> 4) + 8 * ((v & 15) >> 2) + 4 * h) =
+          make_uint2(pack_bf16x2(val[j] * inv, val[j + 1] * inv), pack_bf16x2(val[j + 2] * inv, val[j + 3] * inv));
+    }
+  };
+  if constexpr (NG == 1) {
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
-      const float lt = l[cb] + __shfl_xor(l[cb], 32, 64);
-      if (!col_ok[cb]) continue;
-      const int row = w_first + cb * 32 + r32;
-      if (n_splits > 1) {
-        const size_t at = ((size_t)row * n_head + head) * n_splits + split;
-        float* po = part_o + at * HD;
+      float val[DB * 16];
 #pragma unroll
-        for (int d = 0; d < DB; ++d)
+      for (int v = 0; v < DB * 16; ++v) val[v] = o[cb][v >> 4][v & 15];
+      write_out(cb, val, 0, std::integral_constant<int, DB * 16>{}, mx[cb], l[cb] + __shfl_xor(l[cb], 32, 64));
+    }
+  } else {
+    // The groups merge their partial results through LDS (the stages are free now), each group the
+    // values it owns: values VPG g .. VPG (g + 1) - 1 of every lane are group g's.  A group leaves the
+    // values it does not own (in their order), its maximum and its sum in its part of LDS; after a
+    // barrier it reads the others' contributions to its own values, merges them with its own and
+    // writes them out.  Which registers a group takes its values from is a choice between registers by
+    // the group's number, which every lane of a wavefront shares: the accumulators stay in registers.
+    constexpr int VALS = DB * 16, VPG = VALS / NG, ML = VALS - VPG, SLOTS = ML + 2;
+    static_assert(VALS % NG == 0 && VPG % 4 == 0, "a group owns whole fours of values");
+    static_assert(NG * NW * SLOTS * 64 * 4 <= NG * ST * STAGE, "the partial results fit into the stages");
+    typedef __attribute__((address_space(3))) float lds_float;
+    auto part_of = [&](int g) __attribute__((always_inline)) {
+      return (lds_float*)(size_t)((unsigned)(size_t)smem + (unsigned)(((g * NW + wave) * SLOTS * 64 + lane) * 4));
+    };
+    // only the workgroup's barrier tells that every group is done with its stages
+    if constexpr (NW == 1) __syncthreads();
+    const int first = grp * VPG;                     // this group's first value
 #pragma unroll
-          for (int g4 = 0; g4 < 4; ++g4)
-            *reinterpret_cast<float4*>(po + 32 * d + 8 * g4 + 4 * h) =
-                make_float4(o[cb][d][4 * g4], o[cb][d][4 * g4 + 1], o[cb][d][4 * g4 + 2], o[cb][d][4 * g4 + 3]);
-        if (h == 0) reinterpret_cast<float2*>(part_ml)[at] = make_float2(mx[cb], lt);
-        continue;
+    for (int cb = 0; cb < CB; ++cb) {
+      if (cb > 0) __syncthreads();                   // the block before has been read
+      lds_float* mine = part_of(grp);
+#pragma unroll
+      for (int sl = 0; sl < ML; ++sl)                // slot sl: value sl below this group's own, sl + VPG above them
+        mine[sl * 64] = (sl < first) ? o[cb][sl >> 4][sl & 15] : o[cb][(sl + VPG) >> 4][(sl + VPG) & 15];
+      mine[ML * 64] = mx[cb];
+      mine[(ML + 1) * 64] = l[cb];
+      __syncthreads();
+      float m_g[NG], l_g[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        m_g[g] = part_of(g)[ML * 64];
+        l_g[g] = part_of(g)[(ML + 1) * 64];
       }
-      const float inv = 1.0f / lt;
-      bf16_t* dst = out + ((size_t)row * n_head + head) * HD;
+      float m_all = m_g[0];
 #pragma unroll
-      for (int d = 0; d < DB; ++d)
+      for (int g = 1; g < NG; ++g) m_all = fmaxf(m_all, m_g[g]);
+      const float m_safe = (m_all == -INFINITY) ? 0.f : m_all;
+      float a_g[NG], l_all = 0.f;
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          const uint2 r = make_uint2(pack_bf16x2(o[cb][d][4 * g4] * inv, o[cb][d][4 * g4 + 1] * inv),
-                                     pack_bf16x2(o[cb][d][4 * g4 + 2] * inv, o[cb][d][4 * g4 + 3] * inv));
-          *reinterpret_cast<uint2*>(dst + 32 * d + 8 * g4 + 4 * h) = r;
-        }
+      for (int g = 0; g < NG; ++g) {
+        a_g[g] = __builtin_amdgcn_exp2f(m_g[g] - m_safe);
+        l_all += l_g[g] * a_g[g];
+      }
+      const float a_own = __builtin_amdgcn_exp2f(mx[cb] - m_safe);
+      float val[VPG];
+#pragma unroll
+      for (int j = 0; j < VPG; ++j) {
+        float own = o[cb][j >> 4][j & 15];
+#pragma unroll
+        for (int g = 1; g < NG; ++g)
+          if (grp == g) own = o[cb][(g * VPG + j) >> 4][(g * VPG + j) & 15];
+        val[j] = own * a_own;
+      }
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        if (g == grp) continue;                      // the same in every lane
+        const lds_float* theirs = part_of(g) + (first + (grp > g ? -VPG : 0)) * 64;
+#pragma unroll
+        for (int j = 0; j < VPG; ++j) val[j] += theirs[j * 64] * a_g[g];
+      }
+      write_out(cb, val, first, std::integral_constant<int, VPG>{}, m_all, l_all + __shfl_xor(l_all, 32, 64));
     }
   }
   // the next tile's loads go into the LDS that the merge has just read
@@ -1347,17 +1460,17 @@ extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool,
   TI_REQUIRE(n_splits >= 1 && n_splits <= 8 && (n_splits == 1 || (part_o && part_ml && n_rows > 0)),
              "attention_prefill_paired: 1 to 8 runs of keys, more than one with buffers for their results");
   if (n_tiles == 0) return 0;
-  constexpr int NG = 4, NW = 2, ST = 2;
+  constexpr int NG = 4, NW = 2, ST = 2, CB = 1;
   const int lds = NG * ST * 2 * PF_KEYS * hd * 2;
   static bool ready = false;          // allow more than 64 KiB of dynamic LDS, once
   if (!ready) {
-    if (hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<128, NG, NW, ST, true>,
+    if (hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<128, NG, NW, ST, true, CB>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, NG * ST * 2 * PF_KEYS * 128 * 2) != hipSuccess ||
-        hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<64, NG, NW, ST, true>,
+        hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<64, NG, NW, ST, true, CB>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, NG * ST * 2 * PF_KEYS * 64 * 2) != hipSuccess ||
-        hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<128, NG, NW, ST, false>,
+        hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<128, NG, NW, ST, false, CB>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, NG * ST * 2 * PF_KEYS * 128 * 2) != hipSuccess ||
-        hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<64, NG, NW, ST, false>,
+        hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<64, NG, NW, ST, false, CB>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, NG * ST * 2 * PF_KEYS * 64 * 2) != hipSuccess) {
       ti_set_error("attention_prefill_paired: cannot reserve the LDS");
       return 2;
@@ -1368,7 +1481,7 @@ extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool,
   // heaviest tile then, not as the heaviest and the lightest together)
   dim3 grid(paired ? (n_tiles + 1) / 2 : n_tiles, n_head, n_splits);
 #define TI_GO(H, PAIRED)                                                                                          \
-  attn_prefill_lds_kernel<H, NG, NW, ST, PAIRED><<<grid, 64 * NW * NG, lds, stream>>>(                            \
+  attn_prefill_lds_kernel<H, NG, NW, ST, PAIRED, CB><<<grid, 64 * NW * NG, lds, stream>>>(                            \
       (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, n_tiles, entries, (bf16_t*)out, n_head, \
       n_kv, page_size, scale, window, part_o, part_ml)
   if (hd == 128 && paired) TI_GO(128, true);
