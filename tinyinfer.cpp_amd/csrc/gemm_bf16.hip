@@ -915,6 +915,9 @@ __device__ __forceinline__ void qkv_rows_by_lanes(const QKVEpilogue& ep, float* 
     qkv_rows_by_lanes<HD, BM, NWV, FS, false, false>(ep, ft, s_pos, s_page, s_prow, s_live, hh, u, m0);
 }
 
+// k-steps whose fragments are on their way from LDS while one is multiplied (two: a prompt of 2,048 tokens at
+// Qwen3-0.6B's sizes 0.7 % faster, at Qwen3-8B's 3.7 % slower)
+#define FRAG_AHEAD 1
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_arg,
@@ -936,7 +939,8 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
   const int kt0 = (int)((long)(K / PBK) * blockIdx.z / gridDim.z);
   const int n_k = (int)((long)(K / PBK) * (blockIdx.z + 1) / gridDim.z) - kt0;
   void* __restrict__ out_ = (EPI == TI_EPI_STORE_F32) ? (void*)((float*)out_arg + (size_t)blockIdx.z * M * N) : out_arg;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  // the wavefront's number in a scalar register: where its loads go in LDS is scalar arithmetic then
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int m0 = blockIdx.y * BM;
   const int n0 = n_first + blockIdx.x * (SW ? BN / 2 : BN);
@@ -969,18 +973,20 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
     }
   }
 
-  auto issue = [&](int kt) {
+  // load i of this wavefront's LOADS loads of k-tile kt
+  auto issue_one = [&](int kt, int i) {
     unsigned char* stage = smem + (kt % PSTAGES) * STAGE_BYTES;
     const int k0 = (kt0 + kt) * PBK;
+    const int g = wave + NWV * i;
+    unsigned char* dst = stage + g * 1024;                   // the same in every lane
+    // K is a multiple of 64 here (the dispatcher sees to it): no piece lies past the end
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void*)(gsrc[i] + k0 + gpiece[i] * 8),
+        (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+  };
+  auto issue = [&](int kt) {
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-      const int g = wave + NWV * i;
-      unsigned char* dst = stage + g * 1024;                 // the same in every lane
-      // K is a multiple of 64 here (the dispatcher sees to it): no piece lies past the end
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(gsrc[i] + k0 + gpiece[i] * 8),
-          (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-    }
+    for (int i = 0; i < LOADS; ++i) issue_one(kt, i);
   };
 
   floatx16 acc[TM][TN];
@@ -1016,7 +1022,13 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
     // and every wavefront has finished with the stage that tile kt + 2 goes into
     if (kt + 1 < n_k) wait_vmcnt(LOADS); else wait_vmcnt(0);
     __builtin_amdgcn_s_barrier();
-    if (kt + 2 < n_k) issue(kt + 2);
+    // Tile kt + 2 goes into the stage that everyone has left.  Its loads go out between the k-steps
+    // below, each behind a k-step's matrix instructions: the unit that takes the addresses handles 64
+    // bytes a cycle for the whole compute unit, and eight wavefronts that ask for a whole tile at once
+    // queue there with nothing on the matrix cores meanwhile.
+    // (a prompt of 2,048 tokens 2.5 % faster at Qwen3-0.6B's sizes, 2.1 % at Qwen3-8B's; a k-tile of a 256 x 128
+    // tile from 2,480 to 2,200 cycles)
+    const bool more = kt + 2 < n_k;
     if constexpr (EPI == TI_EPI_ADD_F32) {
       if (kt == n_k - 1) {
 #pragma unroll
@@ -1032,7 +1044,9 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
       }
     }
     const unsigned st = (kt % PSTAGES) * STAGE_BYTES;
-    v4u fa[2][TM], fb[2][TN];
+    // the fragments of FRAG_AHEAD k-steps are on their way from LDS while one is multiplied
+    constexpr int SETS = FRAG_AHEAD + 1, KSTEPS = PBK / 16;
+    v4u fa[SETS][TM], fb[SETS][TN];
     auto read_step = [&](int ks, int set) {
       const unsigned pa = rowA + st + xo[ks], pb = rowB + st + xo[ks];
 #pragma unroll
@@ -1042,21 +1056,22 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
       for (int b = 0; b < TN; ++b)
         asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[set][b]) : "v"(pb), "n"(b * 32 * 128));
     };
-    read_step(0, 0);
 #pragma unroll
-    for (int ks = 0; ks < PBK / 16; ++ks) {
-      const int set = ks & 1;
-      if (ks + 1 < PBK / 16) {
-        read_step(ks + 1, set ^ 1);
-        // all but the TM + TN reads just issued are done: this k-step's fragments are there
-        if (TM + TN == 7) asm volatile("s_waitcnt lgkmcnt(7)" ::: "memory");
-        if (TM + TN == 6) asm volatile("s_waitcnt lgkmcnt(6)" ::: "memory");
-        if (TM + TN == 4) asm volatile("s_waitcnt lgkmcnt(4)" ::: "memory");
-        if (TM + TN == 3) asm volatile("s_waitcnt lgkmcnt(3)" ::: "memory");
-        if (TM + TN == 2) asm volatile("s_waitcnt lgkmcnt(2)" ::: "memory");
-        static_assert(TM + TN == 7 || TM + TN == 6 || TM + TN == 4 || TM + TN == 3 || TM + TN == 2, "a wait for every tile shape");
-      } else {
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    for (int ks = 0; ks < FRAG_AHEAD; ++ks) read_step(ks, ks);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const int set = ks % SETS;
+      if (ks + FRAG_AHEAD < KSTEPS) read_step(ks + FRAG_AHEAD, (ks + FRAG_AHEAD) % SETS);
+      // this k-step's fragments are there when only the reads issued after them are outstanding:
+      // those of the k-steps up to FRAG_AHEAD further on
+      constexpr int PER = TM + TN;
+      const int later = (KSTEPS - 1 - ks < FRAG_AHEAD ? KSTEPS - 1 - ks : FRAG_AHEAD) * PER;
+      static_assert(FRAG_AHEAD * PER <= 15, "lgkmcnt counts to 15");
+      switch (later) {
+#define TI_LGKM(N) case N: asm volatile("s_waitcnt lgkmcnt(" #N ")" ::: "memory"); break;
+        TI_LGKM(0) TI_LGKM(2) TI_LGKM(3) TI_LGKM(4) TI_LGKM(6) TI_LGKM(7) TI_LGKM(8) TI_LGKM(12) TI_LGKM(14)
+#undef TI_LGKM
+        default: asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); break;
       }
       // tie the fragments to the wait, so that no MFMA is moved above it
 #pragma unroll
@@ -1070,6 +1085,10 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
           acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[set][a]),
                                                               __builtin_bit_cast(bf16x8, fb[set][b]), acc[a][b],
                                                               0, 0, 0);
+      if (more) {
+#pragma unroll
+        for (int i = ks; i < LOADS; i += PBK / 16) issue_one(kt + 2, i);
+      }
     }
   }
 
