@@ -864,8 +864,9 @@ struct QKVEpilogue {
 
 // A q or k head (unit u of the fused projection, head hh of the tile) of all BM rows of a tile that
 // lies in LDS in 32-bit (row stride FS): eight lanes a row, 8 NWV rows a pass.  The angles of the
-// next pass are asked for before a pass is finished; a row's bfloat16 then leave LDS in pieces of
-// 16 bytes, the eight lanes writing 128 consecutive bytes.
+// next pass are asked for before a pass is finished; a lane reads its HD / 16 pairs from LDS as runs of
+// 16 bytes and writes its finished elements to memory as two runs of HD / 8 bytes, the eight lanes
+// together the row's 2 HD consecutive bytes.
 template <int HD, int BM, int NWV, int FS, bool NORMED, bool ROTATE>
 __device__ __forceinline__ void qkv_rows_by_lanes(const QKVEpilogue& ep, float* ft, const int* s_pos,
                                                   const int* s_page, const int* s_prow, const int* s_live, int hh,
@@ -882,18 +883,24 @@ __device__ __forceinline__ void qkv_rows_by_lanes(const QKVEpilogue& ep, float* 
       qk_lanes_angles<HD>(next, s_pos[(ps + 1) * NWV * 8 + tid / 8], ep.inv_freq, ep.rope_table, ep.table_len);
     if (ps >= 0) {
       const int r = ps * NWV * 8 + tid / 8;
-      float* row = ft + r * FS + hh * HD;
-      qk_head_lanes<HD, NORMED, ROTATE>(row, wlo, whi, ep.eps, cs);
+      unsigned lo[NP / 2], hi[NP / 2];
+      qk_head_lanes<HD, NORMED, ROTATE>(ft + r * FS + hh * HD, wlo, whi, ep.eps, cs, lo, hi);
       bf16_t* dst = nullptr;
       if (is_q) {
         if (s_live[r] >= 0) dst = ep.q_out + ((size_t)(m0 + r) * ep.n_head + u) * HD;
       } else if (s_page[r] >= 0) {
         dst = kv_page_slot<bf16_t>(ep.pool, s_page[r], 0, u - ep.n_head, s_prow[r], ep.n_kv, ep.P, HD);
       }
-      if (dst)
-#pragma unroll
-        for (int pc = tid & 7; pc < HD / 8; pc += 8)
-          reinterpret_cast<uint4*>(dst)[pc] = reinterpret_cast<const uint4*>(row)[pc];
+      if (dst) {
+        bf16_t* mine = dst + NP * (tid & 7);
+        if constexpr (NP == 8) {
+          *reinterpret_cast<uint4*>(mine) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+          *reinterpret_cast<uint4*>(mine + HD / 2) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        } else {
+          *reinterpret_cast<uint2*>(mine) = make_uint2(lo[0], lo[1]);
+          *reinterpret_cast<uint2*>(mine + HD / 2) = make_uint2(hi[0], hi[1]);
+        }
+      }
     }
 #pragma unroll
     for (int k = 0; k < NP; ++k) cs[k] = next[k];

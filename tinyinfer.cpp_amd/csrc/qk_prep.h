@@ -120,17 +120,19 @@ __device__ __forceinline__ void qk_head_thread(const float* src, bf16_t* dst, co
   }
 }
 
-// One head by eight adjacent lanes of a wavefront: lane j of the eight takes the pairs j, j + 8, ...
-// of the row.  The three functions below give such a lane its norm weights, its angles, and the
-// finished row.  The loads of the first two do not wait for one another, and a caller with several
-// rows asks for all their angles before it finishes the first.
+// One head by eight adjacent lanes of a wavefront: lane j of the eight takes HD / 16 consecutive pairs,
+// HD / 16 j .. HD / 16 (j + 1) - 1, of the row: what it reads (LDS, weights, angles) and what it writes
+// are runs of consecutive bytes.  The three functions below give such a lane its norm weights, its
+// angles, and the finished elements.  The loads of the first two do not wait for one another, and a
+// caller with several rows asks for all their angles before it finishes the first.
 template <int HD>
 __device__ __forceinline__ void qk_lanes_weights(float (&wlo)[HD / 16], float (&whi)[HD / 16], const float* w) {
+  constexpr int PPL = HD / 16;
   const int j = threadIdx.x & 7;
 #pragma unroll
-  for (int k = 0; k < HD / 16; ++k) {
-    wlo[k] = w ? w[j + 8 * k] : 1.f;
-    whi[k] = w ? w[HD / 2 + j + 8 * k] : 1.f;
+  for (int k = 0; k < PPL; ++k) {
+    wlo[k] = w ? w[PPL * j + k] : 1.f;
+    whi[k] = w ? w[HD / 2 + PPL * j + k] : 1.f;
   }
 }
 
@@ -138,67 +140,77 @@ __device__ __forceinline__ void qk_lanes_weights(float (&wlo)[HD / 16], float (&
 template <int HD>
 __device__ __forceinline__ void qk_lanes_angles(float2 (&cs)[HD / 16], int p, const float* inv_freq,
                                                 const float2* rope_table, int table_len) {
-  constexpr int HALF = HD / 2;
+  constexpr int HALF = HD / 2, PPL = HD / 16;
   const int j = threadIdx.x & 7;
   const bool held = rope_table && p < table_len;
   if (rope_table) {
     // every lane loads (a row beyond the table reads the last one and computes below)
-    const float2* tp = rope_table + (size_t)min(p, table_len - 1) * HALF;
+    const float4* tp = reinterpret_cast<const float4*>(rope_table + (size_t)min(p, table_len - 1) * HALF + PPL * j);
 #pragma unroll
-    for (int k = 0; k < HD / 16; ++k) cs[k] = tp[j + 8 * k];
+    for (int k = 0; k < PPL; k += 2) {
+      const float4 v = tp[k / 2];
+      cs[k] = make_float2(v.x, v.y);
+      cs[k + 1] = make_float2(v.z, v.w);
+    }
   }
   if (!held) {
 #pragma unroll
-    for (int k = 0; k < HD / 16; ++k) cs[k] = qk_cos_sin(j + 8 * k, HALF, p, inv_freq, nullptr, 0);
+    for (int k = 0; k < PPL; ++k) cs[k] = qk_cos_sin(PPL * j + k, HALF, p, inv_freq, nullptr, 0);
   }
 }
 
-// From HD floats at `row` (LDS, 16-byte aligned) to HD bfloat16 that overwrite the first half of the
-// same floats.  A lane's own pairs go up the tree of the sum of squares in the lane (partners at
-// distance 32, 16, 8), the rest across the eight lanes (4, 2, 1): the tree of qk_head_wave's
-// butterfly, so the bits are the same.  All lanes of the wavefront call it together; a row that
-// is not wanted is computed and left in LDS.  NORMED: with the norm (weights wlo, whi); ROTATE:
-// with the rotation by cs.
+// From HD floats at `row` (LDS, 16-byte aligned) to this lane's finished elements as bfloat16 pairs:
+// lo[k] holds elements HD / 16 j + 2 k, + 1, hi[k] the same of the second half (HD / 2 further on).  The
+// sum of squares goes up the tree of qk_head_wave's butterfly, so the bits are the same: partners at
+// pair distance HD / 4, HD / 8, HD / 16 sit in the lanes j ^ 4, j ^ 2, j ^ 1 with the same k (every
+// lane's HD / 16 partial sums cross the lanes), the closer ones in the lane itself.  All lanes of the
+// wavefront call it together.  NORMED: with the norm (weights wlo, whi); ROTATE: with the rotation by cs.
 template <int HD, bool NORMED, bool ROTATE>
-__device__ __forceinline__ void qk_head_lanes(float* row, const float (&wlo)[HD / 16], const float (&whi)[HD / 16],
-                                              float eps, const float2 (&cs)[HD / 16]) {
-  constexpr int HALF = HD / 2, NP = HALF / 8;
-  static_assert(NP == 4 || NP == 8, "the tree below is that of a 64-lane butterfly with one pair a lane");
+__device__ __forceinline__ void qk_head_lanes(const float* row, const float (&wlo)[HD / 16], const float (&whi)[HD / 16],
+                                              float eps, const float2 (&cs)[HD / 16], unsigned (&lo_out)[HD / 32],
+                                              unsigned (&hi_out)[HD / 32]) {
+  constexpr int HALF = HD / 2, PPL = HD / 16;
+  static_assert(PPL == 4 || PPL == 8, "the tree below is that of a 64-lane butterfly with one pair a lane");
   const int j = threadIdx.x & 7;
-  float lo[NP], hi[NP];
+  float lo[PPL], hi[PPL];
 #pragma unroll
-  for (int k = 0; k < NP; ++k) {
-    lo[k] = row[j + 8 * k];
-    hi[k] = row[HALF + j + 8 * k];
+  for (int k = 0; k < PPL; k += 4) {
+    const float4 a = *reinterpret_cast<const float4*>(row + PPL * j + k);
+    const float4 b = *reinterpret_cast<const float4*>(row + HALF + PPL * j + k);
+    lo[k] = a.x; lo[k + 1] = a.y; lo[k + 2] = a.z; lo[k + 3] = a.w;
+    hi[k] = b.x; hi[k + 1] = b.y; hi[k + 2] = b.z; hi[k + 3] = b.w;
   }
-  // the eight lanes read all of the row before any of them writes into it (a wavefront runs its
-  // LDS instructions in order; the compiler is told not to move them)
-  asm volatile("" ::: "memory");
   float scale = 1.f;
   if (NORMED) {
-    float t[NP];
+    float t[PPL];
 #pragma unroll
-    for (int k = 0; k < NP; ++k) t[k] = qk_pair_square(lo[k], hi[k]);
+    for (int k = 0; k < PPL; ++k) t[k] = qk_pair_square(lo[k], hi[k]);
 #pragma unroll
-    for (int o = NP / 2; o >= 1; o >>= 1)
+    for (int o = 4; o >= 1; o >>= 1)
+#pragma unroll
+      for (int k = 0; k < PPL; ++k) t[k] += __shfl_xor(t[k], o, TI_WAVE);
+#pragma unroll
+    for (int o = PPL / 2; o >= 1; o >>= 1)
 #pragma unroll
       for (int k = 0; k < o; ++k) t[k] += t[k + o];
-    scale = qk_norm_scale(group_sum<8>(t[0]), HD, eps);
+    scale = qk_norm_scale(t[0], HD, eps);
   }
-  bf16_t* rb = reinterpret_cast<bf16_t*>(row);
 #pragma unroll
-  for (int k = 0; k < NP; ++k) {
-    const int i = j + 8 * k;
-    float a = lo[k] * scale, b = hi[k] * scale;
-    if (NORMED) {
-      a *= wlo[k];
-      b *= whi[k];
+  for (int k = 0; k < PPL; k += 2) {
+    float a[2], b[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      a[e] = lo[k + e] * scale;
+      b[e] = hi[k + e] * scale;
+      if (NORMED) {
+        a[e] *= wlo[k + e];
+        b[e] *= whi[k + e];
+      }
+      if (ROTATE) qk_rotate(a[e], b[e], cs[k + e]);
     }
-    if (ROTATE) qk_rotate(a, b, cs[k]);
-    rb[i] = f2bf(a);
-    rb[i + HALF] = f2bf(b);
+    lo_out[k / 2] = pack_bf16x2(a[0], a[1]);
+    hi_out[k / 2] = pack_bf16x2(b[0], b[1]);
   }
-  asm volatile("" ::: "memory");
 }
 
 // A value head: copied (rounded to T), element d to dst[d * dst_stride]
