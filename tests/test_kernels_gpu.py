@@ -598,6 +598,47 @@ def test_linear_bf16_matrix_cores(ops, M, N, K):
         assert (f64(out) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol
 
 
+@pytest.mark.parametrize("seed", [1, 2])
+def test_linear_bf16_random_sizes(ops, seed):
+    """Sixty products drawn from a seed, whichever kernel the sizes lead to: token rows from 1 to 2,100
+    (around every border between kernels: 8, 12, 16, 64, 128, 256), weights from 2 to 12,288 rows, K from
+    8 to 9,728, every epilogue, and a row behind the output that must stay as it was."""
+    import random
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
+    rnd = random.Random(seed)
+    for case in range(60):
+        M = rnd.choice([1, 2, 3, 5, 8, 9, 12, 13, 16, 17, 31, 32, 33, 48, 63, 64, 65, 100, 127, 128, 129, 255, 256,
+                        257, 300, 511, 777, 1024, 2048, 2100])
+        N = rnd.choice([2, 6, 16, 34, 64, 130, 160, 256, 320, 522, 1000, 1024, 1280, 2048, 3072, 4096, 4100, 6144,
+                        8192, 9728, 12288])
+        K = 8 * rnd.choice([1, 2, 3, 4, 8, 9, 13, 16, 24, 32, 33, 64, 96, 128, 129, 256, 320, 384, 512, 640, 1024, 1216])
+        if M * N > 2100 * 4100 * 2 or N * K > 12288 * 5120:
+            continue
+        what = f"case {case}: {M} rows, weight {N} x {K}"
+        g = torch.Generator().manual_seed(seed * 1000 + case)
+        a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
+        w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+        ref = (a.double() @ w.double().T).cpu()
+        tol = 2e-5 * K
+        out = torch.full((M + 1, N), 7.0, device="cuda")
+        ops.linear(a, w, out[:M], "store")
+        assert (f64(out[:M]) - ref).abs().max() < tol, what
+        assert bool((out[M] == 7.0).all()), what
+        base = torch.randn(M, N, generator=g)
+        acc = dev(base.clone())
+        ops.linear(a, w, acc, "add")
+        assert (f64(acc) - (ref + f64(base))).abs().max() < tol, what
+        out = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+        ops.linear(a, w, out, "store_act")
+        assert (f64(out) - ref).abs().max() < 0.005 * ref.abs().max() + tol, what
+        F = N // 2
+        out = torch.empty(M, F, device="cuda", dtype=torch.bfloat16)
+        ops.linear(a, w, out, "swiglu")
+        gte, up = ref[:, :F], ref[:, F:]
+        want = gte / (1 + torch.exp(-gte)) * up
+        assert (f64(out) - want).abs().max() < 0.005 * want.abs().max() + 10 * tol, what
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 1, 8), (1, 1024, 2048), (8, 1024, 3072), (3, 7, 4096), (2, 4095, 520),
                                    (4, 33, 1032), (8, 5, 24), (5, 1000, 2056), (7, 130, 3080)])
 def test_linear_bf16_weight_row_per_wavefront(ops, M, N, K):
@@ -1379,6 +1420,40 @@ def test_attention_bf16_portions_and_mixed(ops, nh, nkv, hd, P, window, variant)
         ops.force_paired_tiles = None
     assert torch.isfinite(got).all()
     assert (got - want).abs().max() < 2e-2
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_attention_bf16_random_shapes_and_batches(ops, seed):
+    """Sixteen batches drawn from a seed: head size, heads and groups, page size, window, one to six entries
+    of portions and single tokens starting anywhere, and the launch forced or left to choose.  Finds what the
+    hand-picked cases leave out (an entry whose share of the keys is empty, a window that ends inside a
+    run, a tile of one row beside one of 700)."""
+    import random
+    assert ops.use_fast_attention, "the bfloat16 attention kernels are switched off or not built"
+    rnd = random.Random(seed)
+    lib = ops.lib("attention_bf16")
+    for case in range(16):
+        hd = rnd.choice([64, 128])
+        nkv = rnd.choice([1, 2, 4, 8])
+        nh = nkv * rnd.choice([1, 2, 4])
+        P = rnd.choice([16, 32, 48, 64])
+        window = rnd.choice([None, None, None, 40, 300, 1000])
+        entries = [(rnd.choice([1, 2, 3, 16, 17, 31, 32, 33, 63, 64, 65, 100, 128, 129, 200, 333, 700]),
+                    rnd.choice([0, 0, 1, 15, 16, 17, 31, 32, 63, 64, 100, 500, 1000, 1023, 1024, 1500, 3000]))
+                   for _ in range(rnd.randint(1, 6))]
+        variant = rnd.choice(["as the launch chooses", "paired", "a tile each", "one group", "two groups"])
+        lib.ti_tuning_set(b"prefill_groups", {"one group": 1, "two groups": 2}.get(variant, 0))
+        ops.use_paired_prefill = variant in ("as the launch chooses", "paired", "a tile each")
+        ops.force_paired_tiles = {"paired": True, "a tile each": False}.get(variant)
+        try:
+            got, want = fast_attention_case(ops, entries, nh, nkv, hd, P, window, seed=seed * 100 + case)
+        finally:
+            lib.ti_tuning_set(b"prefill_groups", 0)
+            ops.use_paired_prefill = True
+            ops.force_paired_tiles = None
+        what = f"case {case}: head size {hd}, heads {nh}/{nkv}, page {P}, window {window}, {variant}, entries {entries}"
+        assert torch.isfinite(got).all(), what
+        assert (got - want).abs().max() < 2e-2, what
 
 
 def test_attention_bf16_far_into_long_contexts(ops):
