@@ -1143,6 +1143,47 @@ def test_widths_that_160_divides_take_tiles_of_160_columns(ops, M, N, K):
     assert (f64(got[1][2]) - ref).abs().max() < 0.005 * ref.abs().max() + tol
 
 
+@pytest.mark.parametrize("tile,M,N,K", [(1, 700, 2048, 128), (1, 2300, 1024, 64), (3, 700, 1024, 192), (9, 1100, 1280, 64),
+                                        (0, 1500, 2048, 128)])
+@pytest.mark.parametrize("rows", [1, 3, 8])
+def test_tiles_taken_in_the_dies_order(ops, tile, M, N, K, rows):
+    """The order in which workgroups take a tiled product's tiles when the weight is larger than the cache
+    in front of the memory (each die an eighth of the column tiles, in blocks of `rows` row tiles), forced
+    here on small products: every tile is still computed once, with the bits of the grid's order; the last
+    block of row tiles is short where `rows` does not divide their number; tile 0 is a launch in two ranges."""
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
+    lib = ops.lib("gemm_bf16")
+    g = torch.Generator().manual_seed(M + N + rows)
+    a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    w = dev((torch.rand(N, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    base = torch.randn(M, N, generator=g)
+    ref = ref_linear(a.cpu(), w.cpu())
+    got = {}
+    try:
+        lib.ti_tuning_set(b"force_tile", tile)
+        for order in (rows, -1):
+            lib.ti_tuning_set(b"xcd_rows", order)
+            out = torch.full((M + 1, N), 7.0, device="cuda")
+            ops.linear(a, w, out[:M], "store")
+            added = dev(base.clone())
+            ops.linear(a, w, added, "add")
+            act = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+            ops.linear(a, w, act, "store_act")
+            res = [out, added, act]
+            if tile != 9:
+                glu = torch.empty(M, N // 2, device="cuda", dtype=torch.bfloat16)
+                ops.linear(a, w, glu, "swiglu")
+                res.append(glu)
+            got[order] = res
+    finally:
+        lib.ti_tuning_set(b"force_tile", 0)
+        lib.ti_tuning_set(b"xcd_rows", 0)
+    for x, y in zip(got[rows], got[-1]):
+        assert torch.equal(x, y)
+    assert (f64(got[rows][0][:M]) - ref).abs().max() < 2e-5 * K
+    assert bool((got[rows][0][M] == 7.0).all())
+
+
 @pytest.mark.parametrize("M", [17, 40, 64])
 def test_swiglu_of_up_to_64_rows_under_a_wide_weight(ops, M):
     """17 to 64 rows times a stacked [gate; up] weight of 32,768 rows take 64 x 128 tiles (twice the weight
@@ -1667,6 +1708,18 @@ def test_qkv_product_with_prepared_heads_in_two_ranges(ops, M, nh, nkv, hd):
     big = -(-M // 256) * ((nh + 2 * nkv) * hd // 128)
     assert big >= units and 0 < big % units < units * 3 // 4, "the shape does not take the rule"
     qkv_prepared_case(ops, 0, M, nh, nkv, hd, 64, 16, True, "table")
+
+
+@pytest.mark.parametrize("tile_rows,rows", [(128, 4), (256, 2)])
+def test_qkv_product_with_prepared_heads_in_the_dies_order(ops, tile_rows, rows):
+    """The same product with its tiles taken in the dies' order (eight column tiles of whole heads, six or
+    three row tiles in blocks of four or two): the same bits in q and in the cache."""
+    lib = ops.lib("gemm_bf16")
+    lib.ti_tuning_set(b"xcd_rows", rows)
+    try:
+        qkv_prepared_case(ops, tile_rows, 700, 6, 1, 128, 128, 16, True, "table")
+    finally:
+        lib.ti_tuning_set(b"xcd_rows", 0)
 
 
 def qkv_prepared_case(ops, tile_rows, M, nh, nkv, hd, K, P, norm, rope):

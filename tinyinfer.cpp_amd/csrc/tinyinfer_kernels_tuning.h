@@ -9,6 +9,8 @@
 //   normed_weight_below  weights of fewer elements keep the norm inside the product (0: the default)
 //   tiles_160            0: no tiles of 160 columns
 //   two_ranges           0: never split a product's columns between 256 x 128 and 128 x 64 tiles
+//   xcd_rows             row tiles per block of the order in which a die takes the tiles of a tiled product (-1: the grid's order,
+//                        0: by the weight's size)
 //   skinny_waves         4 or 8 wavefronts in the kernel for M <= 64 (0: by the shape)
 //   qkv_prep_min_rows    the fewest rows ti_gemm_bf16_qkv_prep serves (17)
 //   qkv_prep_rows        128 / 256: the rows of ti_gemm_bf16_qkv_prep's tile; 0: by the shape
