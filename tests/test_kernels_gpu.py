@@ -1030,12 +1030,13 @@ def test_rmsnorm_that_adds_partial_sums(ops, rows, H, KS):
         assert (f64(out) - ref_rmsnorm(want_x, w, 1e-6)).abs().max() < (1e-5 if dtype == torch.float32 else 0.03)
 
 
-@pytest.mark.parametrize("tile", [1, 3, 5, 6, 8, 9])
+@pytest.mark.parametrize("tile", [1, 3, 5, 6, 8, 9, 10])
 @pytest.mark.parametrize("M,N,K", [(300, 520, 128), (257, 384, 192), (130, 200, 64), (700, 96, 320)])
 def test_linear_bf16_every_tile(ops, tile, M, N, K):
     """Each tile of the pipelined kernel (256 x 128 with eight wavefronts, 128 x 64, 64 x 128 for the SwiGLU
-    epilogue, 64 x 64, and 128 x 160 and 256 x 160 with four wavefronts, which the SwiGLU epilogue does not
-    take), whatever the dispatch would have chosen for the shape, with every epilogue, against float64."""
+    epilogue, 64 x 64, 128 x 160 and 256 x 160 with four wavefronts, which the SwiGLU epilogue does not
+    take, and 256 x 256 with k-tiles of 32 in a ring of four stages), whatever the dispatch would have chosen
+    for the shape, with every epilogue, against float64."""
     assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
     lib = ops.lib("gemm_bf16")
     g = torch.Generator().manual_seed(M + N + tile)
@@ -1182,6 +1183,35 @@ def test_tiles_taken_in_the_dies_order(ops, tile, M, N, K, rows):
         assert torch.equal(x, y)
     assert (f64(got[rows][0][:M]) - ref).abs().max() < 2e-5 * K
     assert bool((got[rows][0][M] == 7.0).all())
+
+
+@pytest.mark.parametrize("M,F,K", [(2048, 4096, 4096), (2048, 9216, 4096), (1990, 4056, 4160)])
+def test_stacked_gate_up_over_many_rows_takes_tiles_of_256_x_256(ops, M, F, K):
+    """A [gate; up] weight over many rows with a long K: 256 x 256 tiles where they make whole rounds of the
+    compute units (8 x 32 tiles), and where rounds are left over (8 x 72 tiles: two rounds and a quarter) the
+    whole rounds' columns take them and the rest 256 x 128 tiles; rows and columns that fill no tile.
+    The bits of the product with the rule switched off, and the values of float64."""
+    assert ops.use_fast_gemm, "the bfloat16 MFMA kernels are switched off or not built"
+    lib = ops.lib("gemm_bf16")
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    assert -(-M // 256) * -(-2 * F // 256) >= units, "the shape does not take the rule"
+    g = torch.Generator().manual_seed(M + F)
+    a = dev((torch.rand(M, K, generator=g) * 2 - 1).to(torch.bfloat16))
+    w = dev((torch.rand(2 * F, K, generator=g) * 2 - 1).to(torch.bfloat16) * 0.05)
+    outs = []
+    try:
+        for on in (1, 0):
+            lib.ti_tuning_set(b"tiles_256", on)
+            out = torch.full((M + 1, F), 7.0, device="cuda", dtype=torch.bfloat16)
+            ops.linear(a, w, out[:M], "swiglu")
+            assert bool((out[M] == 7.0).all())
+            outs.append(out[:M])
+    finally:
+        lib.ti_tuning_set(b"tiles_256", 1)
+    assert torch.equal(outs[0], outs[1])
+    ref = (a.double() @ w.double().T).cpu()
+    want = ref[:, :F] / (1 + torch.exp(-ref[:, :F])) * ref[:, F:]
+    assert (f64(outs[0]) - want).abs().max() < 0.005 * want.abs().max() + 2e-4 * K
 
 
 @pytest.mark.parametrize("M", [17, 40, 64])

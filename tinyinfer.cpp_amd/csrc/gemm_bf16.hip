@@ -925,7 +925,7 @@ __device__ __forceinline__ void qkv_rows_by_lanes(const QKVEpilogue& ep, float* 
 // k-steps whose fragments are on their way from LDS while one is multiplied (two: a prompt of 2,048 tokens at
 // Qwen3-0.6B's sizes 0.7 % faster, at Qwen3-8B's 3.7 % slower)
 #define FRAG_AHEAD 1
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int STAGES = PSTAGES, int KT = PBK>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ out_arg,
                       int M, int N, int K, long lda, int n_first, int xcd_rows, QKVEpilogue ep = QKVEpilogue{}) {
@@ -953,24 +953,33 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
   constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
   constexpr int NWV = WAVES_M * WAVES_N;                     // wavefronts: 4 or 8
   static_assert(NWV == 4 || NWV == 8, "four or eight wavefronts");
-  static_assert(!SW || TN == 2, "SwiGLU pairs two column tiles per wavefront");
-  constexpr int STAGE_BYTES = (BM + BN) * PBK * 2;
-  constexpr int GROUPS_A = BM / 8, GROUPS_B = BN / 8;        // 8 rows = 1 KiB = one wavefront load
+  static_assert(!SW || TN % 2 == 0, "SwiGLU pairs the column tiles of a wavefront: the first half gate, the second half up");
+  static_assert(STAGES >= 2 && STAGES <= 4, "two to four stages");
+  // KT: the depth of a k-tile, 64 or 32.  A row of a stage is KT bfloat16 (CPR pieces of 16 bytes); a wavefront's
+  // load of 1 KiB covers RPL rows; piece c of row r lies in slot c ^ swz(r), so that the sixteen lanes of a
+  // fragment read (sixteen rows, one piece) touch sixteen different 16-byte columns of the banks
+  static_assert(KT == 64 || KT == 32, "k-tiles of 64 or 32");
+  constexpr int CPR = KT / 8, RPL = 64 / CPR, ROWB = KT * 2;
+  auto swz = [](int r) { return KT == 64 ? (r >> 1) & 7 : (r >> 2) & 3; };
+
+  constexpr int STAGE_BYTES = (BM + BN) * ROWB;
+  constexpr int GROUPS_A = BM / RPL, GROUPS_B = BN / RPL;    // RPL rows = 1 KiB = one wavefront load
   static_assert((GROUPS_A + GROUPS_B) % NWV == 0, "every wavefront issues the same number of loads");
   constexpr int LOADS = (GROUPS_A + GROUPS_B) / NWV;         // per wavefront and k-tile
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   // gridDim.z > 1 (storing epilogue only): K is split; workgroup z takes its share of the k-tiles and
   // stores its sums into the z-th [M, N] of out
-  const int kt0 = (int)((long)(K / PBK) * blockIdx.z / gridDim.z);
-  const int n_k = (int)((long)(K / PBK) * (blockIdx.z + 1) / gridDim.z) - kt0;
+  const int kt0 = (int)((long)(K / KT) * blockIdx.z / gridDim.z);
+  const int n_k = (int)((long)(K / KT) * (blockIdx.z + 1) / gridDim.z) - kt0;
   void* __restrict__ out_ = (EPI == TI_EPI_STORE_F32) ? (void*)((float*)out_arg + (size_t)blockIdx.z * M * N) : out_arg;
   // the wavefront's number in a scalar register: where its loads go in LDS is scalar arithmetic then
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int m0 = by * BM;
   const int n0 = n_first + bx * (SW ? BN / 2 : BN);
-  const int lr = lane >> 3, lc = lane & 7;                   // row within a group of 8, slot within the row
+  const int lr = lane / CPR, lc = lane % CPR;                // row within a load's group of rows, slot within the row
+  const bool spread = K >= 4096;
 
   // the global row each of this lane's loads reads (clamped into the matrix: rows
   // beyond it are computed and thrown away), as a pointer to its first element
@@ -980,29 +989,29 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
   for (int i = 0; i < LOADS; ++i) {
     const int g = wave + NWV * i;                            // groups 0..GROUPS_A-1: A, then B
     if (g < GROUPS_A) {
-      const int row = g * 8 + lr;
+      const int row = g * RPL + lr;
       const int gm = min(m0 + row, M - 1);
       gsrc[i] = A + (size_t)gm * lda;
-      gpiece[i] = lc ^ ((row >> 1) & 7);
+      gpiece[i] = lc ^ swz(row);
     } else {
-      const int row = (g - GROUPS_A) * 8 + lr;
+      const int row = (g - GROUPS_A) * RPL + lr;
       int wr;
       if (SW) {
-        const int span = BN / WAVES_N;                       // 64: LDS rows of one wavefront's columns
-        const int n = n0 + (row / span) * 32 + (row & 31);
-        wr = ((row & 32) ? N : 0) + min(n, N - 1);
+        constexpr int span = BN / WAVES_N, half = span / 2;  // LDS rows of one wavefront's columns: gate rows, then up rows
+        const int n = n0 + (row / span) * half + (row % half);
+        wr = ((row % span) >= half ? N : 0) + min(n, N - 1);
       } else {
         wr = min(n0 + row, N - 1);
       }
       gsrc[i] = W + (size_t)wr * K;
-      gpiece[i] = lc ^ ((row >> 1) & 7);
+      gpiece[i] = lc ^ swz(row);
     }
   }
 
   // load i of this wavefront's LOADS loads of k-tile kt
   auto issue_one = [&](int kt, int i) {
-    unsigned char* stage = smem + (kt % PSTAGES) * STAGE_BYTES;
-    const int k0 = (kt0 + kt) * PBK;
+    unsigned char* stage = smem + (kt % STAGES) * STAGE_BYTES;
+    const int k0 = (kt0 + kt) * KT;
     const int g = wave + NWV * i;
     unsigned char* dst = stage + g * 1024;                   // the same in every lane
     // K is a multiple of 64 here (the dispatcher sees to it): no piece lies past the end
@@ -1032,21 +1041,24 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
   // MFMAs (its fragments have arrived; those of the next k-step are still in flight).
   const int fr = lane & 31, fh = lane >> 5;                  // fragment row, and which half of a 16-wide k-step
   const unsigned lds0 = (unsigned)(size_t)smem;              // LDS byte address of the first stage
-  const unsigned rowA = lds0 + (wm * (BM / WAVES_M) + fr) * 128;
-  const unsigned rowB = lds0 + BM * PBK * 2 + (wn * (BN / WAVES_N) + fr) * 128;
-  unsigned xo[PBK / 16];                                     // swizzled byte offset of this lane's piece, per k-step
+  const unsigned rowA = lds0 + (wm * (BM / WAVES_M) + fr) * ROWB;
+  const unsigned rowB = lds0 + BM * ROWB + (wn * (BN / WAVES_N) + fr) * ROWB;
+  unsigned xo[KT / 16];                                      // swizzled byte offset of this lane's piece, per k-step
 #pragma unroll
-  for (int ks = 0; ks < PBK / 16; ++ks) xo[ks] = ((ks * 2 + fh) ^ ((fr >> 1) & 7)) << 4;
+  for (int ks = 0; ks < KT / 16; ++ks) xo[ks] = ((ks * 2 + fh) ^ swz(fr)) << 4;
 
   // the residual an adding epilogue adds to: asked for while the last k-tile is multiplied
   // (elements outside the matrix read a valid one and are not stored)
-  float prev[EPI == TI_EPI_ADD_F32 ? TM : 1][EPI == TI_EPI_ADD_F32 ? TN : 1][16];
-  issue(0);
-  if (n_k > 1) issue(1);
+  // (a tile of many accumulators has no registers for it and reads the residual in the epilogue)
+  constexpr bool PREV = EPI == TI_EPI_ADD_F32 && (NWV == 4 || TM * TN <= 4);
+  float prev[PREV ? TM : 1][PREV ? TN : 1][16];
+#pragma unroll
+  for (int st = 0; st < STAGES - 1; ++st)
+    if (st < n_k) issue(st);
   for (int kt = 0; kt < n_k; ++kt) {
-    // tile kt has landed (its loads are older than those of tile kt + 1), in every wavefront,
-    // and every wavefront has finished with the stage that tile kt + 2 goes into
-    if (kt + 1 < n_k) wait_vmcnt(LOADS); else wait_vmcnt(0);
+    // tile kt has landed (its loads are older than those of the tiles after it), in every wavefront,
+    // and every wavefront has finished with the stage that tile kt + STAGES - 1 goes into
+    wait_vmcnt(min(STAGES - 2, n_k - 1 - kt) * LOADS);
     __builtin_amdgcn_s_barrier();
     // Tile kt + 2 goes into the stage that everyone has left.  Its loads go out between the k-steps
     // below, each behind a k-step's matrix instructions: the unit that takes the addresses handles 64
@@ -1054,8 +1066,9 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
     // queue there with nothing on the matrix cores meanwhile.
     // (a prompt of 2,048 tokens 2.5 % faster at Qwen3-0.6B's sizes, 2.1 % at Qwen3-8B's; a k-tile of a 256 x 128
     // tile from 2,480 to 2,200 cycles)
-    const bool more = kt + 2 < n_k;
-    if constexpr (EPI == TI_EPI_ADD_F32) {
+    // (spread evenly between the matrix instructions where K is long, k-step by k-step where it is short: see below)
+    const bool more = kt + STAGES - 1 < n_k, more_spread = more && spread, more_steps = more && !spread;
+    if constexpr (PREV) {
       if (kt == n_k - 1) {
 #pragma unroll
         for (int a = 0; a < TM; ++a)
@@ -1069,18 +1082,18 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
             }
       }
     }
-    const unsigned st = (kt % PSTAGES) * STAGE_BYTES;
+    const unsigned st = (kt % STAGES) * STAGE_BYTES;
     // the fragments of FRAG_AHEAD k-steps are on their way from LDS while one is multiplied
-    constexpr int SETS = FRAG_AHEAD + 1, KSTEPS = PBK / 16;
+    constexpr int SETS = FRAG_AHEAD + 1, KSTEPS = KT / 16;
     v4u fa[SETS][TM], fb[SETS][TN];
     auto read_step = [&](int ks, int set) {
       const unsigned pa = rowA + st + xo[ks], pb = rowB + st + xo[ks];
 #pragma unroll
       for (int a = 0; a < TM; ++a)
-        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[set][a]) : "v"(pa), "n"(a * 32 * 128));
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[set][a]) : "v"(pa), "n"(a * 32 * ROWB));
 #pragma unroll
       for (int b = 0; b < TN; ++b)
-        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[set][b]) : "v"(pb), "n"(b * 32 * 128));
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[set][b]) : "v"(pb), "n"(b * 32 * ROWB));
     };
 #pragma unroll
     for (int ks = 0; ks < FRAG_AHEAD; ++ks) read_step(ks, ks);
@@ -1107,13 +1120,25 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
 #pragma unroll
       for (int a = 0; a < TM; ++a)
 #pragma unroll
-        for (int b = 0; b < TN; ++b)
+        for (int b = 0; b < TN; ++b) {
           acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[set][a]),
                                                               __builtin_bit_cast(bf16x8, fb[set][b]), acc[a][b],
                                                               0, 0, 0);
-      if (more) {
+          // load i goes out behind matrix instruction (2 i + 1) NM / (2 LOADS) of the k-tile's NM: spread evenly,
+          // no two wavefronts' loads queue at the unit that takes the addresses (a prompt of 2,048 tokens at
+          // Qwen3-8B's sizes 2.2 % faster, at Qwen3-32B's 3.1 %; at Qwen3-0.6B's, K = 1,024 to 3,072, 0.6 % slower
+          // than with the loads behind each k-step's matrix instructions, which stays for K below 4,096)
+          constexpr int NM = KSTEPS * TM * TN;
+          const int g = (ks * TM + a) * TN + b;
+          if (more_spread) {
 #pragma unroll
-        for (int i = ks; i < LOADS; i += PBK / 16) issue_one(kt + 2, i);
+            for (int i = 0; i < LOADS; ++i)
+              if ((2 * i + 1) * NM / (2 * LOADS) == g) issue_one(kt + STAGES - 1, i);
+          }
+        }
+      if (more_steps) {
+#pragma unroll
+        for (int i = ks; i < LOADS; i += KT / 16) issue_one(kt + STAGES - 1, i);
       }
     }
   }
@@ -1128,7 +1153,7 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
     static_assert((BM == 256 || BM == 128) && NWV == 8, "the first wavefronts look up a row each; 64 rows per pass of all eight");
     constexpr int FS = BN + 8;                              // row stride: the eight rows x eight lanes of a wavefront
                                                             // read 64 different banks
-    static_assert(BM * FS * 4 + 4 * BM * 4 <= PSTAGES * (BM + BN) * PBK * 2, "the 32-bit tile fits into the stages");
+    static_assert(BM * FS * 4 + 4 * BM * 4 <= STAGES * STAGE_BYTES, "the 32-bit tile fits into the stages");
     float* ft = reinterpret_cast<float*>(smem);
     __syncthreads();
 #pragma unroll
@@ -1205,8 +1230,11 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
       const int m = m0 + wm * (BM / WAVES_M) + a * 32 + (i >> 2) * 8 + crow + (i & 3);
       if (m >= M) continue;
       if (SW) {
-        const int n = n0 + wn * 32 + ccol;
-        if (n < N) ((bf16_t*)out_)[(size_t)m * N + n] = f2bf(silu_mul(acc[a][0][i], acc[a][TN - 1][i]));
+#pragma unroll
+        for (int b = 0; b < TN / 2; ++b) {
+          const int n = n0 + wn * (BN / WAVES_N / 2) + b * 32 + ccol;
+          if (n < N) ((bf16_t*)out_)[(size_t)m * N + n] = f2bf(silu_mul(acc[a][b][i], acc[a][b + TN / 2][i]));
+        }
       } else {
 #pragma unroll
         for (int b = 0; b < TN; ++b) {
@@ -1215,7 +1243,7 @@ gemm_pipelined_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W
           const size_t o = (size_t)m * N + n;
           const float v = acc[a][b][i];
           if (EPI == TI_EPI_STORE_F32) ((float*)out_)[o] = v;
-          if constexpr (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] = prev[a][b][i] + v;
+          if constexpr (EPI == TI_EPI_ADD_F32) ((float*)out_)[o] = (PREV ? prev[a][b][i] : ((const float*)out_)[o]) + v;
           if (EPI == TI_EPI_STORE_ACT) ((bf16_t*)out_)[o] = f2bf(v);
         }
       }
@@ -1235,11 +1263,11 @@ static int xcd_rows_for(const dim3& grid, int N, int K) {
   return (long)N * K * 2 >= (192L << 20) ? 8 : 0;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int STAGES = PSTAGES, int KT = PBK>
 static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, int N, int K, long lda,
                             hipStream_t s, int ksplit = 1, int n_first = 0, int n_end = -1) {
-  constexpr int bytes = PSTAGES * (BM + BN) * PBK * 2;
-  auto kernel = gemm_pipelined_kernel<BM, BN, WAVES_M, WAVES_N, EPI>;
+  constexpr int bytes = STAGES * (BM + BN) * KT * 2;
+  auto kernel = gemm_pipelined_kernel<BM, BN, WAVES_M, WAVES_N, EPI, STAGES, KT>;
   static bool ready = false;          // per instantiation: allow more than 64 KiB of dynamic LDS
   if (!ready) {
     if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
@@ -1258,6 +1286,7 @@ static int launch_pipelined(const bf16_t* A, const bf16_t* W, void* out, int M, 
 }
 
 static int g_tiles_160 = 1;      // a hook for measurements: 0 = no tiles of 160 columns
+static int g_tiles_256 = 1;      // a hook for measurements: 0 = no tiles of 256 x 256
 static int g_two_ranges = 1;     // a hook for measurements: 0 = never split the columns between two tile shapes
 static int g_qkv_rows = 0;       // hooks for measurements: 128 or 256 forces the tile's rows;
 static int g_qkv_min_rows = 17;  // the fewest rows served (fewer take the kernels with the norm in front)
@@ -1350,7 +1379,7 @@ extern "C" int ti_gemm_bf16_qkv_prep(const void* A, const void* W, int M, int K,
 }
 
 // for measurements: 0 = choose the tile by the shape, 1 = 256 x 128, 3 = 128 x 64, 5 = 64 x 128 (SwiGLU only), 6 = 64 x 64,
-// 8 = 128 x 160, 9 = 256 x 160 (neither for SwiGLU)
+// 8 = 128 x 160, 9 = 256 x 160 (neither for SwiGLU), 10 = 256 x 256
 static int g_force_tile = 0;
 
 // Three tiles.  256 x 128 with eight wavefronts does the most per byte it loads, one workgroup
@@ -1396,6 +1425,25 @@ static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M,
       else if (whole(wg128) && wg128 <= 2L * units) tile = 8;
     }
   }
+  // A stacked [gate; up] weight over many rows, K long: 256 x 256 tiles (eight wavefronts of 64 x 128, two
+  // stages of 64 KB) load two thirds of what 256 x 128 tiles load per flop.  Taken where they come in whole
+  // rounds of the units (Qwen3-8B's gate/up over 2,048 rows, 8 x 96 tiles: 382 -> 343 us); where rounds are
+  // left over, the columns of the whole rounds take them and the rest 256 x 128 tiles in a launch of its own
+  // (Qwen3-32B's, 8 x 200 tiles).  With the other epilogues they gain nothing or lose (o over 8,192 rows: 285 ->
+  // 314 us).
+  if constexpr (SW) {
+    const long huge = (long)((M + 255) / 256) * ((N * cols + 255) / 256);
+    if (!g_force_tile && g_tiles_256 && M > 256 && K >= 4096 && huge >= units) {
+      const int row_tiles = (M + 255) / 256;
+      if (huge % units == 0 || huge % units >= units * 7 / 8) return launch_pipelined<256, 256, 4, 2, EPI, 4, 32>(A, W, out, M, N, K, lda, s);
+      const int col_tiles = (int)(huge / units * units / row_tiles);
+      const int n_big = col_tiles * 128;                // output columns of the first range
+      if (huge >= 2L * units && col_tiles >= 1 && n_big < N) {
+        if (int rc = launch_pipelined<256, 256, 4, 2, EPI, 4, 32>(A, W, out, M, N, K, lda, s, 1, 0, n_big)) return rc;
+        return launch_pipelined<256, 128, 4, 2, EPI>(A, W, out, M, N, K, lda, s, 1, n_big, N);
+      }
+    }
+  }
   // 256 x 128 tiles that fill the units once or more and leave a round short of three quarters (Qwen3-32B's
   // o and down projections over 2,048 rows: 8 x 40 tiles on 256 units): the columns that make whole rounds
   // take those tiles, the rest 128 x 64 tiles in a launch of their own behind them, rather than everything
@@ -1416,6 +1464,7 @@ static int launch_tiled_best(const bf16_t* A, const bf16_t* W, void* out, int M,
     if (tile == 9) return launch_pipelined<256, 160, 4, 1, EPI>(A, W, out, M, N, K, lda, s);
   }
   if (tile == 1) return launch_pipelined<256, 128, 4, 2, EPI>(A, W, out, M, N, K, lda, s);
+  if (tile == 10) return launch_pipelined<256, 256, 4, 2, EPI, 4, 32>(A, W, out, M, N, K, lda, s);
   if constexpr (EPI == TI_EPI_SWIGLU)
     if (tile == 5) return launch_pipelined<64, 128, 2, 2, EPI>(A, W, out, M, N, K, lda, s);
   if constexpr (EPI != TI_EPI_SWIGLU)                // a SwiGLU wavefront needs two column tiles
@@ -2250,7 +2299,7 @@ extern "C" int ti_gemm_bf16(const void* A, const void* W, void* out, int M, int 
 // The rules are the library's, process-wide; the host library's Ops applies an object's own
 // overrides around its calls and resets them afterwards.  Returns 0, or 1 for an unknown name.
 extern "C" void ti_tuning_reset() {
-  g_xcd_rows = 0; g_tiles_160 = 1; g_two_ranges = 1; g_qkv_rows = 0; g_qkv_min_rows = 17; g_force_tile = 0; g_skinny_waves = 0;
+  g_xcd_rows = 0; g_tiles_160 = 1; g_tiles_256 = 1; g_two_ranges = 1; g_qkv_rows = 0; g_qkv_min_rows = 17; g_force_tile = 0; g_skinny_waves = 0;
   g_skinny_deep = 1; g_use_pipelined = 1; set_tiled_from(280L << 20); g_row_per_wave = 1;
   g_normed_weight_below = NORMED_WEIGHT_BELOW; g_skinny_copy = 1; g_wide_rows = 1; g_pieces = 1; g_add_split = 1;
   g_rows_direct = 1;
@@ -2262,6 +2311,7 @@ extern "C" int ti_tuning_set(const char* name, long value) {
   if (n == "force_tile") g_force_tile = (int)value;
   else if (n == "normed_weight_below") g_normed_weight_below = value > 0 ? value : NORMED_WEIGHT_BELOW;
   else if (n == "tiles_160") g_tiles_160 = (int)value;
+  else if (n == "tiles_256") g_tiles_256 = (int)value;
   else if (n == "two_ranges") g_two_ranges = (int)value;
   else if (n == "xcd_rows") g_xcd_rows = (int)value;
   else if (n == "skinny_waves") g_skinny_waves = (int)value;

@@ -5,9 +5,10 @@
 // (Ops::tune) and resets them afterwards.
 //
 // libti_gemm_bf16:
-//   force_tile           1: 256 x 128, 3: 128 x 64, 5: 64 x 128 (SwiGLU only), 6: 64 x 64, 8: 128 x 160, 9: 256 x 160; 0: by the shape
+//   force_tile           1: 256 x 128, 3: 128 x 64, 5: 64 x 128 (SwiGLU only), 6: 64 x 64, 8: 128 x 160, 9: 256 x 160, 10: 256 x 256; 0: by the shape
 //   normed_weight_below  weights of fewer elements keep the norm inside the product (0: the default)
 //   tiles_160            0: no tiles of 160 columns
+//   tiles_256            0: no tiles of 256 x 256
 //   two_ranges           0: never split a product's columns between 256 x 128 and 128 x 64 tiles
 //   xcd_rows             row tiles per block of the order in which a die takes the tiles of a tiled product (-1: the grid's order,
 //                        0: by the weight's size)
